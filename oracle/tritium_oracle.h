@@ -1,0 +1,155 @@
+/*
+ * tritium_oracle.h — CPU restatement of the reference's packed-ternary linear path.
+ *
+ * TEST INFRASTRUCTURE ONLY. This library is the parity checker and the timed CPU
+ * baseline. The product (the HIP kernel library and its host adapter) never links,
+ * loads or calls it; only the test-suite, the smoke check and the benchmark's
+ * cpu_baseline leg do.
+ *
+ * Every function restates, in plain C, one function of the reference (Rust); the
+ * citation beside each declaration is `path:line` under the reference checkout.
+ * All floating-point code here must be compiled with -ffp-contract=off and without
+ * -ffast-math: the reference's arithmetic is single IEEE-754 binary32 operations in
+ * a fixed order and nothing may be fused or re-associated.
+ *
+ * Parity status: every function below is pinned by a known-answer test, golden bytes
+ * or a mathematical invariant in tests/test_oracle_*.py; none is "parity unpinned".
+ * What cannot be confirmed without the reference's toolchain is only that the
+ * regenerated conformance set is byte-identical to the reference's absent frozen file.
+ */
+#ifndef TRITIUM_ORACLE_H
+#define TRITIUM_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* crates/tritium-format/src/lib.rs:144-150 */
+#define TO_QK_K 256
+#define TO_TQ2_0_BLOCK_BYTES 66
+#define TO_TQ1_0_BLOCK_BYTES 54
+/* IEEE binary16 1.0: the block scale every host packer on this path writes
+ * (crates/tritium-nn/src/layers/linear.rs:166-184, crates/tritium-testkit/src/runner.rs:135-158). */
+#define TO_F16_ONE 0x3C00u
+
+/* crates/tritium-core/src/dtype.rs:89-107 — tags used across this build. */
+enum { TO_FMT_TQ1_0 = 1, TO_FMT_TQ2_0 = 2 };
+
+/* Return codes. 0 = ok. */
+enum {
+  TO_OK = 0,
+  TO_ERR_SHAPE = 1,       /* a length disagrees with the shape */
+  TO_ERR_FORMAT = 2,      /* unsupported format tag */
+  TO_ERR_INVALID = 4,     /* input failed validation */
+  TO_ERR_BACKEND = 5      /* a packed row decodes outside {-1,0,+1} */
+};
+
+/* ---- crates/tritium-format/src/tq2.rs:21-81 ---- */
+int to_pack_tq2_0_block(const int8_t *trits256, uint16_t scale_f16, uint8_t *out66);
+/* returns TO_ERR_BACKEND when a 2-bit slot holds the reserved code 3 (trit 2). */
+int to_unpack_tq2_0_block(const uint8_t *block66, int8_t *trits256, uint16_t *scale_f16);
+
+/* ---- crates/tritium-format/src/tq1.rs:18-30,36-121 ---- */
+int to_pack_tq1_0_block(const int8_t *trits256, uint16_t scale_f16, uint8_t *out54);
+int to_unpack_tq1_0_block(const uint8_t *block54, int8_t *trits256, uint16_t *scale_f16);
+
+/* ---- crates/tritium-format/src/rows.rs:25-151 ---- */
+size_t to_num_blocks(size_t k);
+size_t to_row_bytes(size_t k, int format); /* 0 for an unknown format */
+int to_pack_row(const int8_t *trits, size_t k, const uint16_t *scales_f16, size_t n_scales,
+                int format, uint8_t *out, size_t out_len);
+int to_unpack_row(const uint8_t *packed, size_t packed_len, int format, int8_t *trits, size_t k,
+                  uint16_t *scales_f16, size_t n_scales);
+/* Pack an [n,k] trit matrix row by row with block scale 1.0, as the reference's callers do
+ * (crates/tritium-testkit/src/runner.rs:135-158; crates/tritium-nn/src/layers/linear.rs:143-185). */
+int to_pack_matrix(const int8_t *trits, size_t n, size_t k, int format, uint8_t *out, size_t out_len);
+
+/* ---- crates/tritium-core/src/reference.rs:25-64 ---- */
+int to_reference_mpgemm(const float *act, size_t act_len, const int8_t *trits, size_t w_len,
+                        const float *scale_n, size_t scale_len, size_t m, size_t n, size_t k,
+                        float *out, size_t out_len);
+
+/* ---- crates/tritium-spec/src/lib.rs:338-378 (== crates/tritium-nn/src/ops/act_quant.rs:94-157) ---- */
+void to_quantize_act_int8(const float *act, size_t m, size_t k, float *q_out, float *scale_out);
+
+/* ---- crates/tritium-cpu/src/lib.rs:262-300 : upload_weights ----
+ * Validates the packed length; for TQ2_0 reports the first row holding a reserved code in
+ * *tq2_invalid_row (or -1). The bytes themselves are kept verbatim by the caller. */
+int to_cpu_upload_check(const uint8_t *packed, size_t len, size_t n, size_t k, int format,
+                        long *tq2_invalid_row);
+
+/* ---- crates/tritium-cpu/src/lib.rs:302-345,181-217 + kernel.rs:49-78,670-678 : mpgemm ----
+ * unpack all N*K trits, then the scalar kernel (== reference_mpgemm). The SIMD kernels of the
+ * reference are bit-identical to it by the reference's own tests
+ * (crates/tritium-cpu/src/kernel.rs:1069-1173), so this is the value oracle for every path. */
+int to_cpu_mpgemm(const uint8_t *packed, size_t packed_len, int format, const float *act,
+                  size_t act_len, const float *scales, size_t scales_len, size_t m, size_t n,
+                  size_t k, float *out, size_t out_len);
+
+/* ---- crates/tritium-spec/src/lib.rs:266-318 : default mpgemm_with_act_quant ----
+ * quantize -> mpgemm on int8-valued f32 -> out[m,:] *= act_scale[m]. */
+int to_cpu_mpgemm_with_act_quant(const uint8_t *packed, size_t packed_len, int format,
+                                 const float *act, size_t act_len, const float *scales,
+                                 size_t scales_len, size_t m, size_t n, size_t k, float *out,
+                                 size_t out_len);
+
+/* Exact int32 accumulators Σ_k q[m,k]·trit[n,k] for int8 activations (the value the reference's
+ * f32 fold holds before its two multiplies: crates/tritium-cpu/src/kernel.rs:588-599,824-828). */
+int to_int8_accumulators(const uint8_t *packed, size_t packed_len, int format, const int8_t *q,
+                         size_t m, size_t n, size_t k, int32_t *acc);
+
+/* Additive planes: out = Σ_p mpgemm(plane_p, scales_p) in plane order, f32 adds. The reference has
+ * no single function for this at per-channel-scale granularity; it is the composition through
+ * TernaryBackend::mpgemm (crates/tritium-spec/src/lib.rs:166-215), one call per plane. */
+int to_cpu_mpgemm_planes(const uint8_t *const *packed, const size_t *packed_len, int format,
+                         const float *const *scales, size_t planes, const float *act, size_t m,
+                         size_t n, size_t k, float *out);
+/* int8-activation planes: out[m,n] = (Σ_p ((float)acc_p · s_p[n])) · act_scale[m]; with one plane
+ * this is exactly crates/tritium-cpu/src/kernel.rs:921-922 followed by
+ * crates/tritium-nn/src/layers/linear.rs:272-277. */
+int to_cpu_linear_a8_planes(const uint8_t *const *packed, const size_t *packed_len, int format,
+                            const float *const *scales, size_t planes, const float *act, size_t m,
+                            size_t n, size_t k, float *out);
+
+/* ---- crates/tritium-testkit/src/vector.rs:113-125 ---- */
+int to_accepts_with_floor(float got, float want, float relative, int bit_exact, float floor_);
+
+/* ---- crates/tritium-testkit/src/generate.rs:18-57,65-233 : conformance vectors ---- */
+typedef struct to_vector {
+  char id[40];
+  size_t m, n, k;
+  int format;
+  float *activation; /* [m*k] */
+  int8_t *weights;   /* [n*k] */
+  float *scales;     /* [n]   */
+  float *expected;   /* [m*n] */
+} to_vector;
+typedef struct to_vector_set {
+  size_t count;
+  to_vector *v;
+} to_vector_set;
+to_vector_set *to_generate_vectors(uint64_t seed, size_t count);
+void to_free_vectors(to_vector_set *s);
+/* raw generator access for the known-answer tests */
+uint64_t to_xorshift64_next(uint64_t *state);
+
+/* bf16 helpers (round-to-nearest-even), used to state bf16-in / bf16-out expectations. */
+uint16_t to_f32_to_bf16(float x);
+float to_bf16_to_f32(uint16_t h);
+
+/* ---- timed CPU baseline: crates/tritium-cpu/src/kernel.rs:49-78,568-573,577-664,824-1003 ----
+ * Same dispatch as the reference: unpack every call; rows chunked at clamp(65536/(n*k),1,m)
+ * across `threads` workers; AVX-VNNI/AVX2 int8 kernel when every activation is an integer in
+ * [-128,127] and k <= 65536, else the k-order f32 fold. Values equal to_cpu_mpgemm bit for bit.
+ * Returns the worker count actually used in *threads_used. */
+int to_cpu_mpgemm_fast(const uint8_t *packed, size_t packed_len, int format, const float *act,
+                       const float *scales, size_t m, size_t n, size_t k, float *out, int threads,
+                       int *threads_used, int *kernel_used);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
