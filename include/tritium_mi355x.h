@@ -1,0 +1,205 @@
+/*
+ * tritium_mi355x.h — C ABI of the MI355X (gfx950) packed-ternary linear-layer kernel library.
+ *
+ * This is the boundary a Tritium backend crate binds over FFI: plain pointers and sizes, integer
+ * status codes, no C++ or framework types. Each entry point names the reference interface it
+ * stands behind (paths are relative to the reference checkout).
+ *
+ * Conventions (borrowed from the reference's own C ABI, crates/tritium-ffi/src/lib.rs:9-28,
+ * crates/tritium-ffi/include/tritium.h:19-43):
+ *   - every call returns a tk_status; 0 is success;
+ *   - the message for the last failure on the calling thread is tk_last_error();
+ *   - null pointers are checked and reported as TK_ERR_INVALID_INPUT, never dereferenced;
+ *   - nothing here panics or aborts on bad input (crates/tritium-spec/src/lib.rs:380-381).
+ *
+ * Shapes follow GemmShape (crates/tritium-core/src/shape.rs:10-38): C[M,N] = A[M,K] · Wᵀ with W
+ * the [N,K] ternary weight, row-major, output-major. All matrices are row-major.
+ */
+#ifndef TRITIUM_MI355X_H
+#define TRITIUM_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* One code per BackendError variant (crates/tritium-spec/src/lib.rs:382-405). */
+typedef enum tk_status {
+  TK_OK = 0,
+  TK_ERR_SHAPE_MISMATCH = 1,     /* BackendError::ShapeMismatch{expected,got}: see tk_last_mismatch */
+  TK_ERR_UNSUPPORTED_FORMAT = 2, /* BackendError::UnsupportedFormat */
+  TK_ERR_OUT_OF_MEMORY = 3,      /* BackendError::OutOfMemory{requested}: see tk_last_mismatch */
+  TK_ERR_INVALID_INPUT = 4,      /* BackendError::InvalidInput */
+  TK_ERR_BACKEND = 5             /* BackendError::Backend (any device error, stringified) */
+} tk_status;
+
+/* TernaryFormat (crates/tritium-core/src/dtype.rs:89-107). I2sInt8 is answered with
+ * TK_ERR_UNSUPPORTED_FORMAT, as the CPU backend does (crates/tritium-cpu/src/lib.rs:153-159). */
+typedef enum tk_format { TK_FORMAT_TQ1_0 = 1, TK_FORMAT_TQ2_0 = 2, TK_FORMAT_I2S_INT8 = 3 } tk_format;
+
+/* Element types of device-resident activations and outputs. */
+typedef enum tk_dtype { TK_F32 = 0, TK_BF16 = 1, TK_I8 = 2, TK_I32 = 3 } tk_dtype;
+
+#define TK_MAX_PLANES 4
+
+typedef struct tk_ctx tk_ctx;         /* one device + one stream; Send + Sync, calls serialised inside */
+typedef struct tk_weights tk_weights; /* a DeviceBuffer (crates/tritium-spec/src/lib.rs:147-158) */
+
+/* DeviceCaps (crates/tritium-spec/src/caps.rs:7-20) plus what the roofline report needs. */
+typedef struct tk_device_info {
+  char name[128];
+  char arch[32];
+  uint64_t total_memory_bytes;
+  int compute_units;
+  int clock_khz;
+  int memory_clock_khz;
+  int memory_bus_bits;
+  int wavefront_size;
+  int lds_bytes_per_cu;
+} tk_device_info;
+
+/* ---- lifetime: BackendEntry::init (crates/tritium-runtime/src/lib.rs:73-110) and
+ *      RocmBackend::new(ordinal) (crates/tritium-rocm/src/rocm.rs:234-300) ---- */
+int tk_init(int device, tk_ctx **out);
+void tk_destroy(tk_ctx *ctx);
+const char *tk_last_error(void);
+/* expected/got of the last ShapeMismatch, or requested/0 of the last OutOfMemory, on this thread */
+void tk_last_mismatch(size_t *expected, size_t *got);
+/* TernaryBackend::device_id / capabilities (crates/tritium-spec/src/lib.rs:166-186) */
+const char *tk_device_id(const tk_ctx *ctx); /* "mi355x:<ordinal>" */
+int tk_device_info_get(const tk_ctx *ctx, tk_device_info *out);
+int tk_device_count(int *count);
+
+/* ---- host-side packing: tritium-format row packers as TernaryLinear::pack_rows uses them
+ *      (crates/tritium-format/src/rows.rs:61-151, tq2.rs:21-81, tq1.rs:36-121,
+ *       crates/tritium-nn/src/layers/linear.rs:143-185). Block scale is f16 1.0. ---- */
+size_t tk_packed_len(size_t n, size_t k, int format); /* 0 for an unsupported format */
+int tk_pack_rows(const int8_t *trits, size_t trits_len, size_t n, size_t k, int format,
+                 uint8_t *out, size_t out_len);
+int tk_unpack_rows(const uint8_t *packed, size_t packed_len, size_t n, size_t k, int format,
+                   int8_t *trits, size_t trits_len);
+
+/* ---- TernaryBackend::upload_weights (crates/tritium-spec/src/lib.rs:188-200;
+ *      crates/tritium-cpu/src/lib.rs:262-300; crates/tritium-rocm/src/rocm.rs:446-475).
+ * Copies; the returned handle owns device memory until tk_free_weights. `packed` is the byte
+ * stream tritium-format writes: n rows of ceil(k/256) blocks of 66 (TQ2_0) or 54 (TQ1_0) bytes.
+ * Wrong length -> TK_ERR_INVALID_INPUT. The bytes are re-laid out once into a device-private
+ * 16-row tile order; block scales are not kept (the path ignores them,
+ * crates/tritium-cpu/src/lib.rs:19-21,202-205). ---- */
+int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k,
+                      int format, tk_weights **out);
+void tk_free_weights(tk_weights *w);
+size_t tk_weights_len_bytes(const tk_weights *w); /* DeviceBuffer::len_bytes: the uploaded length */
+size_t tk_weights_n(const tk_weights *w);
+size_t tk_weights_k(const tk_weights *w);
+int tk_weights_format(const tk_weights *w);
+/* Debug/parity aid: decode the device-resident planes back to [n,k] trits. */
+int tk_weights_download_trits(tk_ctx *ctx, const tk_weights *w, int8_t *trits, size_t trits_len);
+
+/* ---- TernaryBackend::mpgemm (crates/tritium-spec/src/lib.rs:202-215; oracle:
+ *      crates/tritium-cpu/src/lib.rs:302-345). Host slices in, host slice out, synchronous.
+ *      out[m,n] = scales[n] · Σ_k act[m,k] · trit[n,k]; `out` fully overwritten.
+ * Errors: act/scales/out length -> TK_ERR_SHAPE_MISMATCH; weights n/k/format differ from the
+ * call's -> TK_ERR_INVALID_INPUT (the CPU backend's choice, crates/tritium-cpu/src/lib.rs:123-135);
+ * a TQ2_0 plane holding the reserved code -> TK_ERR_BACKEND. m == 0 or n == 0 -> TK_OK, no launch. */
+int tk_mpgemm(tk_ctx *ctx, const float *act, size_t act_len, const tk_weights *weights,
+              const float *scales, size_t scales_len, size_t m, size_t n, size_t k, int format,
+              float *out, size_t out_len);
+
+/* ---- TernaryBackend::mpgemm_with_act_quant (crates/tritium-spec/src/lib.rs:228-318) and the
+ *      whole of TernaryLinear::forward (crates/tritium-nn/src/layers/linear.rs:229-280):
+ *      per-token int8 absmax quant on the device, exact int32 contraction, then
+ *      out[m,n] = ((float)acc · scales[n]) · act_scale[m]. Never refuses. ---- */
+int tk_mpgemm_with_act_quant(tk_ctx *ctx, const float *act, size_t act_len,
+                             const tk_weights *weights, const float *scales, size_t scales_len,
+                             size_t m, size_t n, size_t k, int format, float *out, size_t out_len);
+
+/* ---- device-resident extension, reached through TernaryBackend::as_concrete
+ *      (crates/tritium-spec/src/lib.rs:320-332); precedent: the CUDA backend's device-resident
+ *      decode (crates/tritium-cuda/src/cuda/mod.rs:1029-1064,2998-3041). All pointers below are
+ *      device pointers on ctx's device; calls enqueue on ctx's stream and do not synchronise. ---- */
+
+/* One additive-plane linear layer: `planes` weight handles with identical n,k and one per-channel
+ * scale vector (device, [n] f32) per plane. */
+typedef struct tk_linear_desc {
+  const tk_weights *planes[TK_MAX_PLANES];
+  const float *scales[TK_MAX_PLANES];
+  int n_planes;
+} tk_linear_desc;
+
+/* quantize_act_int8 on the device (crates/tritium-spec/src/lib.rs:351-378;
+ * precedent crates/tritium-cuda/kernels/tq2_0_imma.cu:84-141): act [m,k] f32 or bf16 ->
+ * q [m,k] int8 row-major and act_scale [m] f32. Rows holding NaN or Inf cannot be represented in
+ * int8; *their* q is zero and the row is reported in nonfinite_rows (may be null). */
+int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size_t m, size_t k, int8_t *q,
+                    float *act_scale, uint32_t *nonfinite_rows);
+
+/* Float-activation linear (BASELINE configs 1 and 2): act [m,k] f32 or bf16,
+ * out[m,n] = Σ_p scales_p[n] · Σ_k act[m,k]·trit_p[n,k], f32 accumulate, out f32 or bf16. */
+int tk_linear_float(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
+                    size_t m, void *out, int out_dtype);
+
+/* W1.58A8 linear on float activations: quantize per token, contract in int32, fold
+ * out[m,n] = (Σ_p (float)acc_p · scales_p[n]) · act_scale[m]. Chooses the decode GEMV or the
+ * prefill MFMA GEMM by m (crossover: tk_set_gemm_min_m). */
+int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
+                 size_t m, void *out, int out_dtype);
+
+/* Same contraction on activations that are already int8 (q [m,k]) with their per-token scales
+ * (act_scale [m], may be null for 1.0): what the CUDA decode calls gemm_prequantized
+ * (crates/tritium-cuda/src/cuda/mod.rs:1029-1064). out_dtype TK_I32 (one plane only) stores the
+ * raw int32 accumulators Σ_k q·trit instead of the scaled output. */
+int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
+                 size_t m, void *out, int out_dtype);
+
+/* Reference-order float contraction: one thread per output, a single f32 accumulator walked in k
+ * order (crates/tritium-core/src/reference.rs:25-54) — bit-identical to the CPU backend for any
+ * float input, NaN/Inf included. Slow; kept as the exact fallback and as a cross-check. */
+int tk_linear_float_seq(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
+                        size_t m, void *out, int out_dtype);
+
+/* Several independent linears in ONE launch (q/k/v or gate/up sharing a step; or a whole stack of
+ * projections whose inputs are already known). All members must share act_dtype, out_dtype, the
+ * mode and the plane count. Build once, launch many times. */
+typedef struct tk_group tk_group;
+typedef struct tk_group_member {
+  tk_linear_desc layer;
+  const void *act;  /* [m,k] */
+  size_t m;
+  void *out;        /* [m,n] */
+} tk_group_member;
+typedef enum tk_group_mode { TK_GROUP_FLOAT = 0, TK_GROUP_A8 = 1 } tk_group_mode;
+int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size_t count, int mode,
+                    int act_dtype, int out_dtype, tk_group **out);
+int tk_group_launch(tk_ctx *ctx, tk_group *group);
+void tk_group_destroy(tk_group *group);
+
+/* GEMV -> GEMM crossover in activation rows; the reference's knob is TRITIUM_IMMA_MIN_M, default
+ * 32, integer >= 2 (crates/tritium-cuda/src/cuda/backend.rs:6861-6876). The environment variable
+ * TRITIUM_MI355X_GEMM_MIN_M is read at tk_init with the same loud-reject rule. */
+int tk_set_gemm_min_m(tk_ctx *ctx, int min_m);
+int tk_get_gemm_min_m(const tk_ctx *ctx);
+
+/* ---- plumbing: device memory, stream, events (what the harness and a backend crate need) ---- */
+int tk_malloc(tk_ctx *ctx, size_t bytes, void **dptr);
+int tk_free(tk_ctx *ctx, void *dptr);
+int tk_memcpy_h2d(tk_ctx *ctx, void *dst, const void *src, size_t bytes);
+int tk_memcpy_d2h(tk_ctx *ctx, void *dst, const void *src, size_t bytes);
+int tk_memset(tk_ctx *ctx, void *dst, int value, size_t bytes);
+int tk_sync(tk_ctx *ctx);
+void *tk_stream(tk_ctx *ctx); /* the hipStream_t the context launches on */
+typedef struct tk_event tk_event;
+int tk_event_create(tk_ctx *ctx, tk_event **out);
+int tk_event_record(tk_ctx *ctx, tk_event *ev);
+int tk_event_elapsed_ms(tk_event *start, tk_event *stop, float *ms); /* waits for `stop` */
+void tk_event_destroy(tk_event *ev);
+/* A plain device-to-device copy kernel of `bytes` bytes (multiple of 16), used to calibrate
+ * hardware traffic counters against a known size. */
+int tk_copy_kernel(tk_ctx *ctx, void *dst, const void *src, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

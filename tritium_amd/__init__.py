@@ -1,0 +1,13 @@
+"""tritium_amd — MI355X (gfx950) backend for Tritium's packed ternary linear layer.
+
+The HIP kernel library (libtritium_mi355x.so, C ABI in include/tritium_mi355x.h) is the product;
+this package is the thin host mirror of the reference's adapter interface over it.
+"""
+from . import _lib
+from .backend import (BACKENDS, Backend, BackendEntry, BackendError, DeviceArray, DeviceBuffer, DeviceCaps,
+                      GemmShape, InvalidInput, Linear, Mi355xBackend, Mi355xBuffer, MpGemm, OutOfMemory,
+                      Registry, ShapeMismatch, TernaryFormat, UnsupportedFormat, pack_rows, packed_len,
+                      unpack_rows)
+from .linear import TernaryLinear
+
+__all__ = [n for n in dir() if not n.startswith("_")]

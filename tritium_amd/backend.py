@@ -1,0 +1,447 @@
+"""Host-side mirror of the reference's backend adapter for this path.
+
+Names, argument meaning and error behaviour follow `TernaryBackend`, `MpGemm`, `DeviceBuffer`,
+`DeviceCaps`, `BackendError` (crates/tritium-spec/src/lib.rs:64-78,147-158,166-333,382-405;
+caps.rs:7-67) and the registration record (crates/tritium-runtime/src/lib.rs:73-217). Everything
+computes in the HIP library behind the C ABI; nothing here has a CPU path.
+"""
+import ctypes as C
+import enum
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+
+from . import _lib as L
+
+
+# ---- BackendError (crates/tritium-spec/src/lib.rs:382-405) -----------------------------------
+
+class BackendError(Exception):
+    """Base of every error a backend returns; backends never panic on bad input."""
+
+
+class ShapeMismatch(BackendError):
+    def __init__(self, expected, got, msg=None):
+        super().__init__(msg or f"shape mismatch: expected {expected}, got {got}")
+        self.expected, self.got = expected, got
+
+
+class UnsupportedFormat(BackendError):
+    pass
+
+
+class OutOfMemory(BackendError):
+    def __init__(self, requested, msg=None):
+        super().__init__(msg or f"out of device memory: requested {requested} bytes")
+        self.requested = requested
+
+
+class InvalidInput(BackendError):
+    pass
+
+
+class Backend(BackendError):
+    """Device-specific failure, stringified (BackendError::Backend)."""
+
+
+def _raise(code):
+    lib = L.load()
+    msg = (lib.tk_last_error() or b"").decode()
+    if code == L.TK_ERR_SHAPE_MISMATCH:
+        e, g = C.c_size_t(0), C.c_size_t(0)
+        lib.tk_last_mismatch(C.byref(e), C.byref(g))
+        raise ShapeMismatch(e.value, g.value, msg)
+    if code == L.TK_ERR_UNSUPPORTED_FORMAT:
+        raise UnsupportedFormat(msg)
+    if code == L.TK_ERR_OUT_OF_MEMORY:
+        e, g = C.c_size_t(0), C.c_size_t(0)
+        lib.tk_last_mismatch(C.byref(e), C.byref(g))
+        raise OutOfMemory(e.value, msg)
+    if code == L.TK_ERR_INVALID_INPUT:
+        raise InvalidInput(msg)
+    raise Backend(msg)
+
+
+def _check(code):
+    if code != L.TK_OK:
+        _raise(code)
+
+
+# ---- vocabulary (crates/tritium-core/src/{shape.rs:10-38,dtype.rs:89-107}) --------------------
+
+class TernaryFormat(enum.IntEnum):
+    Tq1_0 = 1
+    Tq2_0 = 2
+    I2sInt8 = 3
+
+
+@dataclass(frozen=True)
+class GemmShape:
+    m: int
+    n: int
+    k: int
+
+    def macs(self):
+        return self.m * self.n * self.k
+
+    def buffers_fit(self, act_len, weight_len, out_len):
+        return act_len == self.m * self.k and weight_len == self.n * self.k and out_len == self.m * self.n
+
+
+@dataclass
+class DeviceCaps:
+    backend: str
+    device_name: str
+    features: List[str] = field(default_factory=list)
+    total_memory_bytes: int = 0
+    supports_imma: bool = False
+    supports_fp8: bool = False
+
+    def has_feature(self, name):
+        return name in self.features
+
+
+class DeviceBuffer:
+    """Opaque handle to device-resident memory owned by a backend."""
+
+    def len_bytes(self):
+        raise NotImplementedError
+
+    def is_empty(self):
+        return self.len_bytes() == 0
+
+
+@dataclass
+class MpGemm:
+    """Operands of one ternary mixed-precision GEMM call (crates/tritium-spec/src/lib.rs:64-78)."""
+    act: np.ndarray          # [M,K] f32, row-major (flat or 2-D)
+    weights: DeviceBuffer
+    scales: np.ndarray       # [N] f32
+    shape: GemmShape
+    format: TernaryFormat
+    out: np.ndarray          # [M,N] f32, overwritten
+
+
+DTYPES = {"f32": L.TK_F32, "bf16": L.TK_BF16, "i8": L.TK_I8, "i32": L.TK_I32}
+_NP = {L.TK_F32: np.float32, L.TK_BF16: np.uint16, L.TK_I8: np.int8, L.TK_I32: np.int32}
+
+
+class DeviceArray:
+    """A device allocation with a dtype tag; bf16 travels as uint16 bit patterns on the host."""
+
+    def __init__(self, backend, ptr, count, dtype):
+        self.backend, self.ptr, self.count, self.dtype = backend, ptr, count, dtype
+
+    @property
+    def nbytes(self):
+        return self.count * np.dtype(_NP[self.dtype]).itemsize
+
+    def to_host(self):
+        out = np.empty(self.count, _NP[self.dtype])
+        _check(L.load().tk_memcpy_d2h(self.backend._ctx, out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    def copy_from(self, host):
+        h = np.ascontiguousarray(host, _NP[self.dtype]).reshape(-1)
+        assert h.size == self.count, (h.size, self.count)
+        _check(L.load().tk_memcpy_h2d(self.backend._ctx, self.ptr, h.ctypes.data, h.nbytes))
+        return self
+
+    def free(self):
+        if self.ptr:
+            _check(L.load().tk_free(self.backend._ctx, self.ptr))
+            self.ptr = None
+
+
+class Mi355xBuffer(DeviceBuffer):
+    """Packed ternary weights resident on the device; frees its memory when dropped."""
+
+    def __init__(self, backend, handle):
+        self._backend, self._h = backend, handle
+
+    def len_bytes(self):
+        return L.load().tk_weights_len_bytes(self._h)
+
+    @property
+    def n(self):
+        return L.load().tk_weights_n(self._h)
+
+    @property
+    def k(self):
+        return L.load().tk_weights_k(self._h)
+
+    @property
+    def format(self):
+        return TernaryFormat(L.load().tk_weights_format(self._h))
+
+    def download_trits(self):
+        out = np.empty(self.n * self.k, np.int8)
+        _check(L.load().tk_weights_download_trits(self._backend._ctx, self._h, out.ctypes.data, out.size))
+        return out.reshape(self.n, self.k)
+
+    def free(self):
+        if self._h and self._backend._ctx:
+            L.load().tk_free_weights(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Linear:
+    """Device-resident additive-plane linear layer: plane handles + per-plane scale vectors."""
+
+    def __init__(self, backend, planes, scales):
+        self.backend, self.planes, self.scales = backend, list(planes), list(scales)
+        assert 1 <= len(self.planes) <= L.TK_MAX_PLANES and len(self.planes) == len(self.scales)
+        self.n, self.k = self.planes[0].n, self.planes[0].k
+        d = L.LinearDesc()
+        for i, (p, s) in enumerate(zip(self.planes, self.scales)):
+            d.planes[i] = p._h
+            d.scales[i] = s.ptr
+        d.n_planes = len(self.planes)
+        self.desc = d
+
+    def free(self):
+        for p in self.planes:
+            p.free()
+        for s in self.scales:
+            s.free()
+
+
+class Group:
+    def __init__(self, backend, handle, keep):
+        self.backend, self._h, self._keep = backend, handle, keep
+
+    def launch(self):
+        _check(L.load().tk_group_launch(self.backend._ctx, self._h))
+
+    def destroy(self):
+        if self._h:
+            L.load().tk_group_destroy(self._h)
+            self._h = None
+
+
+class Event:
+    def __init__(self, backend):
+        self.backend = backend
+        h = C.c_void_p()
+        _check(L.load().tk_event_create(backend._ctx, C.byref(h)))
+        self._h = h
+
+    def record(self):
+        _check(L.load().tk_event_record(self.backend._ctx, self._h))
+        return self
+
+    def elapsed_ms(self, stop):
+        ms = C.c_float(0)
+        _check(L.load().tk_event_elapsed_ms(self._h, stop._h, C.byref(ms)))
+        return ms.value
+
+    def destroy(self):
+        if self._h:
+            L.load().tk_event_destroy(self._h)
+            self._h = None
+
+
+def _flat(a, dtype, name):
+    arr = np.ascontiguousarray(a, dtype=dtype).reshape(-1)
+    return arr
+
+
+class Mi355xBackend:
+    """`impl TernaryBackend` for one MI355X (gfx950). Thread-safe; calls are synchronous."""
+
+    NAME = "mi355x"
+
+    def __init__(self, ordinal=0):
+        self._lib = L.load()
+        ctx = C.c_void_p()
+        _check(self._lib.tk_init(ordinal, C.byref(ctx)))
+        self._ctx = ctx
+        info = L.DeviceInfo()
+        _check(self._lib.tk_device_info_get(ctx, C.byref(info)))
+        self.info = info
+
+    def close(self):
+        if self._ctx:
+            self._lib.tk_destroy(self._ctx)
+            self._ctx = None
+
+    # ---- TernaryBackend ----
+    def device_id(self):
+        return self._lib.tk_device_id(self._ctx).decode()
+
+    def physical_device_id(self):
+        return self.device_id()
+
+    def capabilities(self):
+        return DeviceCaps(backend="mi355x", device_name=self.info.name.decode(),
+                          features=["hip", self.info.arch.decode().split(":")[0], "tq2_0", "tq1_0", "mfma_i8",
+                                    "act_quant_i8", "additive_planes"],
+                          total_memory_bytes=int(self.info.total_memory_bytes), supports_imma=True,
+                          supports_fp8=False)
+
+    def upload_weights(self, packed, shape, format):
+        b = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+        h = C.c_void_p()
+        _check(self._lib.tk_upload_weights(self._ctx, b.ctypes.data, b.size, shape.n, shape.k, int(format),
+                                           C.byref(h)))
+        return Mi355xBuffer(self, h)
+
+    def _host_call(self, fn, p):
+        if not isinstance(p.weights, Mi355xBuffer) or p.weights._backend is not self or not p.weights._h:
+            raise InvalidInput("buffer is not a Mi355xBuffer of this backend")
+        if not (isinstance(p.out, np.ndarray) and p.out.dtype == np.float32 and p.out.flags.c_contiguous):
+            raise InvalidInput("out must be a C-contiguous float32 numpy array")
+        act = _flat(p.act, np.float32, "act")
+        scales = _flat(p.scales, np.float32, "scales")
+        s = p.shape
+        _check(fn(self._ctx, act.ctypes.data, act.size, p.weights._h, scales.ctypes.data, scales.size,
+                  s.m, s.n, s.k, int(p.format), p.out.ctypes.data, p.out.size))
+
+    def mpgemm(self, p):
+        self._host_call(self._lib.tk_mpgemm, p)
+
+    def mpgemm_with_act_quant(self, p):
+        self._host_call(self._lib.tk_mpgemm_with_act_quant, p)
+
+    def mpgemm_projected_vjp(self, p=None):
+        # the inference-only default (crates/tritium-spec/src/lib.rs:221-226)
+        raise Backend(f"backend `{self.device_id()}` does not implement packed mpGEMM VJP")
+
+    def as_concrete(self):
+        return self
+
+    # ---- device-resident extension ----
+    def empty(self, count, dtype="f32"):
+        dt = DTYPES[dtype] if isinstance(dtype, str) else dtype
+        ptr = C.c_void_p()
+        _check(self._lib.tk_malloc(self._ctx, count * np.dtype(_NP[dt]).itemsize, C.byref(ptr)))
+        return DeviceArray(self, ptr, count, dt)
+
+    def to_device(self, host, dtype):
+        dt = DTYPES[dtype] if isinstance(dtype, str) else dtype
+        h = np.ascontiguousarray(host, _NP[dt]).reshape(-1)
+        return self.empty(h.size, dt).copy_from(h)
+
+    def sync(self):
+        _check(self._lib.tk_sync(self._ctx))
+
+    def linear(self, packed_planes, scales_planes, n, k, format=TernaryFormat.Tq2_0):
+        shape = GemmShape(0, n, k)  # upload is called with m = 0 (crates/tritium-nn/src/layers/linear.rs:97)
+        planes = [self.upload_weights(p, shape, format) for p in packed_planes]
+        scales = [self.to_device(s, "f32") for s in scales_planes]
+        for s in scales:
+            if s.count != n:
+                raise ShapeMismatch(n, s.count)
+        return Linear(self, planes, scales)
+
+    def _lin(self, fn, layer, act, m, out):
+        _check(fn(self._ctx, C.byref(layer.desc), act.ptr, act.dtype, m, out.ptr, out.dtype))
+
+    def linear_float(self, layer, act, m, out):
+        self._lin(self._lib.tk_linear_float, layer, act, m, out)
+
+    def linear_a8(self, layer, act, m, out):
+        self._lin(self._lib.tk_linear_a8, layer, act, m, out)
+
+    def linear_float_seq(self, layer, act, m, out):
+        self._lin(self._lib.tk_linear_float_seq, layer, act, m, out)
+
+    def linear_i8(self, layer, q, act_scale, m, out):
+        _check(self._lib.tk_linear_i8(self._ctx, C.byref(layer.desc), q.ptr,
+                                      act_scale.ptr if act_scale is not None else None, m, out.ptr, out.dtype))
+
+    def act_quant_i8(self, act, m, k, q, act_scale, nonfinite=None):
+        _check(self._lib.tk_act_quant_i8(self._ctx, act.ptr, act.dtype, m, k, q.ptr, act_scale.ptr,
+                                         nonfinite.ptr if nonfinite is not None else None))
+
+    def group(self, members, mode, act_dtype, out_dtype):
+        """members: list of (Linear, act DeviceArray, m, out DeviceArray)."""
+        arr = (L.GroupMember * len(members))()
+        for i, (layer, act, m, out) in enumerate(members):
+            arr[i].layer = layer.desc
+            arr[i].act = act.ptr
+            arr[i].m = m
+            arr[i].out = out.ptr
+        h = C.c_void_p()
+        _check(self._lib.tk_group_create(self._ctx, arr, len(members), mode, DTYPES[act_dtype], DTYPES[out_dtype],
+                                         C.byref(h)))
+        return Group(self, h, members)
+
+    def set_gemm_min_m(self, v):
+        _check(self._lib.tk_set_gemm_min_m(self._ctx, v))
+
+    def gemm_min_m(self):
+        return self._lib.tk_get_gemm_min_m(self._ctx)
+
+    def event(self):
+        return Event(self)
+
+    def copy_kernel(self, dst, src, nbytes):
+        _check(self._lib.tk_copy_kernel(self._ctx, dst.ptr, src.ptr, nbytes))
+
+
+# ---- host-side packing (tritium-format rows, as TernaryLinear::pack_rows uses them) -----------
+
+def packed_len(n, k, format):
+    return L.load().tk_packed_len(n, k, int(format))
+
+
+def pack_rows(trits, n, k, format=TernaryFormat.Tq2_0):
+    t = np.ascontiguousarray(trits, dtype=np.int8).reshape(-1)
+    out = np.empty(packed_len(n, k, format), np.uint8)
+    _check(L.load().tk_pack_rows(t.ctypes.data, t.size, n, k, int(format), out.ctypes.data, out.size))
+    return out
+
+
+def unpack_rows(packed, n, k, format=TernaryFormat.Tq2_0):
+    b = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+    out = np.empty(n * k, np.int8)
+    _check(L.load().tk_unpack_rows(b.ctypes.data, b.size, n, k, int(format), out.ctypes.data, out.size))
+    return out.reshape(n, k)
+
+
+# ---- registration (crates/tritium-runtime/src/lib.rs:73-217) -----------------------------------
+
+@dataclass
+class BackendEntry:
+    name: str
+    init: object  # () -> backend, raises BackendError when the device is unavailable
+
+
+BACKENDS: List[BackendEntry] = [BackendEntry(Mi355xBackend.NAME, lambda: Mi355xBackend(0))]
+
+
+class Registry:
+    """Initialises every registered backend; a failing init is logged to stderr and skipped."""
+
+    def __init__(self, entries=None):
+        import sys
+        self.backends = []
+        for entry in (BACKENDS if entries is None else entries):
+            try:
+                self.backends.append((entry.name, entry.init()))
+            except BackendError as err:
+                print(f"tritium-runtime: backend `{entry.name}` failed to initialise, skipping: {err}",
+                      file=sys.stderr)
+
+    def get(self, name) -> Optional[Mi355xBackend]:
+        for n, b in self.backends:
+            if n == name:
+                return b
+        return None
+
+    def enumerate(self):
+        return [b.capabilities() for _, b in self.backends]
+
+    def __len__(self):
+        return len(self.backends)
+
+    def is_empty(self):
+        return not self.backends

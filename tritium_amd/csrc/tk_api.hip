@@ -1,0 +1,848 @@
+// Host side of the C ABI: validation in the reference's order, device buffers, dispatch between the
+// decode GEMV and the prefill GEMM, and the trait-shaped host-slice entry points.
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "tk_host.h"
+#include "tk_internal.h"
+
+// ------------------------------------------------------------------------------------------
+// errors: thread-local last message (crates/tritium-ffi/src/lib.rs:9-28)
+// ------------------------------------------------------------------------------------------
+
+static thread_local char g_err[512];
+static thread_local size_t g_expected, g_got;
+
+int tk_fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+int tk_fail_mismatch(size_t expected, size_t got) {
+  g_expected = expected;
+  g_got = got;
+  return tk_fail(TK_ERR_SHAPE_MISMATCH, "shape mismatch: expected %zu, got %zu", expected, got);
+}
+int tk_fail_oom(size_t requested) {
+  g_expected = requested;
+  g_got = 0;
+  return tk_fail(TK_ERR_OUT_OF_MEMORY, "out of device memory: requested %zu bytes", requested);
+}
+extern "C" const char *tk_last_error(void) { return g_err; }
+extern "C" void tk_last_mismatch(size_t *expected, size_t *got) {
+  if (expected) *expected = g_expected;
+  if (got) *got = g_got;
+}
+
+#define HIPCHK(call)                                                                      \
+  do {                                                                                    \
+    hipError_t e_ = (call);                                                               \
+    if (e_ != hipSuccess) return tk_fail(TK_ERR_BACKEND, "%s: %s", #call, hipGetErrorString(e_)); \
+  } while (0)
+#define TKCHK(call)            \
+  do {                         \
+    int rc_ = (call);          \
+    if (rc_ != TK_OK) return rc_; \
+  } while (0)
+
+// ------------------------------------------------------------------------------------------
+// objects
+// ------------------------------------------------------------------------------------------
+
+struct DevBuf {
+  void *p = nullptr;
+  size_t cap = 0;
+};
+
+struct tk_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  std::mutex mu;
+  tk_device_info info{};
+  std::string device_id;
+  int gemm_min_m = 65;
+  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
+  int *d_invalid = nullptr;
+};
+
+struct tk_weights {
+  tk_ctx *ctx;
+  uint8_t *codes;
+  size_t n, k, nb, n_tiles, len_bytes;
+  int format;
+  long invalid_row;
+};
+
+struct tk_event {
+  hipEvent_t ev;
+};
+
+static int dev_malloc(size_t bytes, void **out) {
+  *out = nullptr;
+  if (!bytes) bytes = 16;
+  hipError_t e = hipMalloc(out, bytes);
+  if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) {
+    (void)hipGetLastError();
+    return tk_fail_oom(bytes);
+  }
+  if (e != hipSuccess) return tk_fail(TK_ERR_BACKEND, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  return TK_OK;
+}
+
+// Grow-only workspace. Growth waits for the stream first: an earlier launch may still read it.
+static int ensure(tk_ctx *ctx, DevBuf &b, size_t bytes) {
+  if (bytes <= b.cap) return TK_OK;
+  if (b.p) {
+    HIPCHK(hipStreamSynchronize(ctx->stream));
+    HIPCHK(hipFree(b.p));
+    b.p = nullptr;
+    b.cap = 0;
+  }
+  size_t want = bytes + bytes / 4 + 256;
+  TKCHK(dev_malloc(want, &b.p));
+  b.cap = want;
+  return TK_OK;
+}
+
+static inline size_t num_blocks(size_t k) { return (k + 255) / 256; }
+static inline size_t fmt_block_bytes(int format) {
+  return format == TK_FORMAT_TQ2_0 ? 66 : (format == TK_FORMAT_TQ1_0 ? 54 : 0);
+}
+static inline size_t dtype_size(int dt) { return dt == TK_BF16 ? 2 : (dt == TK_I8 ? 1 : 4); }
+
+// ------------------------------------------------------------------------------------------
+// lifetime
+// ------------------------------------------------------------------------------------------
+
+extern "C" int tk_device_count(int *count) {
+  if (!count) return tk_fail(TK_ERR_INVALID_INPUT, "tk_device_count: null pointer");
+  int c = 0;
+  hipError_t e = hipGetDeviceCount(&c);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *count = 0;
+    return tk_fail(TK_ERR_BACKEND, "hipGetDeviceCount: %s", hipGetErrorString(e));
+  }
+  *count = c;
+  return TK_OK;
+}
+
+extern "C" int tk_init(int device, tk_ctx **out) {
+  if (!out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_init: null out pointer");
+  *out = nullptr;
+  int count = 0;
+  TKCHK(tk_device_count(&count));
+  if (device < 0 || device >= count)
+    return tk_fail(TK_ERR_BACKEND, "tk_init: no HIP device %d (%d visible)", device, count);
+  int min_m = 65;
+  if (const char *env = getenv("TRITIUM_MI355X_GEMM_MIN_M")) {
+    char *end = nullptr;
+    long v = strtol(env, &end, 10);
+    if (!*env || *end || v < 2 || v > 65)
+      return tk_fail(TK_ERR_INVALID_INPUT, "TRITIUM_MI355X_GEMM_MIN_M=\"%s\" - use an integer in 2..65", env);
+    min_m = (int)v;
+  }
+  HIPCHK(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  HIPCHK(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return tk_fail(TK_ERR_BACKEND, "tk_init: device %d is %s; this library holds gfx950 code only", device,
+                   prop.gcnArchName);
+  tk_ctx *ctx = new (std::nothrow) tk_ctx();
+  if (!ctx) return tk_fail(TK_ERR_BACKEND, "tk_init: host allocation failed");
+  ctx->device = device;
+  ctx->gemm_min_m = min_m;
+  ctx->device_id = "mi355x:" + std::to_string(device);
+  snprintf(ctx->info.name, sizeof ctx->info.name, "%s", prop.name);
+  snprintf(ctx->info.arch, sizeof ctx->info.arch, "%s", prop.gcnArchName);
+  ctx->info.total_memory_bytes = prop.totalGlobalMem;
+  ctx->info.compute_units = prop.multiProcessorCount;
+  ctx->info.clock_khz = prop.clockRate;
+  ctx->info.memory_clock_khz = prop.memoryClockRate;
+  ctx->info.memory_bus_bits = prop.memoryBusWidth;
+  ctx->info.wavefront_size = prop.warpSize;
+  ctx->info.lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+  hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete ctx;
+    return tk_fail(TK_ERR_BACKEND, "hipStreamCreate: %s", hipGetErrorString(e));
+  }
+  void *p = nullptr;
+  int rc = dev_malloc(sizeof(int), &p);
+  if (rc) {
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return rc;
+  }
+  ctx->d_invalid = (int *)p;
+  *out = ctx;
+  return TK_OK;
+}
+
+extern "C" void tk_destroy(tk_ctx *ctx) {
+  if (!ctx) return;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  DevBuf *bufs[] = {&ctx->ap, &ctx->rowsum, &ctx->fscale, &ctx->aux, &ctx->exps,
+                    &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp};
+  for (DevBuf *b : bufs)
+    if (b->p) (void)hipFree(b->p);
+  if (ctx->d_invalid) (void)hipFree(ctx->d_invalid);
+  (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+}
+
+extern "C" const char *tk_device_id(const tk_ctx *ctx) { return ctx ? ctx->device_id.c_str() : ""; }
+
+extern "C" int tk_device_info_get(const tk_ctx *ctx, tk_device_info *out) {
+  if (!ctx || !out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_device_info_get: null pointer");
+  *out = ctx->info;
+  return TK_OK;
+}
+
+extern "C" int tk_set_gemm_min_m(tk_ctx *ctx, int min_m) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_min_m: null context");
+  if (min_m < 2 || min_m > 65) return tk_fail(TK_ERR_INVALID_INPUT, "gemm_min_m=%d - use an integer in 2..65", min_m);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->gemm_min_m = min_m;
+  return TK_OK;
+}
+extern "C" int tk_get_gemm_min_m(const tk_ctx *ctx) { return ctx ? ctx->gemm_min_m : 0; }
+
+// ------------------------------------------------------------------------------------------
+// weights
+// ------------------------------------------------------------------------------------------
+
+extern "C" int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k,
+                                 int format, tk_weights **out) {
+  if (!ctx || !out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_weights: null pointer");
+  *out = nullptr;
+  const size_t bb = fmt_block_bytes(format);
+  if (!bb) return tk_fail(TK_ERR_UNSUPPORTED_FORMAT, "unsupported ternary format: %d", format);
+  const size_t nb = num_blocks(k);
+  size_t row_bytes, expected;
+  if (__builtin_mul_overflow(nb, bb, &row_bytes))
+    return tk_fail(TK_ERR_INVALID_INPUT, "packed row byte count overflows");
+  if (__builtin_mul_overflow(n, row_bytes, &expected))
+    return tk_fail(TK_ERR_INVALID_INPUT, "packed weight byte count overflows");
+  if (packed_len != expected)
+    return tk_fail(TK_ERR_INVALID_INPUT, "packed len %zu != expected %zu for shape n=%zu k=%zu format %d",
+                   packed_len, expected, n, k, format);
+  if (!packed && packed_len) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_weights: null packed pointer");
+  if (n > (size_t)INT32_MAX - 16 || k > (size_t)INT32_MAX - 256)
+    return tk_fail(TK_ERR_INVALID_INPUT, "shape n=%zu k=%zu exceeds the kernels' int index range", n, k);
+
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  const size_t n_tiles = (n + 15) / 16;
+  const size_t code_bytes = n_tiles * nb * TK_CHUNK_BYTES;
+  void *codes = nullptr, *raw = nullptr;
+  TKCHK(dev_malloc(code_bytes, &codes));
+  int rc = dev_malloc(packed_len, &raw);
+  if (rc) {
+    (void)hipFree(codes);
+    return rc;
+  }
+  int invalid = INT32_MAX;
+  hipError_t e = hipSuccess;
+  if (packed_len) e = hipMemcpyAsync(raw, packed, packed_len, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(ctx->d_invalid, &invalid, sizeof invalid, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) {
+    if (format == TK_FORMAT_TQ2_0)
+      e = tk_launch_relayout_tq2(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb, ctx->d_invalid);
+    else
+      e = tk_launch_relayout_tq1(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb);
+  }
+  if (e == hipSuccess) e = hipMemcpyAsync(&invalid, ctx->d_invalid, sizeof invalid, hipMemcpyDeviceToHost, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  (void)hipFree(raw);
+  if (e != hipSuccess) {
+    (void)hipFree(codes);
+    return tk_fail(TK_ERR_BACKEND, "upload_weights: %s", hipGetErrorString(e));
+  }
+  tk_weights *w = new (std::nothrow) tk_weights();
+  if (!w) {
+    (void)hipFree(codes);
+    return tk_fail(TK_ERR_BACKEND, "tk_upload_weights: host allocation failed");
+  }
+  w->ctx = ctx;
+  w->codes = (uint8_t *)codes;
+  w->n = n;
+  w->k = k;
+  w->nb = nb;
+  w->n_tiles = n_tiles;
+  w->len_bytes = packed_len;
+  w->format = format;
+  w->invalid_row = invalid == INT32_MAX ? -1 : invalid;
+  *out = w;
+  return TK_OK;
+}
+
+extern "C" void tk_free_weights(tk_weights *w) {
+  if (!w) return;
+  std::lock_guard<std::mutex> lk(w->ctx->mu);
+  (void)hipSetDevice(w->ctx->device);
+  (void)hipStreamSynchronize(w->ctx->stream);
+  (void)hipFree(w->codes);
+  delete w;
+}
+extern "C" size_t tk_weights_len_bytes(const tk_weights *w) { return w ? w->len_bytes : 0; }
+extern "C" size_t tk_weights_n(const tk_weights *w) { return w ? w->n : 0; }
+extern "C" size_t tk_weights_k(const tk_weights *w) { return w ? w->k : 0; }
+extern "C" int tk_weights_format(const tk_weights *w) { return w ? w->format : 0; }
+
+extern "C" int tk_weights_download_trits(tk_ctx *ctx, const tk_weights *w, int8_t *trits, size_t trits_len) {
+  if (!ctx || !w || (!trits && trits_len)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_weights_download_trits: null pointer");
+  if (w->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "buffer belongs to another context");
+  if (trits_len != w->n * w->k) return tk_fail_mismatch(w->n * w->k, trits_len);
+  if (!trits_len) return TK_OK;
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  TKCHK(ensure(ctx, ctx->tmp, trits_len));
+  HIPCHK(tk_launch_decode_trits(ctx->stream, w->codes, w->n, w->k, w->nb, (int8_t *)ctx->tmp.p));
+  HIPCHK(hipMemcpyAsync(trits, ctx->tmp.p, trits_len, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// dispatch
+// ------------------------------------------------------------------------------------------
+
+static const size_t kLdsABudget = 48 * 1024;
+static const int kSkinnyMaxRows = 64;
+
+static int validate_layer(tk_ctx *ctx, const tk_linear_desc *layer, size_t *n, size_t *k) {
+  if (!layer) return tk_fail(TK_ERR_INVALID_INPUT, "null layer descriptor");
+  if (layer->n_planes < 1 || layer->n_planes > TK_MAX_PLANES)
+    return tk_fail(TK_ERR_INVALID_INPUT, "n_planes=%d - use 1..%d", layer->n_planes, TK_MAX_PLANES);
+  for (int p = 0; p < layer->n_planes; ++p) {
+    const tk_weights *w = layer->planes[p];
+    if (!w) return tk_fail(TK_ERR_INVALID_INPUT, "plane %d: null weights handle", p);
+    if (w->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "plane %d: buffer belongs to another context", p);
+    if (!layer->scales[p] && w->n) return tk_fail(TK_ERR_INVALID_INPUT, "plane %d: null scales pointer", p);
+    if (p && (w->n != layer->planes[0]->n || w->k != layer->planes[0]->k))
+      return tk_fail(TK_ERR_INVALID_INPUT, "plane %d is [%zu,%zu] but plane 0 is [%zu,%zu]", p, w->n, w->k,
+                     layer->planes[0]->n, layer->planes[0]->k);
+    if (w->invalid_row >= 0)  // what the CPU backend's unpack reports (crates/tritium-cpu/src/lib.rs:213)
+      return tk_fail(TK_ERR_BACKEND, "unpack row %ld: decoded value 2 outside ternary range", w->invalid_row);
+  }
+  *n = layer->planes[0]->n;
+  *k = layer->planes[0]->k;
+  return TK_OK;
+}
+
+struct Plan {
+  TkProblem pr;
+  TkPrep prep;
+  int prep_kind;
+  bool skinny;
+  TkLaunchCfg cfg;
+  unsigned grid_m, grid_n;
+};
+
+// Fills everything of a plan that does not depend on workspace addresses.
+static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_t k, size_t m, int mode,
+                       int out_dtype, Plan *pl) {
+  memset(pl, 0, sizeof *pl);
+  TkProblem &pr = pl->pr;
+  const size_t nb = num_blocks(k);
+  const size_t R = mode == TK_MODE_DIGITS ? 4 * m : m;
+  for (int p = 0; p < layer->n_planes; ++p) {
+    pr.codes[p] = layer->planes[p]->codes;
+    pr.scales[p] = layer->scales[p];
+  }
+  pr.n = (int)n;
+  pr.k = (int)k;
+  pr.nb = (int)nb;
+  pr.R = (int)R;
+  pr.M = (int)m;
+  pr.mode = mode;
+  pr.out_dtype = out_dtype;
+  pr.planes = layer->n_planes;
+  pr.n_tiles = (int)((n + 15) / 16);
+  const bool small = R <= (size_t)kSkinnyMaxRows && (mode == TK_MODE_DIGITS || m < (size_t)ctx->gemm_min_m);
+  pl->skinny = small;
+  pl->cfg.planes = layer->n_planes;
+  if (small) {
+    const int rt = R <= 16 ? 1 : (R <= 32 ? 2 : 4);
+    size_t kc = kLdsABudget / (256 * (R ? R : 1));
+    if (kc < 1) kc = 1;
+    if (kc > nb) kc = nb ? nb : 1;
+    pr.kc = (int)kc;
+    size_t lds_a = kc * 256 * R, lds_r = (size_t)4 * layer->n_planes * rt * 1024;
+    pl->cfg.rt = rt;
+    pl->cfg.lds_bytes = lds_a > lds_r ? lds_a : lds_r;
+    pl->cfg.grid = (unsigned)pr.n_tiles;
+  } else {
+    pl->cfg.rt = 8;
+    pl->cfg.lds_bytes = 16 * 8 * 16 * 16;
+    pl->grid_m = (unsigned)((R + 127) / 128);
+    pl->grid_n = (unsigned)((pr.n_tiles + 7) / 8);
+  }
+}
+
+static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int prep_kind, const void *act,
+                      int act_dtype, const float *act_scale_in, size_t m, void *out, int out_dtype) {
+  size_t n, k;
+  TKCHK(validate_layer(ctx, layer, &n, &k));
+  if (m == 0 || n == 0) return TK_OK;  // crates/tritium-rocm/src/rocm.rs:521-523
+  if (!act || !out) return tk_fail(TK_ERR_INVALID_INPUT, "null activation or output pointer");
+  if (out_dtype == TK_I32 && (layer->n_planes != 1 || mode != TK_MODE_INT8))
+    return tk_fail(TK_ERR_INVALID_INPUT, "raw int32 accumulators need one plane and int8 activations");
+  size_t total;
+  if (__builtin_mul_overflow(m, n, &total) || total > (size_t)INT32_MAX || m * 4 > (size_t)INT32_MAX)
+    return tk_fail(TK_ERR_INVALID_INPUT, "shape m=%zu n=%zu k=%zu exceeds the kernels' int index range", m, n, k);
+
+  Plan pl;
+  plan_shape(ctx, layer, n, k, m, mode, out_dtype, &pl);
+  const size_t nb = pl.pr.nb, R = pl.pr.R;
+  TKCHK(ensure(ctx, ctx->ap, R * nb * 256));
+  TKCHK(ensure(ctx, ctx->rowsum, R * 4));
+  TKCHK(ensure(ctx, ctx->fscale, m * 4));
+  TKCHK(ensure(ctx, ctx->aux, m * 4));
+  TKCHK(ensure(ctx, ctx->exps, m * 4));
+  TKCHK(ensure(ctx, ctx->flags, m * 4));
+
+  TkPrep &pp = pl.prep;
+  pp.act = act;
+  pp.ap = (int8_t *)ctx->ap.p;
+  pp.rowsum = (int32_t *)ctx->rowsum.p;
+  pp.act_scale = (float *)ctx->fscale.p;
+  pp.aux = (float *)ctx->aux.p;
+  pp.exps = (int32_t *)ctx->exps.p;
+  pp.flags = (uint32_t *)ctx->flags.p;
+  pp.k = k;
+  pp.nb = nb;
+  pp.R = R;
+  pp.act_dtype = act_dtype;
+  pp.m = (int)m;
+  HIPCHK(tk_launch_prep(ctx->stream, prep_kind, &pp, nullptr, 0, (unsigned)m));
+
+  TkProblem &pr = pl.pr;
+  pr.ap = pp.ap;
+  pr.rowsum = pp.rowsum;
+  pr.out = out;
+  if (prep_kind == TK_PREP_A8) {
+    pr.act_scale = pp.act_scale;
+    pr.aux = pp.aux;
+    pr.flags = pp.flags;
+    pr.raw_act = act;
+    pr.raw_dtype = act_dtype;
+  } else if (prep_kind == TK_PREP_DIGITS) {
+    pr.exps = pp.exps;
+    pr.flags = pp.flags;
+    pr.raw_act = act;
+    pr.raw_dtype = act_dtype;
+  } else {
+    pr.act_scale = act_scale_in;
+  }
+  if (pl.skinny)
+    HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
+  else
+    HIPCHK(tk_launch_gemm(ctx->stream, &pr, pl.cfg, pl.grid_m, pl.grid_n));
+  return TK_OK;
+}
+
+static int check_act_dtype(int dt) {
+  if (dt != TK_F32 && dt != TK_BF16) return tk_fail(TK_ERR_INVALID_INPUT, "activation dtype %d - use f32 or bf16", dt);
+  return TK_OK;
+}
+static int check_out_dtype(int dt, bool allow_i32) {
+  if (dt == TK_F32 || dt == TK_BF16 || (allow_i32 && dt == TK_I32)) return TK_OK;
+  return tk_fail(TK_ERR_INVALID_INPUT, "output dtype %d not supported here", dt);
+}
+
+extern "C" int tk_linear_float(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype, size_t m,
+                               void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_DIGITS, TK_PREP_DIGITS, act, act_dtype, nullptr, m, out, out_dtype);
+}
+
+extern "C" int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype, size_t m,
+                            void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, act, act_dtype, nullptr, m, out, out_dtype);
+}
+
+extern "C" int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
+                            size_t m, void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_out_dtype(out_dtype, true));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_I8, q, TK_I8, act_scale, m, out, out_dtype);
+}
+
+extern "C" int tk_linear_float_seq(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype, size_t m,
+                                   void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  size_t n, k;
+  TKCHK(validate_layer(ctx, layer, &n, &k));
+  if (m == 0 || n == 0) return TK_OK;
+  if (!act || !out) return tk_fail(TK_ERR_INVALID_INPUT, "null activation or output pointer");
+  size_t total;
+  if (__builtin_mul_overflow(m, n, &total) || total > (size_t)INT32_MAX)
+    return tk_fail(TK_ERR_INVALID_INPUT, "shape m=%zu n=%zu exceeds the kernels' int index range", m, n);
+  Plan pl;
+  plan_shape(ctx, layer, n, k, m, TK_MODE_DIGITS, out_dtype, &pl);
+  pl.pr.raw_act = act;
+  pl.pr.raw_dtype = act_dtype;
+  pl.pr.out = out;
+  HIPCHK(tk_launch_seq(ctx->stream, &pl.pr));
+  return TK_OK;
+}
+
+extern "C" int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size_t m, size_t k, int8_t *q,
+                               float *act_scale, uint32_t *nonfinite_rows) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  if (m == 0) return TK_OK;
+  if ((!act && k) || (!q && k) || !act_scale) return tk_fail(TK_ERR_INVALID_INPUT, "tk_act_quant_i8: null pointer");
+  if (m > (size_t)INT32_MAX || k > (size_t)INT32_MAX - 256)
+    return tk_fail(TK_ERR_INVALID_INPUT, "shape m=%zu k=%zu exceeds the kernels' int index range", m, k);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  TkPrep pp = {};
+  pp.act = act;
+  pp.act_scale = act_scale;
+  pp.flags = nonfinite_rows;
+  pp.q_rowmajor = q;
+  pp.k = k;
+  pp.nb = num_blocks(k);
+  pp.R = m;
+  pp.act_dtype = act_dtype;
+  pp.m = (int)m;
+  HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_A8, &pp, nullptr, 0, (unsigned)m));
+  return TK_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// trait-shaped host-slice entry points
+// ------------------------------------------------------------------------------------------
+
+static int host_call(tk_ctx *ctx, bool a8, const float *act, size_t act_len, const tk_weights *weights,
+                     const float *scales, size_t scales_len, size_t m, size_t n, size_t k, int format, float *out,
+                     size_t out_len) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  if (!weights) return tk_fail(TK_ERR_INVALID_INPUT, "buffer is not a tritium-mi355x buffer");
+  if (weights->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "buffer belongs to another context");
+  const bool identity_ok = weights->n == n && weights->k == k && weights->format == format;
+  if (a8) {
+    // the default fused path validates operand lengths first (crates/tritium-spec/src/lib.rs:275-292)
+    if (act_len != m * k) return tk_fail_mismatch(m * k, act_len);
+    if (out_len != m * n) return tk_fail_mismatch(m * n, out_len);
+    if (scales_len != n) return tk_fail_mismatch(n, scales_len);
+  }
+  if (!fmt_block_bytes(format)) return tk_fail(TK_ERR_UNSUPPORTED_FORMAT, "unsupported ternary format: %d", format);
+  if (!identity_ok)  // crates/tritium-cpu/src/lib.rs:123-135
+    return tk_fail(TK_ERR_INVALID_INPUT, "buffer identity N=%zu K=%zu format=%d does not match N=%zu K=%zu format=%d",
+                   weights->n, weights->k, weights->format, n, k, format);
+  if (act_len != m * k) return tk_fail_mismatch(m * k, act_len);      // crates/tritium-cpu/src/lib.rs:319-324
+  if (scales_len != n) return tk_fail_mismatch(n, scales_len);        // :325-330
+  if (out_len != m * n) return tk_fail_mismatch(m * n, out_len);      // :331-336
+  if (weights->invalid_row >= 0)
+    return tk_fail(TK_ERR_BACKEND, "unpack row %ld: decoded value 2 outside ternary range", weights->invalid_row);
+  if (m == 0 || n == 0) return TK_OK;
+  if ((!act && act_len) || !scales || !out) return tk_fail(TK_ERR_INVALID_INPUT, "null operand pointer");
+
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  TKCHK(ensure(ctx, ctx->h_act, act_len * 4));
+  TKCHK(ensure(ctx, ctx->h_scales, n * 4));
+  TKCHK(ensure(ctx, ctx->h_out, out_len * 4));
+  if (act_len) HIPCHK(hipMemcpyAsync(ctx->h_act.p, act, act_len * 4, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(hipMemcpyAsync(ctx->h_scales.p, scales, n * 4, hipMemcpyHostToDevice, ctx->stream));
+  tk_linear_desc layer = {};
+  layer.planes[0] = weights;
+  layer.scales[0] = (const float *)ctx->h_scales.p;
+  layer.n_planes = 1;
+  if (a8)
+    TKCHK(run_linear(ctx, &layer, TK_MODE_INT8, TK_PREP_A8, ctx->h_act.p, TK_F32, nullptr, m, ctx->h_out.p, TK_F32));
+  else
+    TKCHK(run_linear(ctx, &layer, TK_MODE_DIGITS, TK_PREP_DIGITS, ctx->h_act.p, TK_F32, nullptr, m, ctx->h_out.p, TK_F32));
+  HIPCHK(hipMemcpyAsync(out, ctx->h_out.p, out_len * 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+
+extern "C" int tk_mpgemm(tk_ctx *ctx, const float *act, size_t act_len, const tk_weights *weights,
+                         const float *scales, size_t scales_len, size_t m, size_t n, size_t k, int format,
+                         float *out, size_t out_len) {
+  return host_call(ctx, false, act, act_len, weights, scales, scales_len, m, n, k, format, out, out_len);
+}
+
+extern "C" int tk_mpgemm_with_act_quant(tk_ctx *ctx, const float *act, size_t act_len, const tk_weights *weights,
+                                        const float *scales, size_t scales_len, size_t m, size_t n, size_t k,
+                                        int format, float *out, size_t out_len) {
+  return host_call(ctx, true, act, act_len, weights, scales, scales_len, m, n, k, format, out, out_len);
+}
+
+// ------------------------------------------------------------------------------------------
+// grouped launches
+// ------------------------------------------------------------------------------------------
+
+struct tk_group {
+  tk_ctx *ctx;
+  void *ws = nullptr;        // one allocation holding every member's operand rows and side arrays
+  void *tables = nullptr;    // TkProblem[count] then TkPrep[nprep]
+  int nprobs = 0, nprep = 0, prep_kind = 0;
+  unsigned prep_rows = 0;
+  TkLaunchCfg cfg{};
+};
+
+extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size_t count, int mode, int act_dtype,
+                               int out_dtype, tk_group **out) {
+  if (!ctx || !out || (!members && count)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_group_create: null pointer");
+  *out = nullptr;
+  if (mode != TK_GROUP_FLOAT && mode != TK_GROUP_A8) return tk_fail(TK_ERR_INVALID_INPUT, "group mode %d", mode);
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  if (count == 0 || count > 65536) return tk_fail(TK_ERR_INVALID_INPUT, "group size %zu - use 1..65536", count);
+  const int kmode = mode == TK_GROUP_FLOAT ? TK_MODE_DIGITS : TK_MODE_INT8;
+  const int prep_kind = mode == TK_GROUP_FLOAT ? TK_PREP_DIGITS : TK_PREP_A8;
+
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  std::vector<Plan> plans(count);
+  std::vector<int> prep_of(count, -1);
+  std::vector<TkPrep> preps;
+  std::vector<size_t> prep_off;  // workspace offset of each distinct activation tensor
+  size_t ws_bytes = 0;
+  auto take = [&](size_t bytes) { size_t o = ws_bytes; ws_bytes += (bytes + 255) & ~(size_t)255; return o; };
+  unsigned tiles = 0, rows = 0;
+  int planes = 0, rt = 1;
+  size_t lds = 0;
+  for (size_t i = 0; i < count; ++i) {
+    size_t n, k;
+    TKCHK(validate_layer(ctx, &members[i].layer, &n, &k));
+    const size_t m = members[i].m;
+    if (!m || !n) return tk_fail(TK_ERR_INVALID_INPUT, "group member %zu is empty", i);
+    if (!members[i].act || !members[i].out) return tk_fail(TK_ERR_INVALID_INPUT, "group member %zu: null pointer", i);
+    plan_shape(ctx, &members[i].layer, n, k, m, kmode, out_dtype, &plans[i]);
+    if (!plans[i].skinny)
+      return tk_fail(TK_ERR_INVALID_INPUT, "group member %zu has %d operand rows; grouped launches take at most %d", i,
+                     plans[i].pr.R, kSkinnyMaxRows);
+    if (i == 0) planes = plans[i].cfg.planes;
+    if (plans[i].cfg.planes != planes) return tk_fail(TK_ERR_INVALID_INPUT, "group members differ in plane count");
+    if (plans[i].cfg.rt > rt) rt = plans[i].cfg.rt;
+    if (plans[i].cfg.lds_bytes > lds) lds = plans[i].cfg.lds_bytes;
+    // members reading the same activation tensor share one prep (q/k/v, gate/up)
+    for (size_t j = 0; j < i; ++j)
+      if (members[j].act == members[i].act && members[j].m == m && plans[j].pr.k == plans[i].pr.k) {
+        prep_of[i] = prep_of[j];
+        break;
+      }
+    if (prep_of[i] < 0) {
+      TkPrep pp = {};
+      const size_t R = plans[i].pr.R, nb = plans[i].pr.nb;
+      pp.act = members[i].act;
+      pp.k = k;
+      pp.nb = nb;
+      pp.R = R;
+      pp.act_dtype = act_dtype;
+      pp.m = (int)m;
+      pp.row_begin = (int)rows;
+      rows += (unsigned)m;
+      prep_of[i] = (int)preps.size();
+      preps.push_back(pp);
+      prep_off.push_back(take(R * nb * 256));
+      take(R * 4); take(m * 4); take(m * 4); take(m * 4); take(m * 4);
+    }
+    plans[i].pr.tile_begin = (int)tiles;
+    tiles += plans[i].cfg.grid;
+  }
+  size_t lds_r = (size_t)4 * planes * rt * 1024;
+  if (lds_r > lds) lds = lds_r;
+
+  tk_group *g = new (std::nothrow) tk_group();
+  if (!g) return tk_fail(TK_ERR_BACKEND, "tk_group_create: host allocation failed");
+  g->ctx = ctx;
+  int rc = dev_malloc(ws_bytes, &g->ws);
+  if (!rc) rc = dev_malloc(count * sizeof(TkProblem) + preps.size() * sizeof(TkPrep), &g->tables);
+  if (rc) {
+    if (g->ws) (void)hipFree(g->ws);
+    delete g;
+    return rc;
+  }
+  // hand out the side arrays in the same order `take` reserved them
+  for (size_t j = 0; j < preps.size(); ++j) {
+    const size_t R = preps[j].R, nb = preps[j].nb, m = (size_t)preps[j].m;
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    uint8_t *base = (uint8_t *)g->ws + prep_off[j];
+    preps[j].ap = (int8_t *)base; base += al(R * nb * 256);
+    preps[j].rowsum = (int32_t *)base; base += al(R * 4);
+    preps[j].act_scale = (float *)base; base += al(m * 4);
+    preps[j].aux = (float *)base; base += al(m * 4);
+    preps[j].exps = (int32_t *)base; base += al(m * 4);
+    preps[j].flags = (uint32_t *)base;
+  }
+  std::vector<TkProblem> probs(count);
+  for (size_t i = 0; i < count; ++i) {
+    TkProblem pr = plans[i].pr;
+    const TkPrep &pp = preps[prep_of[i]];
+    pr.ap = pp.ap;
+    pr.rowsum = pp.rowsum;
+    pr.flags = pp.flags;
+    pr.raw_act = members[i].act;
+    pr.raw_dtype = act_dtype;
+    pr.out = members[i].out;
+    if (prep_kind == TK_PREP_A8) {
+      pr.act_scale = pp.act_scale;
+      pr.aux = pp.aux;
+    } else {
+      pr.exps = pp.exps;
+    }
+    probs[i] = pr;
+  }
+  hipError_t e = hipMemcpy(g->tables, probs.data(), count * sizeof(TkProblem), hipMemcpyHostToDevice);
+  if (e == hipSuccess)
+    e = hipMemcpy((uint8_t *)g->tables + count * sizeof(TkProblem), preps.data(), preps.size() * sizeof(TkPrep),
+                  hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(g->ws);
+    (void)hipFree(g->tables);
+    delete g;
+    return tk_fail(TK_ERR_BACKEND, "tk_group_create: %s", hipGetErrorString(e));
+  }
+  g->nprobs = (int)count;
+  g->nprep = (int)preps.size();
+  g->prep_kind = prep_kind;
+  g->prep_rows = rows;
+  g->cfg.planes = planes;
+  g->cfg.rt = rt;
+  g->cfg.lds_bytes = lds;
+  g->cfg.grid = tiles;
+  *out = g;
+  return TK_OK;
+}
+
+extern "C" int tk_group_launch(tk_ctx *ctx, tk_group *g) {
+  if (!ctx || !g || g->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_group_launch: bad group");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  const TkProblem *probs = (const TkProblem *)g->tables;
+  const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
+  HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_rows));
+  HIPCHK(tk_launch_skinny(ctx->stream, nullptr, probs, g->nprobs, g->cfg));
+  return TK_OK;
+}
+
+extern "C" void tk_group_destroy(tk_group *g) {
+  if (!g) return;
+  {
+    std::lock_guard<std::mutex> lk(g->ctx->mu);
+    (void)hipSetDevice(g->ctx->device);
+    (void)hipStreamSynchronize(g->ctx->stream);
+    if (g->ws) (void)hipFree(g->ws);
+    if (g->tables) (void)hipFree(g->tables);
+  }
+  delete g;
+}
+
+// ------------------------------------------------------------------------------------------
+// plumbing
+// ------------------------------------------------------------------------------------------
+
+extern "C" int tk_malloc(tk_ctx *ctx, size_t bytes, void **dptr) {
+  if (!ctx || !dptr) return tk_fail(TK_ERR_INVALID_INPUT, "tk_malloc: null pointer");
+  HIPCHK(hipSetDevice(ctx->device));
+  return dev_malloc(bytes, dptr);
+}
+extern "C" int tk_free(tk_ctx *ctx, void *dptr) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_free: null context");
+  if (!dptr) return TK_OK;
+  HIPCHK(hipSetDevice(ctx->device));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  HIPCHK(hipFree(dptr));
+  return TK_OK;
+}
+extern "C" int tk_memcpy_h2d(tk_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  if (!ctx || ((!dst || !src) && bytes)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_memcpy_h2d: null pointer");
+  if (!bytes) return TK_OK;
+  HIPCHK(hipSetDevice(ctx->device));
+  HIPCHK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+extern "C" int tk_memcpy_d2h(tk_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  if (!ctx || ((!dst || !src) && bytes)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_memcpy_d2h: null pointer");
+  if (!bytes) return TK_OK;
+  HIPCHK(hipSetDevice(ctx->device));
+  HIPCHK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+extern "C" int tk_memset(tk_ctx *ctx, void *dst, int value, size_t bytes) {
+  if (!ctx || (!dst && bytes)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_memset: null pointer");
+  if (!bytes) return TK_OK;
+  HIPCHK(hipSetDevice(ctx->device));
+  HIPCHK(hipMemsetAsync(dst, value, bytes, ctx->stream));
+  return TK_OK;
+}
+extern "C" int tk_sync(tk_ctx *ctx) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_sync: null context");
+  HIPCHK(hipSetDevice(ctx->device));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+extern "C" void *tk_stream(tk_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+extern "C" int tk_event_create(tk_ctx *ctx, tk_event **out) {
+  if (!ctx || !out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_event_create: null pointer");
+  HIPCHK(hipSetDevice(ctx->device));
+  tk_event *ev = new (std::nothrow) tk_event();
+  if (!ev) return tk_fail(TK_ERR_BACKEND, "tk_event_create: host allocation failed");
+  hipError_t e = hipEventCreate(&ev->ev);
+  if (e != hipSuccess) {
+    delete ev;
+    return tk_fail(TK_ERR_BACKEND, "hipEventCreate: %s", hipGetErrorString(e));
+  }
+  *out = ev;
+  return TK_OK;
+}
+extern "C" int tk_event_record(tk_ctx *ctx, tk_event *ev) {
+  if (!ctx || !ev) return tk_fail(TK_ERR_INVALID_INPUT, "tk_event_record: null pointer");
+  HIPCHK(hipEventRecord(ev->ev, ctx->stream));
+  return TK_OK;
+}
+extern "C" int tk_event_elapsed_ms(tk_event *start, tk_event *stop, float *ms) {
+  if (!start || !stop || !ms) return tk_fail(TK_ERR_INVALID_INPUT, "tk_event_elapsed_ms: null pointer");
+  HIPCHK(hipEventSynchronize(stop->ev));
+  HIPCHK(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return TK_OK;
+}
+extern "C" void tk_event_destroy(tk_event *ev) {
+  if (!ev) return;
+  (void)hipEventDestroy(ev->ev);
+  delete ev;
+}
+
+extern "C" int tk_copy_kernel(tk_ctx *ctx, void *dst, const void *src, size_t bytes) {
+  if (!ctx || !dst || !src) return tk_fail(TK_ERR_INVALID_INPUT, "tk_copy_kernel: null pointer");
+  if (bytes % 16) return tk_fail(TK_ERR_INVALID_INPUT, "tk_copy_kernel: %zu bytes is not a multiple of 16", bytes);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  HIPCHK(tk_launch_copy(ctx->stream, dst, src, bytes));
+  return TK_OK;
+}

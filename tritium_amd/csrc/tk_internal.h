@@ -1,0 +1,90 @@
+// Internal declarations shared by the host API and the kernel translation unit.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/tritium_mi355x.h"
+
+// ---- device-private weight layout ("T16") -------------------------------------------------
+// A plane is cut into tiles of 16 output rows. Tile t, 256-trit block kb is one contiguous
+// 1024-byte chunk at ((t*nb + kb) * 1024). Inside a chunk, lane l = g*16 + r (r = row in tile,
+// g = 0..3) owns 16 bytes: bytes [g*16, g*16+16) of the TQ2_0 code block of row t*16+r.
+// Byte (g*16 + 4j + b), 2-bit slot s, is trit index
+//     kb*256 + (g/2)*128 + s*32 + (g%2)*16 + 4j + b            (crates/tritium-format/src/tq2.rs:15-18)
+// Rows past n are filled with 0x55 (all-zero trits). Block scales are dropped.
+#define TK_TILE_ROWS 16
+#define TK_CHUNK_BYTES 1024
+
+// ---- activation operand layout ("Ap") -----------------------------------------------------
+// int8 rows (R of them), laid out so that one 16-byte read is one MFMA A operand matching the
+// B operand obtained from dword j of a weight lane:
+//   offset((kb,j,g), row) = (((kb*4 + j)*4 + g) * R + row) * 16,   byte s*4+b inside
+// holds q[row][kb*256 + (g/2)*128 + s*32 + (g%2)*16 + 4j + b]  (0 beyond k).
+
+enum { TK_MODE_INT8 = 0, TK_MODE_DIGITS = 1 };
+
+struct TkProblem {
+  const uint8_t *codes[TK_MAX_PLANES];
+  const float *scales[TK_MAX_PLANES];
+  const int8_t *ap;          // operand rows, row stride R
+  const int32_t *rowsum;     // [R]
+  const float *act_scale;    // INT8: [M] or null
+  const float *aux;          // INT8 from float: [M] 127/gamma (for the exact fallback)
+  const int32_t *exps;       // DIGITS: [M] binary exponent of the fixed-point grid
+  const uint32_t *flags;     // [M] non-zero -> row takes the exact sequential fallback (or null)
+  const void *raw_act;       // original activations [M,K] for the fallback (or null)
+  void *out;                 // [M,N]
+  int n, k, nb, R, M;
+  int mode, raw_dtype, out_dtype, planes;
+  int tile_begin;            // first launch-wide tile index of this problem
+  int n_tiles;               // ceil(n/16)
+  int kc;                    // K blocks staged in LDS per pass (skinny kernel)
+};
+
+enum { TK_PREP_A8 = 0, TK_PREP_DIGITS = 1, TK_PREP_I8 = 2 };
+
+// One activation tensor to bring into operand order (one workgroup per token).
+struct TkPrep {
+  const void *act;      // [m,k] f32 / bf16 (A8, DIGITS) or int8 (I8)
+  int8_t *ap;           // operand rows, row stride R (may be null for A8 when only q_rowmajor is wanted)
+  int32_t *rowsum;      // [R]
+  float *act_scale;     // A8: [m]
+  float *aux;           // A8: [m] 127/gamma
+  int32_t *exps;        // DIGITS: [m]
+  uint32_t *flags;      // [m]
+  int8_t *q_rowmajor;   // A8: optional plain [m,k] int8 copy
+  size_t k, nb, R;
+  int act_dtype;
+  int row_begin;        // first launch-wide token index of this tensor
+  int m;
+};
+
+struct TkLaunchCfg {
+  int planes;   // 1..TK_MAX_PLANES
+  int rt;       // row tiles per workgroup (skinny: 1,2,4 ; gemm: 8)
+  size_t lds_bytes;
+  unsigned grid;
+};
+
+#ifdef __cplusplus
+extern "C++" {
+#endif
+// kernel launchers (tk_kernels.hip). Return hipError_t from the launch.
+hipError_t tk_launch_relayout_tq2(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb,
+                                  int *invalid_row);
+hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb);
+hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
+                                  int8_t *trits);
+hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep,
+                          unsigned rows);
+hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
+                            const TkLaunchCfg &cfg);
+hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
+                          unsigned grid_n);
+hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);
+hipError_t tk_launch_copy(hipStream_t s, void *dst, const void *src, size_t bytes);
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,709 @@
+// gfx950 (CDNA4) kernels for the packed ternary linear layer.
+//
+// Everything that contracts goes through v_mfma_i32_16x16x64_i8:
+//   * weights stay 2-bit packed in HBM and in registers; one dword (16 trits of one output row)
+//     becomes one 16-byte MFMA B operand with four shift+and pairs, as codes {0,1,2} = trit+1.
+//     The "+1" is undone with the identity  Σ_k (code-1)·a = Σ_k code·a − Σ_k a  (per-row sum Σa
+//     is produced once by the activation prep kernels).
+//   * int8 activations (the W1.58A8 decode/prefill path) are MFMA A operands directly: the int32
+//     accumulators are exact.
+//   * float activations (f32 / bf16) are split per token into four balanced base-256 digits of a
+//     31-bit fixed-point number against the token's own power-of-two exponent; the four digit rows
+//     ride in the four accumulator registers of one lane, and are recombined exactly in f64.
+//     The result is the exactly-rounded sum of the fixed-point values: tighter than the f32
+//     k-order fold it is compared with. Tokens holding NaN/Inf take an in-kernel sequential
+//     fallback that walks k in order with one f32 accumulator, like the reference does.
+//
+// Compiled with -ffp-contract=off: the epilogue multiplies must round exactly as the CPU's do.
+
+#include "tk_internal.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+#define TK_WG 256
+
+// ------------------------------------------------------------------------------------------
+// small helpers
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
+  uint32_t u = __float_as_uint(x);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_act(const void *p, int dtype, size_t idx) {
+  return dtype == TK_BF16 ? bf16_to_f32(((const uint16_t *)p)[idx]) : ((const float *)p)[idx];
+}
+
+__device__ __forceinline__ void store_out(void *out, int dtype, size_t idx, float v) {
+  if (dtype == TK_BF16)
+    ((uint16_t *)out)[idx] = f32_to_bf16_rne(v);
+  else
+    ((float *)out)[idx] = v;
+}
+
+__device__ __forceinline__ v4i expand_codes(uint32_t w) {
+  v4i b;
+  b.x = (int)(w & 0x03030303u);
+  b.y = (int)((w >> 2) & 0x03030303u);
+  b.z = (int)((w >> 4) & 0x03030303u);
+  b.w = (int)((w >> 6) & 0x03030303u);
+  return b;
+}
+
+// 2-bit code (trit+1) of element k of row n from a T16 plane.
+__device__ __forceinline__ int code_at(const uint8_t *codes, int nb, int n, int k) {
+  int kb = k >> 8, e = k & 255;
+  int c = e >> 7, s = (e & 127) >> 5, mm = e & 31;
+  int byteidx = c * 32 + mm;
+  int g = byteidx >> 4, bi = byteidx & 15;
+  size_t off = (((size_t)(n >> 4) * nb + kb) * 64 + g * 16 + (n & 15)) * 16 + bi;
+  return (codes[off] >> (2 * s)) & 3;
+}
+
+// The reference's contraction for one (token, output): one f32 accumulator, k in order,
+// add / subtract / skip (crates/tritium-core/src/reference.rs:42-51). With a8 != 0 the activation
+// is first quantized exactly as the host default does (crates/tritium-spec/src/lib.rs:369-374),
+// kept in f32 so NaN survives.
+__device__ float seq_dot(const TkProblem &pr, int p, int n, int tok, int a8) {
+  const uint8_t *codes = pr.codes[p];
+  float s = a8 ? pr.aux[tok] : 0.0f;
+  const bool gamma_zero = a8 && pr.act_scale[tok] == 0.0f;
+  float acc = 0.0f;
+  for (int k = 0; k < pr.k; ++k) {
+    int code = code_at(codes, pr.nb, n, k);
+    if (code == 1) continue;
+    float a = load_act(pr.raw_act, pr.raw_dtype, (size_t)tok * pr.k + k);
+    if (a8) {
+      if (gamma_zero) {
+        a = 0.0f;
+      } else {
+        a = rintf(__fmul_rn(a, s));
+        a = a < -128.0f ? -128.0f : (a > 127.0f ? 127.0f : a);
+      }
+    }
+    acc = (code == 2) ? __fadd_rn(acc, a) : __fsub_rn(acc, a);
+  }
+  return acc;
+}
+
+// Fold one plane's accumulators of one lane (4 consecutive operand rows starting at rowbase,
+// output column n) into the running float outputs.
+__device__ __forceinline__ void fold_plane(const TkProblem &pr, int p, int n, int rowbase, v4i v,
+                                           float out[4], bool first) {
+  const float sc = pr.scales[p][n];
+  if (pr.mode == TK_MODE_INT8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      int m = rowbase + r;
+      if (m < pr.R) {
+        float f = __fmul_rn((float)(v[r] - pr.rowsum[m]), sc);
+        out[r] = first ? f : __fadd_rn(out[r], f);
+      }
+    }
+  } else {
+    int tok = rowbase >> 2;
+    if (tok < pr.M) {
+      long long V = 0;
+#pragma unroll
+      for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(v[r] - pr.rowsum[rowbase + r]);
+      float val = (float)ldexp((double)V, pr.exps[tok]);
+      float f = __fmul_rn(val, sc);
+      out[0] = first ? f : __fadd_rn(out[0], f);
+    }
+  }
+}
+
+__device__ __forceinline__ void finish_lane(const TkProblem &pr, int n, int rowbase, float out[4]) {
+  if (pr.mode == TK_MODE_INT8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      int m = rowbase + r;
+      if (m >= pr.R) continue;
+      float f = out[r];
+      if (pr.flags && pr.flags[m]) {
+        f = 0.0f;
+        for (int p = 0; p < pr.planes; ++p) {
+          float t = __fmul_rn(seq_dot(pr, p, n, m, 1), pr.scales[p][n]);
+          f = p == 0 ? t : __fadd_rn(f, t);
+        }
+      }
+      if (pr.act_scale) f = __fmul_rn(f, pr.act_scale[m]);
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
+    }
+  } else {
+    int tok = rowbase >> 2;
+    if (tok >= pr.M) return;
+    float f = out[0];
+    if (pr.flags && pr.flags[tok]) {
+      f = 0.0f;
+      for (int p = 0; p < pr.planes; ++p) {
+        float t = __fmul_rn(seq_dot(pr, p, n, tok, 0), pr.scales[p][n]);
+        f = p == 0 ? t : __fadd_rn(f, t);
+      }
+    }
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
+  }
+}
+
+// raw int32 accumulators (single plane, INT8 mode): Σ_k q·trit
+__device__ __forceinline__ void store_raw(const TkProblem &pr, int n, int rowbase, v4i v) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    int m = rowbase + r;
+    if (m < pr.R) ((int32_t *)pr.out)[(size_t)m * pr.n + n] = v[r] - pr.rowsum[m];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// decode GEMV ("skinny"): R <= 16*RT operand rows, one workgroup per 16-row output tile.
+// The four waves split the K blocks; each streams 1 KiB weight chunks with one 128-bit load per
+// lane, expands, and issues MFMAs against A operands held in LDS.
+// ------------------------------------------------------------------------------------------
+
+template <int P, int RT>
+__global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, const TkProblem *__restrict__ table,
+                                                          int nprobs) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tile = blockIdx.x;
+  const TkProblem *prp = &single;
+  if (table) {
+    int lo = 0, hi = nprobs - 1;  // last problem with tile_begin <= tile
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (table[mid].tile_begin <= tile) lo = mid; else hi = mid - 1;
+    }
+    prp = &table[lo];
+  }
+  const TkProblem &pr = *prp;
+  const int t = tile - pr.tile_begin;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int i = lane & 15, g = lane >> 4;
+  const int nb = pr.nb, R = pr.R, kc = pr.kc;
+
+  v4i acc[P][RT];
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[p][rt] = v4i{0, 0, 0, 0};
+
+  const uint4 *ap4 = (const uint4 *)pr.ap;
+  uint4 *lds4 = (uint4 *)smem;
+
+  for (int kb0 = 0; kb0 < nb; kb0 += kc) {
+    const int kcn = min(kc, nb - kb0);
+    __syncthreads();
+    const int cnt = kcn * 16 * R;  // 16-byte pieces in this K chunk
+    const uint4 *src = ap4 + (size_t)kb0 * 16 * R;
+    for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4[idx] = src[idx];
+    __syncthreads();
+
+    for (int kbl = wave; kbl < kcn; kbl += 4) {
+      uint4 w[P];
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+        w[p] = *(const uint4 *)(pr.codes[p] + (((size_t)t * nb + kb0 + kbl) * 64 + lane) * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v4i a[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const int row = rt * 16 + i;
+          uint4 q = make_uint4(0, 0, 0, 0);
+          if (row < R) q = lds4[((kbl * 4 + j) * 4 + g) * R + row];
+          a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+        }
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          const uint32_t wj = j == 0 ? w[p].x : (j == 1 ? w[p].y : (j == 2 ? w[p].z : w[p].w));
+          const v4i b = expand_codes(wj);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[p][rt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[p][rt], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // cross-wave reduction through LDS
+  __syncthreads();
+  v4i *red = (v4i *)smem;
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) red[((wave * P + p) * RT + rt) * 64 + lane] = acc[p][rt];
+  __syncthreads();
+
+  const int n = t * 16 + i;
+  for (int rt = wave; rt < RT; rt += 4) {
+    const int rowbase = rt * 16 + 4 * g;
+    float out[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      v4i v = red[((0 * P + p) * RT + rt) * 64 + lane];
+#pragma unroll
+      for (int w2 = 1; w2 < 4; ++w2) v += red[((w2 * P + p) * RT + rt) * 64 + lane];
+      if (n < pr.n) {
+        if (pr.out_dtype == TK_I32) {
+          if (p == 0) store_raw(pr, n, rowbase, v);
+        } else {
+          fold_plane(pr, p, n, rowbase, v, out, p == 0);
+        }
+      }
+    }
+    if (n < pr.n && pr.out_dtype != TK_I32) finish_lane(pr, n, rowbase, out);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// prefill GEMM: workgroup tile = (RT*16 operand rows) x (4 waves * NT * 16 outputs).
+// A operands are staged per K block in LDS and shared by the four waves; weights are never
+// staged: each wave streams the 2-bit chunks of its own output tiles straight into registers and
+// expands them when the MFMA operand is formed.
+// ------------------------------------------------------------------------------------------
+
+template <int P, int RT, int NT>
+__global__ __launch_bounds__(TK_WG) void tk_gemm_kernel(TkProblem pr) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int i = lane & 15, g = lane >> 4;
+  const int nb = pr.nb, R = pr.R;
+  const int row0 = blockIdx.x * RT * 16;
+  const int tile0 = (blockIdx.y * 4 + wave) * NT;  // first output tile of this wave
+  uint4 *lds4 = (uint4 *)smem;
+  const uint4 *ap4 = (const uint4 *)pr.ap;
+
+  float outf[RT][NT][4];
+  v4i acc[RT][NT];
+
+#pragma unroll 1
+  for (int p = 0; p < P; ++p) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = v4i{0, 0, 0, 0};
+
+    const uint8_t *codes = pr.codes[p];
+    for (int kb = 0; kb < nb; ++kb) {
+      uint4 w[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int tl = tile0 + nt;
+        w[nt] = make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
+        if (tl < pr.n_tiles) w[nt] = *(const uint4 *)(codes + (((size_t)tl * nb + kb) * 64 + lane) * 16);
+      }
+      __syncthreads();
+      // stage A: 16 (j,g) segments of RT*16 rows each
+      for (int idx = threadIdx.x; idx < 16 * RT * 16; idx += TK_WG) {
+        const int seg = idx / (RT * 16), rr = idx % (RT * 16);
+        uint4 q = make_uint4(0, 0, 0, 0);
+        if (row0 + rr < R) q = ap4[((size_t)kb * 16 + seg) * R + row0 + rr];
+        lds4[idx] = q;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v4i b[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const uint32_t wj = j == 0 ? w[nt].x : (j == 1 ? w[nt].y : (j == 2 ? w[nt].z : w[nt].w));
+          b[nt] = expand_codes(wj);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const uint4 q = lds4[(j * 4 + g) * (RT * 16) + rt * 16 + i];
+          const v4i a = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            acc[rt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[nt], acc[rt][nt], 0, 0, 0);
+        }
+      }
+    }
+    // fold this plane
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int n = (tile0 + nt) * 16 + i;
+        const int rowbase = row0 + rt * 16 + 4 * g;
+        if (n < pr.n) {
+          if (pr.out_dtype == TK_I32) {
+            if (p == 0) store_raw(pr, n, rowbase, acc[rt][nt]);
+          } else {
+            fold_plane(pr, p, n, rowbase, acc[rt][nt], outf[rt][nt], p == 0);
+          }
+        }
+      }
+  }
+  if (pr.out_dtype == TK_I32) return;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int n = (tile0 + nt) * 16 + i;
+      const int rowbase = row0 + rt * 16 + 4 * g;
+      if (n < pr.n) finish_lane(pr, n, rowbase, outf[rt][nt]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// reference-order float kernel: one thread per (token, output)
+// ------------------------------------------------------------------------------------------
+
+__global__ __launch_bounds__(TK_WG) void tk_seq_kernel(TkProblem pr) {
+  size_t idx = (size_t)blockIdx.x * TK_WG + threadIdx.x;
+  size_t total = (size_t)pr.M * pr.n;
+  if (idx >= total) return;
+  int tok = (int)(idx / pr.n), n = (int)(idx % pr.n);
+  float f = 0.0f;
+  for (int p = 0; p < pr.planes; ++p) {
+    float t = __fmul_rn(seq_dot(pr, p, n, tok, 0), pr.scales[p][n]);
+    f = p == 0 ? t : __fadd_rn(f, t);
+  }
+  store_out(pr.out, pr.out_dtype, idx, f);
+}
+
+// ------------------------------------------------------------------------------------------
+// upload-time re-layout
+// ------------------------------------------------------------------------------------------
+
+// TQ2_0 (66-byte blocks, only 2-byte aligned) -> T16. One thread per 16-byte piece.
+__global__ void tk_relayout_tq2_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ codes, size_t n,
+                                       size_t nb, size_t pieces, int *invalid_row) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= pieces) return;
+  size_t l = idx & 63, chunk = idx >> 6;
+  size_t kb = chunk % nb, t = chunk / nb;
+  size_t row = t * 16 + (l & 15), g = l >> 4;
+  uint32_t w[4] = {0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u};
+  if (row < n) {
+    const uint8_t *src = raw + (row * nb + kb) * 66 + g * 16;
+    bool bad = false;
+    for (int d = 0; d < 4; ++d) {
+      uint32_t v = 0;
+      for (int b = 0; b < 4; ++b) {
+        uint32_t by = src[d * 4 + b];
+        bad |= (by & (by >> 1) & 0x55u) != 0;  // reserved code 3 (crates/tritium-cpu/src/lib.rs:282-292)
+        v |= by << (8 * b);
+      }
+      w[d] = v;
+    }
+    if (bad) atomicMin(invalid_row, (int)row);
+  }
+  ((uint4 *)codes)[idx] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// TQ1_0 (54-byte base-3 blocks, crates/tritium-format/src/tq1.rs:85-121) -> T16 2-bit codes.
+__global__ void tk_relayout_tq1_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ codes, size_t n,
+                                       size_t nb, size_t pieces) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= pieces) return;
+  size_t l = idx & 63, chunk = idx >> 6;
+  size_t kb = chunk % nb, t = chunk / nb;
+  size_t row = t * 16 + (l & 15), g = l >> 4;
+  uint32_t w[4] = {0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u};
+  if (row < n) {
+    const uint8_t *blk = raw + (row * nb + kb) * 54;
+    const uint32_t pow3[5] = {1, 3, 9, 27, 81};
+    for (int d = 0; d < 4; ++d) {
+      uint32_t v = 0;
+      for (int b = 0; b < 4; ++b) {
+        int byteidx = (int)g * 16 + d * 4 + b;
+        int c = byteidx >> 5, mm = byteidx & 31;
+        uint32_t by = 0;
+        for (int s = 0; s < 4; ++s) {
+          int e = c * 128 + s * 32 + mm;
+          uint32_t src, dig;
+          if (e < 160) { src = blk[e & 31]; dig = e >> 5; }
+          else if (e < 240) { src = blk[32 + ((e - 160) & 15)]; dig = (e - 160) >> 4; }
+          else { src = blk[48 + ((e - 240) & 3)]; dig = (e - 240) >> 2; }
+          uint32_t q = (src * pow3[dig]) & 0xFFu;   // u8 wraparound is part of the scheme
+          uint32_t code = (q * 3u) >> 8;            // {0,1,2} = trit + 1
+          by |= code << (2 * s);
+        }
+        v |= by << (8 * b);
+      }
+      w[d] = v;
+    }
+  }
+  ((uint4 *)codes)[idx] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ void tk_decode_trits_kernel(const uint8_t *__restrict__ codes, size_t n, size_t k, size_t nb,
+                                       int8_t *__restrict__ trits) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n * k) return;
+  int row = (int)(idx / k), kk = (int)(idx % k);
+  trits[idx] = (int8_t)(code_at(codes, (int)nb, row, kk) - 1);
+}
+
+// ------------------------------------------------------------------------------------------
+// activation prep: one workgroup per token
+// ------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ size_t ap_offset(size_t k0, size_t R, size_t row) {
+  // k0 is a multiple of 4: the dword (s, b=0..3) of piece (kb, j, g)
+  size_t kb = k0 >> 8, e = k0 & 255;
+  size_t c = e >> 7, s = (e & 127) >> 5, mm = e & 31;
+  size_t g = c * 2 + (mm >> 4), j = (mm & 15) >> 2;
+  return ((((kb * 4 + j) * 4 + g) * R + row) * 16 + s * 4);
+}
+
+__device__ float block_max(float v, float *sh) {
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  __syncthreads();
+  return r;
+}
+__device__ int block_sum(int v, int *sh) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  int r = sh[0] + sh[1] + sh[2] + sh[3];
+  __syncthreads();
+  return r;
+}
+
+// gamma = max |a| with the reference's `a > gamma` rule (NaN never wins), plus a non-finite flag.
+__device__ void row_absmax(const void *act, int dtype, size_t base, size_t k, float *sh, float &gamma,
+                           int &nonfinite, int *shi) {
+  float g = 0.0f;
+  int nf = 0;
+  for (size_t c = threadIdx.x; c < k; c += TK_WG) {
+    float a = fabsf(load_act(act, dtype, base + c));
+    if (a > g) g = a;
+    nf |= !(a <= 3.402823466e38f);  // NaN or Inf
+  }
+  gamma = block_max(g, sh);
+  nonfinite = block_sum(nf, shi) != 0;
+}
+
+__device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const TkPrep *table, int nprep, int &row) {
+  if (!table) { row = blockIdx.x; return single; }
+  int lo = 0, hi = nprep - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (table[mid].row_begin <= (int)blockIdx.x) lo = mid; else hi = mid - 1;
+  }
+  row = blockIdx.x - table[lo].row_begin;
+  return table[lo];
+}
+
+// Per-token int8 absmax quant (crates/tritium-spec/src/lib.rs:351-378) straight into operand order.
+__global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const TkPrep *__restrict__ table,
+                                                           int nprep) {
+  __shared__ float shf[4];
+  __shared__ int shi[4];
+  int rowi;
+  const TkPrep &pp = find_prep(single, table, nprep, rowi);
+  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.R;
+  const size_t base = row * k;
+  float gamma;
+  int nonfinite;
+  row_absmax(pp.act, pp.act_dtype, base, k, shf, gamma, nonfinite, shi);
+  const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
+  int sum = 0;
+  for (size_t d = threadIdx.x; d < nb * 64; d += TK_WG) {
+    const size_t k0 = d * 4;
+    uint32_t packed = 0;
+    for (int b = 0; b < 4; ++b) {
+      int q = 0;
+      if (k0 + b < k && gamma != 0.0f && !nonfinite) {
+        float a = load_act(pp.act, pp.act_dtype, base + k0 + b);
+        float r = rintf(__fmul_rn(a, s));  // one multiply, ties to even
+        r = r < -128.0f ? -128.0f : (r > 127.0f ? 127.0f : r);
+        q = (int)r;
+      }
+      sum += q;
+      packed |= ((uint32_t)q & 0xFFu) << (8 * b);
+      if (pp.q_rowmajor && k0 + b < k) pp.q_rowmajor[base + k0 + b] = (int8_t)q;
+    }
+    if (pp.ap) *(uint32_t *)(pp.ap + ap_offset(k0, R, row)) = packed;
+  }
+  sum = block_sum(sum, shi);
+  if (threadIdx.x == 0) {
+    if (pp.rowsum) pp.rowsum[row] = sum;
+    pp.act_scale[row] = gamma == 0.0f ? 0.0f : __fdiv_rn(gamma, 127.0f);
+    if (pp.aux) pp.aux[row] = s;
+    if (pp.flags) pp.flags[row] = nonfinite ? 1u : 0u;
+  }
+}
+
+// Float token -> four balanced base-256 digit rows of round(a · 2^(30-E)), 2^(E-1) <= max|a| < 2^E.
+__global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, const TkPrep *__restrict__ table,
+                                                               int nprep) {
+  __shared__ float shf[4];
+  __shared__ int shi[4];
+  int rowi;
+  const TkPrep &pp = find_prep(single, table, nprep, rowi);
+  const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.R;
+  const size_t base = tok * k;
+  float gamma;
+  int nonfinite;
+  row_absmax(pp.act, pp.act_dtype, base, k, shf, gamma, nonfinite, shi);
+  int E = 0;
+  if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
+  const int shift = 30 - E;
+  int sums[4] = {0, 0, 0, 0};
+  for (size_t d = threadIdx.x; d < nb * 64; d += TK_WG) {
+    const size_t k0 = d * 4;
+    uint32_t packed[4] = {0, 0, 0, 0};
+    for (int b = 0; b < 4; ++b) {
+      int q = 0;
+      if (k0 + b < k && gamma != 0.0f && !nonfinite)
+        q = __double2int_rn(ldexp((double)load_act(pp.act, pp.act_dtype, base + k0 + b), shift));  // |q| <= 2^30
+#pragma unroll
+      for (int dg = 0; dg < 4; ++dg) {
+        int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
+        q = (q - dv) >> 8;
+        sums[dg] += dv;
+        packed[dg] |= ((uint32_t)dv & 0xFFu) << (8 * b);
+      }
+    }
+#pragma unroll
+    for (int dg = 0; dg < 4; ++dg) *(uint32_t *)(pp.ap + ap_offset(k0, R, tok * 4 + dg)) = packed[dg];
+  }
+#pragma unroll
+  for (int dg = 0; dg < 4; ++dg) {
+    int s = block_sum(sums[dg], shi);
+    if (threadIdx.x == 0) pp.rowsum[tok * 4 + dg] = s;
+  }
+  if (threadIdx.x == 0) {
+    pp.exps[tok] = -shift;
+    pp.flags[tok] = nonfinite ? 1u : 0u;
+  }
+}
+
+// Already-quantized int8 rows -> operand order + row sums.
+__global__ __launch_bounds__(TK_WG) void tk_prep_i8_kernel(TkPrep single, const TkPrep *__restrict__ table,
+                                                           int nprep) {
+  __shared__ int shi[4];
+  int rowi;
+  const TkPrep &pp = find_prep(single, table, nprep, rowi);
+  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.R;
+  const int8_t *q = (const int8_t *)pp.act;
+  const size_t base = row * k;
+  int sum = 0;
+  for (size_t d = threadIdx.x; d < nb * 64; d += TK_WG) {
+    const size_t k0 = d * 4;
+    uint32_t packed = 0;
+    for (int b = 0; b < 4; ++b) {
+      int v = k0 + b < k ? (int)q[base + k0 + b] : 0;
+      sum += v;
+      packed |= ((uint32_t)v & 0xFFu) << (8 * b);
+    }
+    *(uint32_t *)(pp.ap + ap_offset(k0, R, row)) = packed;
+  }
+  sum = block_sum(sum, shi);
+  if (threadIdx.x == 0) pp.rowsum[row] = sum;
+}
+
+__global__ void tk_copy_kernel_dev(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+// ------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------
+
+static inline unsigned grid_for(size_t total, unsigned block) { return (unsigned)((total + block - 1) / block); }
+
+hipError_t tk_launch_relayout_tq2(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb,
+                                  int *invalid_row) {
+  size_t pieces = ((n + 15) / 16) * nb * 64;
+  if (!pieces) return hipSuccess;
+  hipLaunchKernelGGL(tk_relayout_tq2_kernel, dim3(grid_for(pieces, 256)), dim3(256), 0, s, raw, codes, n, nb, pieces,
+                     invalid_row);
+  return hipGetLastError();
+}
+
+hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb) {
+  size_t pieces = ((n + 15) / 16) * nb * 64;
+  if (!pieces) return hipSuccess;
+  hipLaunchKernelGGL(tk_relayout_tq1_kernel, dim3(grid_for(pieces, 256)), dim3(256), 0, s, raw, codes, n, nb, pieces);
+  return hipGetLastError();
+}
+
+hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb, int8_t *trits) {
+  if (!(n * k)) return hipSuccess;
+  hipLaunchKernelGGL(tk_decode_trits_kernel, dim3(grid_for(n * k, 256)), dim3(256), 0, s, codes, n, k, nb, trits);
+  return hipGetLastError();
+}
+
+hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep,
+                          unsigned rows) {
+  if (!rows) return hipSuccess;
+  TkPrep dummy = {};
+  const TkPrep &sg = single ? *single : dummy;
+  switch (kind) {
+    case TK_PREP_A8: hipLaunchKernelGGL(tk_prep_a8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep); break;
+    case TK_PREP_DIGITS: hipLaunchKernelGGL(tk_prep_digits_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep); break;
+    case TK_PREP_I8: hipLaunchKernelGGL(tk_prep_i8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+template <int P>
+static hipError_t launch_skinny_p(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
+                                  const TkLaunchCfg &cfg) {
+  TkProblem dummy = {};
+  const TkProblem &sg = single ? *single : dummy;
+  dim3 grid(cfg.grid), block(TK_WG);
+  switch (cfg.rt) {
+    case 1: hipLaunchKernelGGL((tk_skinny_kernel<P, 1>), grid, block, cfg.lds_bytes, s, sg, table, nprobs); break;
+    case 2: hipLaunchKernelGGL((tk_skinny_kernel<P, 2>), grid, block, cfg.lds_bytes, s, sg, table, nprobs); break;
+    case 4: hipLaunchKernelGGL((tk_skinny_kernel<P, 4>), grid, block, cfg.lds_bytes, s, sg, table, nprobs); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
+                            const TkLaunchCfg &cfg) {
+  if (!cfg.grid) return hipSuccess;
+  switch (cfg.planes) {
+    case 1: return launch_skinny_p<1>(s, single, table, nprobs, cfg);
+    case 2: return launch_skinny_p<2>(s, single, table, nprobs, cfg);
+    case 3: return launch_skinny_p<3>(s, single, table, nprobs, cfg);
+    case 4: return launch_skinny_p<4>(s, single, table, nprobs, cfg);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
+                          unsigned grid_n) {
+  if (!grid_m || !grid_n) return hipSuccess;
+  dim3 grid(grid_m, grid_n), block(TK_WG);
+  switch (cfg.planes) {
+    case 1: hipLaunchKernelGGL((tk_gemm_kernel<1, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 2: hipLaunchKernelGGL((tk_gemm_kernel<2, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 3: hipLaunchKernelGGL((tk_gemm_kernel<3, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 4: hipLaunchKernelGGL((tk_gemm_kernel<4, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single) {
+  size_t total = (size_t)single->M * single->n;
+  if (!total) return hipSuccess;
+  hipLaunchKernelGGL(tk_seq_kernel, dim3(grid_for(total, TK_WG)), dim3(TK_WG), 0, s, *single);
+  return hipGetLastError();
+}
+
+hipError_t tk_launch_copy(hipStream_t s, void *dst, const void *src, size_t bytes) {
+  size_t n16 = bytes / 16;
+  if (!n16) return hipSuccess;
+  unsigned grid = (unsigned)((n16 + 255) / 256);
+  if (grid > 256 * 32) grid = 256 * 32;
+  hipLaunchKernelGGL(tk_copy_kernel_dev, dim3(grid), dim3(256), 0, s, (uint4 *)dst, (const uint4 *)src, n16);
+  return hipGetLastError();
+}
