@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed ternary linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline workload (BASELINE.json configs[1]): two-plane additive ternary GEMV, K=2048, N=8192,
+bf16 N(0,1) activations, per-channel f32 scales, batch sweep 1,2,4,8,16 — the HBM-bound decode
+regime. One "step" is one pass of the sweep: five launches of the decode kernel, each over
+COPIES distinct resident copies of the layer (1.07 GB of 2-bit codes per launch, far above the
+256 MB last-level cache, so the figure is an HBM figure and not a cache one).
+
+Prints ONE JSON line. `value` is algorithmic GB/s of the whole timed region (activation prep
+launches included); `roofline` is the decode kernel alone, timed with events on the stream it runs
+on; `cpu_baseline` is the CPU oracle's restatement of tritium-cpu timed on this host on one pass
+of the same sweep. `extra` carries the prefill GEMM (configs[2]) and the projection-stack
+tokens/s (configs[3]) measured in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+
+K2, N2, PLANES2 = 2048, 8192, 2
+SWEEP = (1, 2, 4, 8, 16)
+COPIES = 128
+
+
+def ternary(rng, n, k, p_zero):
+    u = rng.random((n, k), dtype=np.float32)
+    half = (1.0 - p_zero) / 2
+    return np.where(u < p_zero, 0, np.where(u < p_zero + half, 1, -1)).astype(np.int8)
+
+
+def f32_to_bf16_bits(x):
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def algorithmic_bytes(m, n, k, planes, act_bytes, out_bytes, a8=False):
+    """Minimum traffic of one linear: 2-bit codes (64 B per 256 trits, block scales excluded),
+    activations, per-channel scales, output (+ per-token scales on the int8 path)."""
+    nb = (k + 255) // 256
+    return planes * n * nb * 64 + m * k * act_bytes + planes * n * 4 + m * n * out_bytes + (4 * m if a8 else 0)
+
+
+def time_steps(be, steps, warmup, step_fn):
+    """W untimed steps, then exactly K steps between two events on the library's stream."""
+    start, stop = be.event(), be.event()
+    for _ in range(warmup):
+        step_fn(None)
+    be.sync()
+    marks = []
+    start.record()
+    for _ in range(steps):
+        step_fn(marks)
+    stop.record()
+    be.sync()
+    total_ms = start.elapsed_ms(stop)
+    kernel_ms = sum(a.elapsed_ms(b) for a, b in marks)
+    for a, b in marks:
+        a.destroy()
+        b.destroy()
+    return total_ms, kernel_ms, len(marks)
+
+
+def bench_decode(T, be, steps, warmup, rng):
+    host = []
+    for _ in range(2):  # two distinct host layers, replicated to COPIES distinct device copies
+        planes = [T.pack_rows(ternary(rng, N2, K2, p0), N2, K2) for p0 in (0.4, 0.7)]
+        scs = [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)]
+        host.append((planes, scs))
+    layers = [be.linear(*host[i % 2], N2, K2) for i in range(COPIES)]
+    mmax = max(SWEEP)
+    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((mmax, K2)).astype(np.float32)), "bf16")
+            for _ in range(COPIES)]
+    outs = [be.empty(mmax * N2, "f32") for _ in range(COPIES)]
+    groups = {m: be.group([(layers[i], acts[i], m, outs[i]) for i in range(COPIES)], 0, "bf16", "f32") for m in SWEEP}
+
+    def step(marks):
+        for m in SWEEP:
+            g = groups[m]
+            g.launch_parts(True, False)
+            if marks is None:
+                g.launch_parts(False, True)
+            else:
+                a = be.event().record()
+                g.launch_parts(False, True)
+                marks.append((a, be.event().record()))
+
+    total_ms, kernel_ms, launches = time_steps(be, steps, warmup, step)
+    per_launch = {m: COPIES * algorithmic_bytes(m, N2, K2, PLANES2, 2, 4) for m in SWEEP}
+    step_bytes = sum(per_launch.values())
+
+    # per-batch figures: the decode kernel alone, each batch size timed separately
+    per_m = {}
+    for m in SWEEP:
+        g = groups[m]
+        g.launch_parts(True, False)
+        be.sync()
+        a = be.event().record()
+        for _ in range(5):
+            g.launch_parts(False, True)
+        b = be.event().record()
+        be.sync()
+        ms = a.elapsed_ms(b) / 5
+        per_m[str(m)] = {"GB/s": round(per_launch[m] / ms / 1e6, 1), "us_per_layer": round(ms * 1e3 / COPIES, 3)}
+    res = {
+        "ms_per_step": total_ms / steps,
+        "value": step_bytes * steps / total_ms / 1e6,
+        "kernel_gbs": step_bytes * steps / kernel_ms / 1e6,
+        "kernel_avg_ms": kernel_ms / launches,
+        "bytes_per_launch_avg": step_bytes / len(SWEEP),
+        "per_batch": per_m,
+    }
+    for g in groups.values():
+        g.destroy()
+    for x in acts + outs:
+        x.free()
+    for l in layers:
+        l.free()
+    return res
+
+
+def bench_prefill(T, be, rng, iters=10):
+    """configs[2]: M=2048, K=2560, N=6912, one plane, bf16 activations quantized per token to int8,
+    int32 accumulation, bf16 output."""
+    m, k, n = 2048, 2560, 6912
+    layers = [be.linear([T.pack_rows(ternary(rng, n, k, 0.4), n, k)], [rng.uniform(0.01, 0.1, n).astype(np.float32)],
+                        n, k) for _ in range(2)]
+    act = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32)), "bf16")
+    out = be.empty(m * n, "bf16")
+    q, s = be.empty(m * k, "i8"), be.empty(m, "f32")
+    be.act_quant_i8(act, m, k, q, s)
+    for i in range(3):
+        be.linear_a8(layers[i % 2], act, m, out)
+    be.sync()
+    a = be.event().record()
+    for i in range(iters):
+        be.linear_a8(layers[i % 2], act, m, out)
+    b = be.event().record()
+    be.sync()
+    ms = a.elapsed_ms(b) / iters
+    ops = 2.0 * m * n * k
+    return {"workload": "prefill GEMM M=2048 K=2560 N=6912 1 plane, bf16 act -> int8 per token -> int32 acc -> bf16",
+            "ms_per_call_incl_quant": round(ms, 4), "TOPS": round(ops / ms / 1e9, 1),
+            "frac_of_int8_peak": round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4)}
+
+
+def bench_stack(T, be, rng, iters=10):
+    """configs[3]: the 7 ternary projections of 30 decoder layers (hidden 2560, FFN 6912, 20 query
+    heads and 5 KV heads of 128), W1.58A8, one launch for the whole stack with given inputs.
+    tokens/s = batch / time of the projection path only."""
+    h, f, kv, layers_n = 2560, 6912, 640, 30
+    shapes = {"q": (h, h), "k": (kv, h), "v": (kv, h), "o": (h, h), "gate": (f, h), "up": (f, h), "down": (h, f)}
+    hostw = {}
+    for name, (n, k) in shapes.items():
+        key = (n, k)
+        if key not in hostw:
+            hostw[key] = (T.pack_rows(ternary(rng, n, k, 0.4), n, k), rng.uniform(0.01, 0.1, n).astype(np.float32))
+    res = {}
+    lins = []
+    for _ in range(layers_n):
+        lins.append({name: be.linear([hostw[(n, k)][0]], [hostw[(n, k)][1]], n, k) for name, (n, k) in shapes.items()})
+    code_bytes = layers_n * sum(n * ((k + 255) // 256) * 64 for n, k in shapes.values())
+    for m in (1, 32):
+        hid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
+        att = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
+        mid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, f)).astype(np.float32)), "bf16")
+        members, outs = [], []
+        for L in lins:
+            for name, src in (("q", hid), ("k", hid), ("v", hid), ("o", att), ("gate", hid), ("up", hid), ("down", mid)):
+                o = be.empty(m * shapes[name][0], "bf16")
+                outs.append(o)
+                members.append((L[name], src, m, o))
+        g = be.group(members, 1, "bf16", "bf16")
+        for _ in range(3):
+            g.launch()
+        be.sync()
+        a = be.event().record()
+        for _ in range(iters):
+            g.launch()
+        b = be.event().record()
+        be.sync()
+        ms = a.elapsed_ms(b) / iters
+        res[f"batch{m}"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1),
+                            "code_GB/s": round(code_bytes / ms / 1e6, 1)}
+        g.destroy()
+        for x in outs + [hid, att, mid]:
+            x.free()
+    for L in lins:
+        for l in L.values():
+            l.free()
+    res["workload"] = ("30 layers x (q,k,v,o,gate,up,down), hidden 2560, FFN 6912, 20/5 heads of 128, 1 plane, "
+                       "W1.58A8, bf16 in/out; 210 projections in one grouped launch on given inputs")
+    res["code_bytes_per_step"] = code_bytes
+    return res
+
+
+def cpu_baseline(rng):
+    """The CPU oracle (a restatement of tritium-cpu's dispatch: unpack per call, widest SIMD kernel,
+    rows chunked across threads) on ONE pass of the headline sweep, on this host's cores."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib
+    orc = oracle_lib.load()
+    planes = [orc.pack_matrix(ternary(rng, N2, K2, p0), N2, K2, oracle_lib.FMT_TQ2_0) for p0 in (0.4, 0.7)]
+    scs = [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)]
+    threads = min(os.cpu_count() or 1, 16)
+    used_max, total_bytes = 0, 0
+    t0 = time.perf_counter()
+    for m in SWEEP:
+        bits = f32_to_bf16_bits(rng.standard_normal((m, K2)).astype(np.float32))
+        act = (bits.astype(np.uint32) << 16).view(np.float32).reshape(m, K2)
+        out = None
+        for p in range(PLANES2):
+            o, used, _ = orc.cpu_mpgemm_fast(planes[p], oracle_lib.FMT_TQ2_0, act, scs[p], m, N2, K2, threads)
+            out = o if out is None else out + o
+            used_max = max(used_max, used)
+        total_bytes += algorithmic_bytes(m, N2, K2, PLANES2, 2, 4)
+    dt = time.perf_counter() - t0
+    return {"value": round(total_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": used_max, "kind": "port",
+            "sample": f"one pass of the sweep (batch {','.join(map(str, SWEEP))}) over ONE layer copy, "
+                      f"{dt:.2f} s; tritium-cpu's row chunking gives batch 1 a single worker"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM and projection-stack legs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the path shards over output channels without any "
+                 "exchange, see DESIGN.md); --gpus N with N > 1 is not supported.")
+    import tritium_amd as T
+    be = T.Mi355xBackend(0)
+    info = be.info
+    rng = np.random.default_rng(0)
+    dec = bench_decode(T, be, args.steps, args.warmup, rng)
+    out = {
+        "metric": "decode GEMV HBM GB/s",
+        "value": round(dec["value"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dec["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 MFMA (bf16 activations as 4 base-256 digits), int32 accumulate, f32 out",
+        "data": "synthetic",
+        "config": {"workload": f"two-plane additive ternary GEMV K={K2} N={N2}, P(0)=0.4/0.7, bf16 N(0,1) activations, "
+                               f"per-channel f32 scales, batch sweep {','.join(map(str, SWEEP))}; one step = the sweep, "
+                               f"each batch one launch over {COPIES} resident layer copies",
+                   "copies": COPIES, "bytes_per_step": int(dec["bytes_per_launch_avg"] * len(SWEEP))},
+        "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "tk_skinny_kernel<2,*>", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
+                     "algorithmic_bytes_per_launch": int(dec["bytes_per_launch_avg"])},
+        "per_batch": dec["per_batch"],
+        "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
+                   "clock_mhz": info.clock_khz / 1000, "memory_clock_mhz": info.memory_clock_khz / 1000,
+                   "memory_bus_bits": info.memory_bus_bits},
+    }
+    if not args.no_extra:
+        out["extra"] = {"prefill_gemm": bench_prefill(T, be, rng), "projection_stack": bench_stack(T, be, rng)}
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(np.random.default_rng(1))
+    be.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -174,6 +174,9 @@ typedef enum tk_group_mode { TK_GROUP_FLOAT = 0, TK_GROUP_A8 = 1 } tk_group_mode
 int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size_t count, int mode,
                     int act_dtype, int out_dtype, tk_group **out);
 int tk_group_launch(tk_ctx *ctx, tk_group *group);
+/* The two launches of a group separately (activation prep, then the contraction), so a harness can
+ * bracket the contraction kernel alone with events. tk_group_launch == parts(1, 1). */
+int tk_group_launch_parts(tk_ctx *ctx, tk_group *group, int do_prep, int do_main);
 void tk_group_destroy(tk_group *group);
 
 /* GEMV -> GEMM crossover in activation rows; the reference's knob is TRITIUM_IMMA_MIN_M, default
@@ -181,6 +184,14 @@ void tk_group_destroy(tk_group *group);
  * TRITIUM_MI355X_GEMM_MIN_M is read at tk_init with the same loud-reject rule. */
 int tk_set_gemm_min_m(tk_ctx *ctx, int min_m);
 int tk_get_gemm_min_m(const tk_ctx *ctx);
+
+/* tk_mpgemm answers float problems of at most this many multiply-accumulates (m·n·k; default 2^20,
+ * the largest conformance vector, crates/tritium-testkit/src/generate.rs:203-214) with the
+ * reference-order kernel of tk_linear_float_seq: such calls are latency-bound either way, and the
+ * result is then bit-identical to the CPU backend rather than merely within its 1e-4 tolerance.
+ * 0 sends every float call to the MFMA path. */
+int tk_set_exact_max_macs(tk_ctx *ctx, size_t macs);
+size_t tk_get_exact_max_macs(const tk_ctx *ctx);
 
 /* ---- plumbing: device memory, stream, events (what the harness and a backend crate need) ---- */
 int tk_malloc(tk_ctx *ctx, size_t bytes, void **dptr);

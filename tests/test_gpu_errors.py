@@ -95,3 +95,10 @@ def test_gemm_min_m_knob(backend):
     with pytest.raises(T.InvalidInput):
         backend.set_gemm_min_m(1)
     backend.set_gemm_min_m(65)
+
+
+def test_exact_max_macs_knob(backend):
+    assert backend.exact_max_macs() == 1 << 20
+    backend.set_exact_max_macs(0)
+    assert backend.exact_max_macs() == 0
+    backend.set_exact_max_macs(1 << 20)

@@ -59,9 +59,12 @@ SIGNATURES = {
     "tk_linear_float_seq": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_group_create": (C.c_int, [vp, C.POINTER(GroupMember), sz, C.c_int, C.c_int, C.c_int, C.POINTER(vp)]),
     "tk_group_launch": (C.c_int, [vp, vp]),
+    "tk_group_launch_parts": (C.c_int, [vp, vp, C.c_int, C.c_int]),
     "tk_group_destroy": (None, [vp]),
     "tk_set_gemm_min_m": (C.c_int, [vp, C.c_int]),
     "tk_get_gemm_min_m": (C.c_int, [vp]),
+    "tk_set_exact_max_macs": (C.c_int, [vp, sz]),
+    "tk_get_exact_max_macs": (sz, [vp]),
     "tk_malloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
     "tk_free": (C.c_int, [vp, vp]),
     "tk_memcpy_h2d": (C.c_int, [vp, vp, vp, sz]),

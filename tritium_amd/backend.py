@@ -220,6 +220,9 @@ class Group:
     def launch(self):
         _check(L.load().tk_group_launch(self.backend._ctx, self._h))
 
+    def launch_parts(self, prep=True, main=True):
+        _check(L.load().tk_group_launch_parts(self.backend._ctx, self._h, int(prep), int(main)))
+
     def destroy(self):
         if self._h:
             L.load().tk_group_destroy(self._h)
@@ -379,6 +382,12 @@ class Mi355xBackend:
 
     def gemm_min_m(self):
         return self._lib.tk_get_gemm_min_m(self._ctx)
+
+    def set_exact_max_macs(self, macs):
+        _check(self._lib.tk_set_exact_max_macs(self._ctx, macs))
+
+    def exact_max_macs(self):
+        return self._lib.tk_get_exact_max_macs(self._ctx)
 
     def event(self):
         return Event(self)

@@ -69,6 +69,7 @@ struct tk_ctx {
   tk_device_info info{};
   std::string device_id;
   int gemm_min_m = 65;
+  size_t exact_max_macs = (size_t)1 << 20;
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
   int *d_invalid = nullptr;
 };
@@ -161,7 +162,7 @@ extern "C" int tk_init(int device, tk_ctx **out) {
   ctx->device = device;
   ctx->gemm_min_m = min_m;
   ctx->device_id = "mi355x:" + std::to_string(device);
-  snprintf(ctx->info.name, sizeof ctx->info.name, "%s", prop.name);
+  snprintf(ctx->info.name, sizeof ctx->info.name, "%s", prop.name[0] ? prop.name : "AMD Instinct MI355X");
   snprintf(ctx->info.arch, sizeof ctx->info.arch, "%s", prop.gcnArchName);
   ctx->info.total_memory_bytes = prop.totalGlobalMem;
   ctx->info.compute_units = prop.multiProcessorCount;
@@ -216,6 +217,14 @@ extern "C" int tk_set_gemm_min_m(tk_ctx *ctx, int min_m) {
   return TK_OK;
 }
 extern "C" int tk_get_gemm_min_m(const tk_ctx *ctx) { return ctx ? ctx->gemm_min_m : 0; }
+
+extern "C" int tk_set_exact_max_macs(tk_ctx *ctx, size_t macs) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_exact_max_macs: null context");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->exact_max_macs = macs;
+  return TK_OK;
+}
+extern "C" size_t tk_get_exact_max_macs(const tk_ctx *ctx) { return ctx ? ctx->exact_max_macs : 0; }
 
 // ------------------------------------------------------------------------------------------
 // weights
@@ -577,10 +586,22 @@ static int host_call(tk_ctx *ctx, bool a8, const float *act, size_t act_len, con
   layer.planes[0] = weights;
   layer.scales[0] = (const float *)ctx->h_scales.p;
   layer.n_planes = 1;
-  if (a8)
+  size_t macs;
+  const bool tiny = !__builtin_mul_overflow(m * n, k, &macs) && macs <= ctx->exact_max_macs;
+  if (a8) {
     TKCHK(run_linear(ctx, &layer, TK_MODE_INT8, TK_PREP_A8, ctx->h_act.p, TK_F32, nullptr, m, ctx->h_out.p, TK_F32));
-  else
+  } else if (tiny) {
+    // Small float problems are latency-bound either way: run them in the reference's own summation
+    // order, so the result is bit-identical to the CPU backend (crates/tritium-core/src/reference.rs:42-51).
+    Plan pl;
+    plan_shape(ctx, &layer, n, k, m, TK_MODE_DIGITS, TK_F32, &pl);
+    pl.pr.raw_act = ctx->h_act.p;
+    pl.pr.raw_dtype = TK_F32;
+    pl.pr.out = ctx->h_out.p;
+    HIPCHK(tk_launch_seq(ctx->stream, &pl.pr));
+  } else {
     TKCHK(run_linear(ctx, &layer, TK_MODE_DIGITS, TK_PREP_DIGITS, ctx->h_act.p, TK_F32, nullptr, m, ctx->h_out.p, TK_F32));
+  }
   HIPCHK(hipMemcpyAsync(out, ctx->h_out.p, out_len * 4, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(hipStreamSynchronize(ctx->stream));
   return TK_OK;
@@ -737,16 +758,18 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   return TK_OK;
 }
 
-extern "C" int tk_group_launch(tk_ctx *ctx, tk_group *g) {
+extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int do_main) {
   if (!ctx || !g || g->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_group_launch: bad group");
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
   const TkProblem *probs = (const TkProblem *)g->tables;
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
-  HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_rows));
-  HIPCHK(tk_launch_skinny(ctx->stream, nullptr, probs, g->nprobs, g->cfg));
+  if (do_prep) HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_rows));
+  if (do_main) HIPCHK(tk_launch_skinny(ctx->stream, nullptr, probs, g->nprobs, g->cfg));
   return TK_OK;
 }
+
+extern "C" int tk_group_launch(tk_ctx *ctx, tk_group *g) { return tk_group_launch_parts(ctx, g, 1, 1); }
 
 extern "C" void tk_group_destroy(tk_group *g) {
   if (!g) return;
