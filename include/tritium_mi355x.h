@@ -185,6 +185,17 @@ void tk_group_destroy(tk_group *group);
 int tk_set_gemm_min_m(tk_ctx *ctx, int min_m);
 int tk_get_gemm_min_m(const tk_ctx *ctx);
 
+/* The decode path has two kernels with identical results: one splits K over the waves of a
+ * workgroup (fine grain, for a single narrow layer) and one streams whole output tiles per wave
+ * (for launches that fill the chip). The streaming form is taken when a launch needs at least
+ * this many workgroups; default = the device's CU count. */
+/* Force one decode kernel for every later launch: 0 automatic, 1 K-split, 2 streaming (K passes
+ * through LDS), 3 flow (all of K resident in LDS; falls back to 2 when it does not fit). All give
+ * identical bits; the knob exists for tests and tuning. */
+int tk_set_decode_kernel(tk_ctx *ctx, int variant);
+int tk_set_stream_min_groups(tk_ctx *ctx, int groups);
+int tk_get_stream_min_groups(const tk_ctx *ctx);
+
 /* tk_mpgemm answers float problems of at most this many multiply-accumulates (m·n·k; default 2^20,
  * the largest conformance vector, crates/tritium-testkit/src/generate.rs:203-214) with the
  * reference-order kernel of tk_linear_float_seq: such calls are latency-bound either way, and the

@@ -16,6 +16,15 @@ DECODE_SHAPES = [(1, 1, 1), (1, 7, 300), (5, 130, 257), (64, 3, 2560), (3, 33, 6
 GEMM_SHAPES = [(65, 8, 256), (100, 50, 700), (130, 257, 512), (128, 40, 2560), (200, 129, 300), (257, 16, 256)]
 
 
+@pytest.fixture(params=["ksplit", "stream", "flow"], autouse=True)
+def decode_kernel(request, backend):
+    """Every case runs through all three decode kernels: K-split (default for narrow launches),
+    streaming and flow (forced here; the defaults for launches that fill the chip)."""
+    backend.set_decode_kernel({"ksplit": 1, "stream": 2, "flow": 3}[request.param])
+    yield request.param
+    backend.set_decode_kernel(0)
+
+
 def _layer(backend, oracle, ws, scs, fmt=FMT_TQ2_0):
     n, k = ws[0].shape
     packed = [oracle.pack_matrix(w, n, k, fmt) for w in ws]
@@ -283,3 +292,57 @@ def test_ternary_linear_forward(backend, oracle):
     assert same_bits(out, want)
     with pytest.raises(T.ShapeMismatch):
         lin.forward(backend, act[:, :-1], m, out)
+
+
+def test_streaming_kernel_by_default_on_wide_launch(backend, oracle, decode_kernel):
+    """A launch wide enough to take the streaming kernel on its own (>= one workgroup per CU), ragged
+    tile count, three planes, 64 operand rows -> two LDS passes over K."""
+    if decode_kernel != "stream":
+        pytest.skip("single configuration")
+    backend.set_decode_kernel(0)
+    rng = np.random.default_rng(41)
+    m, n, k = 64, 33000, 1300
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)]
+    scs = [scales(rng, n) for _ in range(3)]
+    packed = [T.pack_rows(w, n, k) for w in ws]
+    layer = backend.linear(packed, scs, n, k)
+    q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    s_a = rng.uniform(0.001, 0.1, m).astype(np.float32)
+    dq, ds, dout = backend.to_device(q, "i8"), backend.to_device(s_a, "f32"), backend.empty(m * n, "f32")
+    backend.linear_i8(layer, dq, ds, m, dout)
+    got = dout.to_host().reshape(m, n)
+    accs = [q.astype(np.int32) @ w.T.astype(np.int32) for w in ws]  # exact integer reference
+    want = np.zeros((m, n), np.float32)
+    for p, (a, sc) in enumerate(zip(accs, scs)):
+        t = a.astype(np.float32) * sc[None, :]
+        want = t if p == 0 else want + t
+    want = want * s_a[:, None]
+    assert same_bits(got, want)
+    rows = [0, 31, 63]
+    for p in range(3):
+        assert (oracle.int8_accumulators(packed[p], FMT_TQ2_0, q[rows], 3, n, k) == accs[p][rows]).all()
+
+
+def test_flow_kernel_by_default_on_wide_launch(backend, oracle, decode_kernel):
+    """Wide launch whose operand rows fit in LDS: takes the flow kernel on its own. Ragged tile count
+    (runs clamp at the end of the plane), two planes, bf16 in, bf16 out."""
+    if decode_kernel != "flow":
+        pytest.skip("single configuration")
+    backend.set_decode_kernel(0)
+    rng = np.random.default_rng(43)
+    m, n, k = 3, 70001, 700
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7)]
+    scs = [scales(rng, n) for _ in range(2)]
+    packed = [T.pack_rows(w, n, k) for w in ws]
+    layer = backend.linear(packed, scs, n, k)
+    bits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    act = bf16_bits_to_f32(bits).reshape(m, k)
+    dact, dout = backend.to_device(bits, "bf16"), backend.empty(m * n, "f32")
+    backend.linear_float(layer, dact, m, dout)
+    got = dout.to_host().reshape(m, n)
+    want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    assert rel_err(got, want) <= 1e-3 and accepts(got, want).all()
+    dob = backend.empty(m * n, "bf16")
+    backend.linear_a8(layer, dact, m, dob)
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    assert (dob.to_host() == f32_to_bf16_bits(want).reshape(-1)).all()

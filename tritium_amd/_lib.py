@@ -63,6 +63,9 @@ SIGNATURES = {
     "tk_group_destroy": (None, [vp]),
     "tk_set_gemm_min_m": (C.c_int, [vp, C.c_int]),
     "tk_get_gemm_min_m": (C.c_int, [vp]),
+    "tk_set_decode_kernel": (C.c_int, [vp, C.c_int]),
+    "tk_set_stream_min_groups": (C.c_int, [vp, C.c_int]),
+    "tk_get_stream_min_groups": (C.c_int, [vp]),
     "tk_set_exact_max_macs": (C.c_int, [vp, sz]),
     "tk_get_exact_max_macs": (sz, [vp]),
     "tk_malloc": (C.c_int, [vp, sz, C.POINTER(vp)]),

@@ -383,6 +383,16 @@ class Mi355xBackend:
     def gemm_min_m(self):
         return self._lib.tk_get_gemm_min_m(self._ctx)
 
+    def set_decode_kernel(self, variant):
+        """0 automatic, 1 K-split, 2 streaming, 3 flow."""
+        _check(self._lib.tk_set_decode_kernel(self._ctx, variant))
+
+    def set_stream_min_groups(self, groups):
+        _check(self._lib.tk_set_stream_min_groups(self._ctx, groups))
+
+    def stream_min_groups(self):
+        return self._lib.tk_get_stream_min_groups(self._ctx)
+
     def set_exact_max_macs(self, macs):
         _check(self._lib.tk_set_exact_max_macs(self._ctx, macs))
 

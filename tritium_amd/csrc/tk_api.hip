@@ -70,6 +70,8 @@ struct tk_ctx {
   std::string device_id;
   int gemm_min_m = 65;
   size_t exact_max_macs = (size_t)1 << 20;
+  int stream_min_groups = 0;  // set at init to the CU count
+  int decode_force = 0;  // DECODE_AUTO
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
   int *d_invalid = nullptr;
 };
@@ -119,6 +121,21 @@ static inline size_t fmt_block_bytes(int format) {
 }
 static inline size_t dtype_size(int dt) { return dt == TK_BF16 ? 2 : (dt == TK_I8 ? 1 : 4); }
 
+static bool prefer_stream(const tk_ctx *ctx, unsigned groups) { return groups >= (unsigned)ctx->stream_min_groups; }
+
+// Which decode kernel a launch takes. All three give identical bits.
+static int choose_decode(const tk_ctx *ctx, bool flow_ok, unsigned flow_groups, unsigned stream_groups) {
+  switch (ctx->decode_force) {
+    case 1: return 1;
+    case 2: return 2;
+    case 3: return flow_ok ? 3 : 2;
+    default: break;
+  }
+  if (flow_ok && prefer_stream(ctx, flow_groups)) return 3;
+  if (!flow_ok && prefer_stream(ctx, stream_groups)) return 2;
+  return 1;
+}
+
 // ------------------------------------------------------------------------------------------
 // lifetime
 // ------------------------------------------------------------------------------------------
@@ -166,6 +183,7 @@ extern "C" int tk_init(int device, tk_ctx **out) {
   snprintf(ctx->info.arch, sizeof ctx->info.arch, "%s", prop.gcnArchName);
   ctx->info.total_memory_bytes = prop.totalGlobalMem;
   ctx->info.compute_units = prop.multiProcessorCount;
+  ctx->stream_min_groups = prop.multiProcessorCount;
   ctx->info.clock_khz = prop.clockRate;
   ctx->info.memory_clock_khz = prop.memoryClockRate;
   ctx->info.memory_bus_bits = prop.memoryBusWidth;
@@ -217,6 +235,23 @@ extern "C" int tk_set_gemm_min_m(tk_ctx *ctx, int min_m) {
   return TK_OK;
 }
 extern "C" int tk_get_gemm_min_m(const tk_ctx *ctx) { return ctx ? ctx->gemm_min_m : 0; }
+
+extern "C" int tk_set_stream_min_groups(tk_ctx *ctx, int groups) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_stream_min_groups: null context");
+  if (groups < 1) return tk_fail(TK_ERR_INVALID_INPUT, "stream_min_groups=%d - use a positive integer", groups);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->stream_min_groups = groups;
+  return TK_OK;
+}
+extern "C" int tk_get_stream_min_groups(const tk_ctx *ctx) { return ctx ? ctx->stream_min_groups : 0; }
+
+extern "C" int tk_set_decode_kernel(tk_ctx *ctx, int variant) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_decode_kernel: null context");
+  if (variant < 0 || variant > 3) return tk_fail(TK_ERR_INVALID_INPUT, "decode kernel %d - use 0..3", variant);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->decode_force = variant;
+  return TK_OK;
+}
 
 extern "C" int tk_set_exact_max_macs(tk_ctx *ctx, size_t macs) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_exact_max_macs: null context");
@@ -353,10 +388,34 @@ struct Plan {
   TkProblem pr;
   TkPrep prep;
   int prep_kind;
-  bool skinny;
-  TkLaunchCfg cfg;
+  bool skinny;            // a decode kernel (<= 64 operand rows), else the GEMM
+  TkLaunchCfg cfg;        // K-split decode kernel or GEMM
   unsigned grid_m, grid_n;
+  // streaming decode kernel (same rt / planes as cfg)
+  unsigned stream_groups; // workgroups this problem needs
+  size_t stream_lds;
+  int stream_kc;
+  // flow decode kernel: needs every K block of the operand rows in LDS
+  bool flow_ok;
+  size_t flow_lds;
 };
+
+enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3 };
+
+// Consecutive tiles per run of the flow kernel: enough workgroups to give every CU several, few
+// enough that a workgroup's start-up (descriptor, operand staging) is amortised.
+static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt) {
+  const unsigned per_s = 4u * (unsigned)tk_flow_runs_per_wave(planes, rt);
+  unsigned s = total_tiles / (per_s * (unsigned)ctx->info.compute_units * 6u);
+  if (s < 1) s = 1;
+  if (s > 16) s = 16;
+  return (int)s;
+}
+
+static const size_t kLdsStreamBudget = 64 * 1024;
+
+// The streaming kernel wants every CU busy; below that the K-split kernel's finer grain wins.
+static bool prefer_stream(const tk_ctx *ctx, unsigned groups);
 
 // Fills everything of a plan that does not depend on workspace addresses.
 static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_t k, size_t m, int mode,
@@ -391,6 +450,15 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->cfg.rt = rt;
     pl->cfg.lds_bytes = lds_a > lds_r ? lds_a : lds_r;
     pl->cfg.grid = (unsigned)pr.n_tiles;
+    const unsigned tpw = (unsigned)tk_stream_tiles_per_wg(layer->n_planes, rt);
+    pl->stream_groups = ((unsigned)pr.n_tiles + tpw - 1) / tpw;
+    size_t skc = kLdsStreamBudget / (256 * (R ? R : 1));
+    if (skc < 1) skc = 1;
+    if (skc > nb) skc = nb ? nb : 1;
+    pl->stream_kc = (int)skc;
+    pl->stream_lds = skc * 256 * R;
+    pl->flow_lds = nb * 256 * R;
+    pl->flow_ok = pl->flow_lds <= kLdsStreamBudget;
   } else {
     pl->cfg.rt = 8;
     pl->cfg.lds_bytes = 16 * 8 * 16 * 16;
@@ -454,10 +522,33 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else {
     pr.act_scale = act_scale_in;
   }
-  if (pl.skinny)
+  int variant = DECODE_KSPLIT, run_tiles = 1;
+  unsigned flow_groups = 0;
+  if (pl.skinny) {
+    run_tiles = flow_run_tiles(ctx, (unsigned)pr.n_tiles, pl.cfg.planes, pl.cfg.rt);
+    const unsigned per_wg = 4u * (unsigned)tk_flow_runs_per_wave(pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
+    flow_groups = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
+    variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
+  }
+  if (pl.skinny && variant == DECODE_FLOW) {
+    TkLaunchCfg cfg = pl.cfg;
+    cfg.grid = flow_groups;
+    cfg.lds_bytes = pl.flow_lds;
+    pr.run_tiles = run_tiles;
+    pr.group_begin = 0;
+    HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
+  } else if (pl.skinny && variant == DECODE_STREAM) {
+    TkLaunchCfg cfg = pl.cfg;
+    cfg.grid = pl.stream_groups;
+    cfg.lds_bytes = pl.stream_lds;
+    pr.kc = pl.stream_kc;
+    pr.group_begin = 0;
+    HIPCHK(tk_launch_stream(ctx->stream, &pr, nullptr, nullptr, cfg));
+  } else if (pl.skinny) {
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
-  else
+  } else {
     HIPCHK(tk_launch_gemm(ctx->stream, &pr, pl.cfg, pl.grid_m, pl.grid_n));
+  }
   return TK_OK;
 }
 
@@ -626,9 +717,11 @@ extern "C" int tk_mpgemm_with_act_quant(tk_ctx *ctx, const float *act, size_t ac
 struct tk_group {
   tk_ctx *ctx;
   void *ws = nullptr;        // one allocation holding every member's operand rows and side arrays
-  void *tables = nullptr;    // TkProblem[count] then TkPrep[nprep]
+  void *tables = nullptr;    // TkProblem[count], TkPrep[nprep], then int wg_prob[] (streaming form)
   int nprobs = 0, nprep = 0, prep_kind = 0;
   unsigned prep_rows = 0;
+  int variant = 1;
+  size_t wg_prob_off = 0;
   TkLaunchCfg cfg{};
 };
 
@@ -651,9 +744,9 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   std::vector<size_t> prep_off;  // workspace offset of each distinct activation tensor
   size_t ws_bytes = 0;
   auto take = [&](size_t bytes) { size_t o = ws_bytes; ws_bytes += (bytes + 255) & ~(size_t)255; return o; };
-  unsigned tiles = 0, rows = 0;
+  unsigned tiles = 0, rows = 0, sgroups = 0;
   int planes = 0, rt = 1;
-  size_t lds = 0;
+  size_t lds = 0, slds = 0;
   for (size_t i = 0; i < count; ++i) {
     size_t n, k;
     TKCHK(validate_layer(ctx, &members[i].layer, &n, &k));
@@ -695,12 +788,40 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   }
   size_t lds_r = (size_t)4 * planes * rt * 1024;
   if (lds_r > lds) lds = lds_r;
-
+  // streaming / flow forms: every member is re-planned with the group's common rt
+  const unsigned tpw = (unsigned)tk_stream_tiles_per_wg(planes, rt);
+  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt);
+  const unsigned fper = 4u * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)run_tiles;
+  unsigned fgroups = 0;
+  bool flow_ok = true;
+  size_t flds = 0;
+  for (size_t i = 0; i < count; ++i) {
+    sgroups += ((unsigned)plans[i].pr.n_tiles + tpw - 1) / tpw;
+    fgroups += ((unsigned)plans[i].pr.n_tiles + fper - 1) / fper;
+    if (plans[i].stream_lds > slds) slds = plans[i].stream_lds;
+    if (plans[i].flow_lds > flds) flds = plans[i].flow_lds;
+    flow_ok = flow_ok && plans[i].flow_ok;
+  }
+  const int variant = choose_decode(ctx, flow_ok, fgroups, sgroups);
+  std::vector<int> wg_prob;
+  unsigned groups_total = 0;
+  if (variant != DECODE_KSPLIT) {
+    const unsigned per = variant == DECODE_FLOW ? fper : tpw;
+    for (size_t i = 0; i < count; ++i) {
+      const unsigned gi = ((unsigned)plans[i].pr.n_tiles + per - 1) / per;
+      plans[i].pr.group_begin = (int)groups_total;
+      plans[i].pr.run_tiles = run_tiles;
+      if (variant == DECODE_STREAM) plans[i].pr.kc = plans[i].stream_kc;
+      for (unsigned j = 0; j < gi; ++j) wg_prob.push_back((int)i);
+      groups_total += gi;
+    }
+  }
   tk_group *g = new (std::nothrow) tk_group();
   if (!g) return tk_fail(TK_ERR_BACKEND, "tk_group_create: host allocation failed");
   g->ctx = ctx;
   int rc = dev_malloc(ws_bytes, &g->ws);
-  if (!rc) rc = dev_malloc(count * sizeof(TkProblem) + preps.size() * sizeof(TkPrep), &g->tables);
+  const size_t wg_prob_off = count * sizeof(TkProblem) + preps.size() * sizeof(TkPrep);
+  if (!rc) rc = dev_malloc(wg_prob_off + wg_prob.size() * sizeof(int), &g->tables);
   if (rc) {
     if (g->ws) (void)hipFree(g->ws);
     delete g;
@@ -740,20 +861,25 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   if (e == hipSuccess)
     e = hipMemcpy((uint8_t *)g->tables + count * sizeof(TkProblem), preps.data(), preps.size() * sizeof(TkPrep),
                   hipMemcpyHostToDevice);
+  if (e == hipSuccess && !wg_prob.empty())
+    e = hipMemcpy((uint8_t *)g->tables + wg_prob_off, wg_prob.data(), wg_prob.size() * sizeof(int),
+                  hipMemcpyHostToDevice);
   if (e != hipSuccess) {
     (void)hipFree(g->ws);
     (void)hipFree(g->tables);
     delete g;
     return tk_fail(TK_ERR_BACKEND, "tk_group_create: %s", hipGetErrorString(e));
   }
+  g->variant = variant;
+  g->wg_prob_off = wg_prob_off;
   g->nprobs = (int)count;
   g->nprep = (int)preps.size();
   g->prep_kind = prep_kind;
   g->prep_rows = rows;
   g->cfg.planes = planes;
   g->cfg.rt = rt;
-  g->cfg.lds_bytes = lds;
-  g->cfg.grid = tiles;
+  g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
+  g->cfg.grid = variant == DECODE_KSPLIT ? tiles : groups_total;
   *out = g;
   return TK_OK;
 }
@@ -765,7 +891,13 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   const TkProblem *probs = (const TkProblem *)g->tables;
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
   if (do_prep) HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_rows));
-  if (do_main) HIPCHK(tk_launch_skinny(ctx->stream, nullptr, probs, g->nprobs, g->cfg));
+  const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
+  if (do_main && g->variant == DECODE_FLOW)
+    HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, wg_prob, g->cfg));
+  else if (do_main && g->variant == DECODE_STREAM)
+    HIPCHK(tk_launch_stream(ctx->stream, nullptr, probs, wg_prob, g->cfg));
+  else if (do_main)
+    HIPCHK(tk_launch_skinny(ctx->stream, nullptr, probs, g->nprobs, g->cfg));
   return TK_OK;
 }
 

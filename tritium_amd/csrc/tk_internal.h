@@ -40,7 +40,9 @@ struct TkProblem {
   int mode, raw_dtype, out_dtype, planes;
   int tile_begin;            // first launch-wide tile index of this problem
   int n_tiles;               // ceil(n/16)
-  int kc;                    // K blocks staged in LDS per pass (skinny kernel)
+  int kc;                    // K blocks staged in LDS per pass (decode kernels)
+  int group_begin;           // streaming / flow kernels: first workgroup index of this problem
+  int run_tiles;             // flow kernel: consecutive tiles per run (S)
 };
 
 enum { TK_PREP_A8 = 0, TK_PREP_DIGITS = 1, TK_PREP_I8 = 2 };
@@ -81,6 +83,13 @@ hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const T
                           unsigned rows);
 hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
                             const TkLaunchCfg &cfg);
+// streaming decode kernel: tiles per workgroup for a (planes, rt) pair, and the launcher
+int tk_stream_tiles_per_wg(int planes, int rt);
+hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                            const TkLaunchCfg &cfg);
+int tk_flow_runs_per_wave(int planes, int rt);
+hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                          const TkLaunchCfg &cfg);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

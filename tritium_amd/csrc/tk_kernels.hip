@@ -68,16 +68,14 @@ __device__ __forceinline__ int code_at(const uint8_t *codes, int nb, int n, int 
 // The reference's contraction for one (token, output): one f32 accumulator, k in order,
 // add / subtract / skip (crates/tritium-core/src/reference.rs:42-51). With a8 != 0 the activation
 // is first quantized exactly as the host default does (crates/tritium-spec/src/lib.rs:369-374),
-// kept in f32 so NaN survives.
-__device__ float seq_dot(const TkProblem &pr, int p, int n, int tok, int a8) {
-  const uint8_t *codes = pr.codes[p];
-  float s = a8 ? pr.aux[tok] : 0.0f;
-  const bool gamma_zero = a8 && pr.act_scale[tok] == 0.0f;
+// kept in f32 so NaN survives. Takes plain scalars so callers keep their problem in registers.
+__device__ __noinline__ float seq_dot_raw(const uint8_t *codes, int nb, int kdim, const void *raw_act,
+                                          int raw_dtype, int n, int tok, int a8, float s, int gamma_zero) {
   float acc = 0.0f;
-  for (int k = 0; k < pr.k; ++k) {
-    int code = code_at(codes, pr.nb, n, k);
+  for (int k = 0; k < kdim; ++k) {
+    int code = code_at(codes, nb, n, k);
     if (code == 1) continue;
-    float a = load_act(pr.raw_act, pr.raw_dtype, (size_t)tok * pr.k + k);
+    float a = load_act(raw_act, raw_dtype, (size_t)tok * kdim + k);
     if (a8) {
       if (gamma_zero) {
         a = 0.0f;
@@ -89,6 +87,12 @@ __device__ float seq_dot(const TkProblem &pr, int p, int n, int tok, int a8) {
     acc = (code == 2) ? __fadd_rn(acc, a) : __fsub_rn(acc, a);
   }
   return acc;
+}
+
+__device__ __forceinline__ float seq_dot(const TkProblem &pr, int p, int n, int tok, int a8) {
+  const float s = a8 ? pr.aux[tok] : 0.0f;
+  const int gamma_zero = a8 && pr.act_scale[tok] == 0.0f;
+  return seq_dot_raw(pr.codes[p], pr.nb, pr.k, pr.raw_act, pr.raw_dtype, n, tok, a8, s, gamma_zero);
 }
 
 // Fold one plane's accumulators of one lane (4 consecutive operand rows starting at rowbase,
@@ -256,6 +260,344 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
       }
     }
     if (n < pr.n && pr.out_dtype != TK_I32) finish_lane(pr, n, rowbase, out);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// decode GEMV, streaming form: used when a launch holds enough output tiles to fill the chip
+// (grouped launches, wide layers). A workgroup owns 4*TW consecutive 16-row tiles; each wave owns
+// TW of them outright, so there is no cross-wave reduction, and every wave walks contiguous
+// 1 KiB chunks of its tiles with the next K block's chunks already in flight. The activation
+// operand rows stay resident in LDS for all tiles of the workgroup.
+// ------------------------------------------------------------------------------------------
+
+template <int P, int RT, int TW>
+__global__ __launch_bounds__(TK_WG) void tk_stream_kernel(TkProblem single, const TkProblem *__restrict__ table,
+                                                          const int *__restrict__ wg_prob) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const TkProblem *prp = &single;
+  if (table) prp = &table[wg_prob[blockIdx.x]];
+  const TkProblem &pr = *prp;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int i = lane & 15, g = lane >> 4;
+  const int nb = pr.nb, R = pr.R, kc = pr.kc;
+  const int tile0 = ((blockIdx.x - pr.group_begin) * 4 + wave) * TW;
+
+  const uint8_t *wp[TW][P];
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw) {
+    // tiles past the end re-read the last tile (results discarded) so every load stays in bounds
+    const int t = min(tile0 + tw, pr.n_tiles - 1);
+#pragma unroll
+    for (int p = 0; p < P; ++p) wp[tw][p] = pr.codes[p] + ((size_t)t * nb * 64 + lane) * 16;
+  }
+
+  v4i acc[TW][P][RT];
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) acc[tw][p][rt] = v4i{0, 0, 0, 0};
+
+  const uint4 *ap4 = (const uint4 *)pr.ap;
+  uint4 *lds4 = (uint4 *)smem;
+  uint4 wc[TW][P], wn[TW][P];
+
+  if (nb > 0) {
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int p = 0; p < P; ++p) wc[tw][p] = *(const uint4 *)(wp[tw][p]);
+  }
+
+  for (int kb0 = 0; kb0 < nb; kb0 += kc) {
+    const int kcn = min(kc, nb - kb0);
+    __syncthreads();
+    const int cnt = kcn * 16 * R;
+    const uint4 *src = ap4 + (size_t)kb0 * 16 * R;
+    for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4[idx] = src[idx];
+    __syncthreads();
+
+    for (int kbl = 0; kbl < kcn; ++kbl) {
+      const int kb = kb0 + kbl;
+      if (kb + 1 < nb) {
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+          for (int p = 0; p < P; ++p) wn[tw][p] = *(const uint4 *)(wp[tw][p] + (size_t)(kb + 1) * TK_CHUNK_BYTES);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v4i a[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const int row = rt * 16 + i;
+          uint4 q = make_uint4(0, 0, 0, 0);
+          if (row < R) q = lds4[((kbl * 4 + j) * 4 + g) * R + row];
+          a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+        }
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+          for (int p = 0; p < P; ++p) {
+            const uint4 w = wc[tw][p];
+            const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
+            const v4i b = expand_codes(wj);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              acc[tw][p][rt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[tw][p][rt], 0, 0, 0);
+          }
+      }
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+        for (int p = 0; p < P; ++p) wc[tw][p] = wn[tw][p];
+    }
+  }
+
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw) {
+    const int t = tile0 + tw;
+    const int n = t * 16 + i;
+    if (t >= pr.n_tiles || n >= pr.n) continue;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int rowbase = rt * 16 + 4 * g;
+      if (pr.out_dtype == TK_I32) {
+        store_raw(pr, n, rowbase, acc[tw][0][rt]);
+      } else {
+        float out[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < P; ++p) fold_plane(pr, p, n, rowbase, acc[tw][p][rt], out, p == 0);
+        finish_lane(pr, n, rowbase, out);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// decode GEMV, flow form: the bandwidth kernel. Requirements: all K blocks of the operand rows fit
+// in LDS. A wave owns TW runs of S consecutive output tiles; in the device layout the chunks of
+// consecutive tiles are consecutive in memory, so each run is ONE contiguous byte stream of
+// S*nb KiB, walked with a D-deep ring of 128-bit loads that never drains at tile boundaries.
+// Per-row constants are loaded once per wave, per-tile scales at the start of the tile, so the
+// epilogue of a tile waits on nothing that was issued behind the stream's prefetches.
+// ------------------------------------------------------------------------------------------
+
+struct RowConst {
+  int rs[4];       // row sums of the 4 operand rows this lane finishes
+  float as[4];     // INT8: per-token activation scale (1.0 when absent)
+  int exp;         // DIGITS: grid exponent of the token
+  unsigned flag;   // any of the rows takes the exact fallback
+};
+
+__device__ __forceinline__ RowConst load_row_const(const TkProblem &pr, int rowbase) {
+  RowConst rc;
+  rc.exp = 0;
+  rc.flag = 0;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = rowbase + r;
+    rc.rs[r] = m < pr.R ? pr.rowsum[m] : 0;
+    rc.as[r] = 1.0f;
+  }
+  if (pr.mode == TK_MODE_INT8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = rowbase + r;
+      if (m < pr.R) {
+        if (pr.act_scale) rc.as[r] = pr.act_scale[m];
+        if (pr.flags && pr.flags[m]) rc.flag |= 1u << r;
+      }
+    }
+  } else {
+    const int tok = rowbase >> 2;
+    if (tok < pr.M) {
+      rc.exp = pr.exps[tok];
+      if (pr.flags && pr.flags[tok]) rc.flag = 1u;
+    }
+  }
+  return rc;
+}
+
+// Finish one lane's 4 accumulator registers for every plane, with preloaded constants.
+template <int P>
+__device__ __forceinline__ void flow_epilogue(const TkProblem &pr, int n, int rowbase, const v4i (&acc)[P],
+                                              const float (&sc)[P], const RowConst &rc) {
+  if (pr.out_dtype == TK_I32) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = rowbase + r;
+      if (m < pr.R) ((int32_t *)pr.out)[(size_t)m * pr.n + n] = acc[0][r] - rc.rs[r];
+    }
+    return;
+  }
+  if (pr.mode == TK_MODE_INT8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = rowbase + r;
+      if (m >= pr.R) continue;
+      float f = 0.0f;
+      if (rc.flag & (1u << r)) {
+        for (int p = 0; p < P; ++p) {
+          float t = __fmul_rn(seq_dot(pr, p, n, m, 1), sc[p]);
+          f = p == 0 ? t : __fadd_rn(f, t);
+        }
+      } else {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          float t = __fmul_rn((float)(acc[p][r] - rc.rs[r]), sc[p]);
+          f = p == 0 ? t : __fadd_rn(f, t);
+        }
+      }
+      if (pr.act_scale) f = __fmul_rn(f, rc.as[r]);
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
+    }
+  } else {
+    const int tok = rowbase >> 2;
+    if (tok >= pr.M) return;
+    float f = 0.0f;
+    if (rc.flag) {
+      for (int p = 0; p < P; ++p) {
+        float t = __fmul_rn(seq_dot(pr, p, n, tok, 0), sc[p]);
+        f = p == 0 ? t : __fadd_rn(f, t);
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        long long V = 0;
+#pragma unroll
+        for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(acc[p][r] - rc.rs[r]);
+        float t = __fmul_rn((float)ldexp((double)V, rc.exp), sc[p]);
+        f = p == 0 ? t : __fadd_rn(f, t);
+      }
+    }
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
+  }
+}
+
+template <int P, int RT, int TW, int D, bool TABLE>
+__global__ __launch_bounds__(TK_WG) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+                                                        const int *__restrict__ wg_prob) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int i = lane & 15, g = lane >> 4;
+  const int nb = pr.nb, R = pr.R, S = pr.run_tiles;
+  const int nbpad = (nb + D - 1) / D * D;
+  const int first = ((blockIdx.x - pr.group_begin) * 4 + wave) * TW * S;  // first tile of this wave
+  const unsigned last_chunk = (unsigned)pr.n_tiles * (unsigned)nb - 1u;   // clamp: stay inside the plane
+
+  // the stream position is a chunk index inside the plane; lane offset is added at the load
+  unsigned cbase[TW];
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw) cbase[tw] = (unsigned)(first + tw * S) * (unsigned)nb;
+
+  auto load_chunk = [&](int tw, int p, int s, int kb) -> uint4 {
+    unsigned c = cbase[tw] + (unsigned)s * (unsigned)nb + (unsigned)kb;
+    c = c < last_chunk ? c : last_chunk;
+    return *(const uint4 *)(pr.codes[p] + ((size_t)c * 64 + lane) * 16);
+  };
+
+  uint4 ring[D][TW][P];
+  if (nb > 0) {
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+      if (d < nb) {
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+          for (int p = 0; p < P; ++p) ring[d][tw][p] = load_chunk(tw, p, 0, d);
+      }
+  }
+
+  // stage every operand row of the problem in LDS
+  {
+    const uint4 *ap4 = (const uint4 *)pr.ap;
+    uint4 *lds4w = (uint4 *)smem;
+    const int cnt = nb * 16 * R;
+    for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4w[idx] = ap4[idx];
+  }
+  RowConst rc[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) rc[rt] = load_row_const(pr, rt * 16 + 4 * g);
+  __syncthreads();
+  const uint4 *lds4 = (const uint4 *)smem;
+
+  for (int s = 0; s < S; ++s) {
+    // per-tile scales, issued now, consumed in the epilogue
+    float sc[TW][P];
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+      const int n = min((first + tw * S + s) * 16 + i, pr.n - 1);
+#pragma unroll
+      for (int p = 0; p < P; ++p) sc[tw][p] = pr.scales[p][n];
+    }
+    v4i acc[TW][RT][P];
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int p = 0; p < P; ++p) acc[tw][rt][p] = v4i{0, 0, 0, 0};
+
+    for (int kbg = 0; kbg < nbpad; kbg += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int kb = kbg + d;
+        if (kb < nb) {
+          uint4 cur[TW][P];
+#pragma unroll
+          for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+            for (int p = 0; p < P; ++p) cur[tw][p] = ring[d][tw][p];
+          // refill this ring slot with the chunk D positions ahead in the padded stream
+          {
+            int kb2 = kb + D, s2 = s;
+            if (kb2 >= nbpad) { kb2 -= nbpad; s2 += 1; }
+            if (kb2 < nb && s2 < S) {
+#pragma unroll
+              for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+                for (int p = 0; p < P; ++p) ring[d][tw][p] = load_chunk(tw, p, s2, kb2);
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v4i a[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+              const int row = rt * 16 + i;
+              uint4 q = make_uint4(0, 0, 0, 0);
+              if (row < R) q = lds4[((kb * 4 + j) * 4 + g) * R + row];
+              a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+            }
+#pragma unroll
+            for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+              for (int p = 0; p < P; ++p) {
+                const uint4 w = cur[tw][p];
+                const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
+                const v4i b = expand_codes(wj);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                  acc[tw][rt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[tw][rt][p], 0, 0, 0);
+              }
+          }
+        }
+      }
+    }
+
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+      const int t = first + tw * S + s;
+      const int n = t * 16 + i;
+      if (t < pr.n_tiles && n < pr.n) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) flow_epilogue<P>(pr, n, rt * 16 + 4 * g, acc[tw][rt], sc[tw], rc[rt]);
+      }
+    }
   }
 }
 
@@ -674,6 +1016,86 @@ hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProb
     case 2: return launch_skinny_p<2>(s, single, table, nprobs, cfg);
     case 3: return launch_skinny_p<3>(s, single, table, nprobs, cfg);
     case 4: return launch_skinny_p<4>(s, single, table, nprobs, cfg);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <int P, int RT>
+static hipError_t launch_stream_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
+                                   const TkLaunchCfg &cfg) {
+  constexpr int TW = (P * RT <= 4) ? 4 : ((P * RT <= 8) ? 2 : 1);
+  hipLaunchKernelGGL((tk_stream_kernel<P, RT, TW>), dim3(cfg.grid), dim3(TK_WG), cfg.lds_bytes, s, sg, table, wg_prob);
+  return hipGetLastError();
+}
+
+template <int P>
+static hipError_t launch_stream_p(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
+                                  const TkLaunchCfg &cfg) {
+  switch (cfg.rt) {
+    case 1: return launch_stream_pr<P, 1>(s, sg, table, wg_prob, cfg);
+    case 2: return launch_stream_pr<P, 2>(s, sg, table, wg_prob, cfg);
+    case 4: return launch_stream_pr<P, 4>(s, sg, table, wg_prob, cfg);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+int tk_stream_tiles_per_wg(int planes, int rt) {
+  const int pr = planes * rt;
+  return 4 * (pr <= 4 ? 4 : (pr <= 8 ? 2 : 1));
+}
+
+hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                            const TkLaunchCfg &cfg) {
+  if (!cfg.grid) return hipSuccess;
+  TkProblem dummy = {};
+  const TkProblem &sg = single ? *single : dummy;
+  switch (cfg.planes) {
+    case 1: return launch_stream_p<1>(s, sg, table, wg_prob, cfg);
+    case 2: return launch_stream_p<2>(s, sg, table, wg_prob, cfg);
+    case 3: return launch_stream_p<3>(s, sg, table, wg_prob, cfg);
+    case 4: return launch_stream_p<4>(s, sg, table, wg_prob, cfg);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <int P, int RT>
+static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
+                                 const TkLaunchCfg &cfg) {
+  constexpr int TW = (RT >= 4 && P <= 2) ? 2 : 1;
+  constexpr int D = (P * TW >= 4) ? 2 : 4;
+  if (table)
+    hipLaunchKernelGGL((tk_flow_kernel<P, RT, TW, D, true>), dim3(cfg.grid), dim3(TK_WG), cfg.lds_bytes, s, sg, table,
+                       wg_prob);
+  else
+    hipLaunchKernelGGL((tk_flow_kernel<P, RT, TW, D, false>), dim3(cfg.grid), dim3(TK_WG), cfg.lds_bytes, s, sg, table,
+                       wg_prob);
+  return hipGetLastError();
+}
+
+template <int P>
+static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
+                                const TkLaunchCfg &cfg) {
+  switch (cfg.rt) {
+    case 1: return launch_flow_pr<P, 1>(s, sg, table, wg_prob, cfg);
+    case 2: return launch_flow_pr<P, 2>(s, sg, table, wg_prob, cfg);
+    case 4: return launch_flow_pr<P, 4>(s, sg, table, wg_prob, cfg);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// lock-step runs per wave of the flow kernel for a (planes, rt) pair
+int tk_flow_runs_per_wave(int planes, int rt) { return (rt >= 4 && planes <= 2) ? 2 : 1; }
+
+hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                          const TkLaunchCfg &cfg) {
+  if (!cfg.grid) return hipSuccess;
+  TkProblem dummy = {};
+  const TkProblem &sg = single ? *single : dummy;
+  switch (cfg.planes) {
+    case 1: return launch_flow_p<1>(s, sg, table, wg_prob, cfg);
+    case 2: return launch_flow_p<2>(s, sg, table, wg_prob, cfg);
+    case 3: return launch_flow_p<3>(s, sg, table, wg_prob, cfg);
+    case 4: return launch_flow_p<4>(s, sg, table, wg_prob, cfg);
     default: return hipErrorInvalidValue;
   }
 }
