@@ -404,8 +404,11 @@ enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3 };
 
 // Consecutive tiles per run of the flow kernel: enough workgroups to give every CU several, few
 // enough that a workgroup's start-up (descriptor, operand staging) is amortised.
-static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt) {
-  const unsigned per_s = 4u * (unsigned)tk_flow_runs_per_wave(planes, rt);
+static const size_t kLdsFlowMax = 160 * 1024;
+static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
+
+static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves) {
+  const unsigned per_s = (unsigned)waves * (unsigned)tk_flow_runs_per_wave(planes, rt);
   unsigned s = total_tiles / (per_s * (unsigned)ctx->info.compute_units * 6u);
   if (s < 1) s = 1;
   if (s > 16) s = 16;
@@ -458,7 +461,7 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->stream_kc = (int)skc;
     pl->stream_lds = skc * 256 * R;
     pl->flow_lds = nb * 256 * R;
-    pl->flow_ok = pl->flow_lds <= kLdsStreamBudget;
+    pl->flow_ok = pl->flow_lds <= kLdsFlowMax;
   } else {
     pl->cfg.rt = 8;
     pl->cfg.lds_bytes = 16 * 8 * 16 * 16;
@@ -525,8 +528,9 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   int variant = DECODE_KSPLIT, run_tiles = 1;
   unsigned flow_groups = 0;
   if (pl.skinny) {
-    run_tiles = flow_run_tiles(ctx, (unsigned)pr.n_tiles, pl.cfg.planes, pl.cfg.rt);
-    const unsigned per_wg = 4u * (unsigned)tk_flow_runs_per_wave(pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
+    const int fw = flow_waves(pl.flow_lds);
+    run_tiles = flow_run_tiles(ctx, (unsigned)pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw);
+    const unsigned per_wg = (unsigned)fw * (unsigned)tk_flow_runs_per_wave(pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
     variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
   }
@@ -534,6 +538,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = flow_groups;
     cfg.lds_bytes = pl.flow_lds;
+    cfg.waves = flow_waves(pl.flow_lds);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -790,17 +795,20 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   if (lds_r > lds) lds = lds_r;
   // streaming / flow forms: every member is re-planned with the group's common rt
   const unsigned tpw = (unsigned)tk_stream_tiles_per_wg(planes, rt);
-  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt);
-  const unsigned fper = 4u * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)run_tiles;
-  unsigned fgroups = 0;
-  bool flow_ok = true;
   size_t flds = 0;
+  bool flow_ok = true;
+  for (size_t i = 0; i < count; ++i) {
+    if (plans[i].flow_lds > flds) flds = plans[i].flow_lds;
+    flow_ok = flow_ok && plans[i].flow_ok;
+  }
+  const int fw = flow_waves(flds);
+  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw);
+  const unsigned fper = (unsigned)fw * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)run_tiles;
+  unsigned fgroups = 0;
   for (size_t i = 0; i < count; ++i) {
     sgroups += ((unsigned)plans[i].pr.n_tiles + tpw - 1) / tpw;
     fgroups += ((unsigned)plans[i].pr.n_tiles + fper - 1) / fper;
     if (plans[i].stream_lds > slds) slds = plans[i].stream_lds;
-    if (plans[i].flow_lds > flds) flds = plans[i].flow_lds;
-    flow_ok = flow_ok && plans[i].flow_ok;
   }
   const int variant = choose_decode(ctx, flow_ok, fgroups, sgroups);
   std::vector<int> wg_prob;
@@ -880,6 +888,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   g->cfg.rt = rt;
   g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
   g->cfg.grid = variant == DECODE_KSPLIT ? tiles : groups_total;
+  g->cfg.waves = fw;
   *out = g;
   return TK_OK;
 }

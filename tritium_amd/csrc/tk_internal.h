@@ -68,6 +68,7 @@ struct TkLaunchCfg {
   int rt;       // row tiles per workgroup (skinny: 1,2,4 ; gemm: 8)
   size_t lds_bytes;
   unsigned grid;
+  int waves;    // flow kernel: waves per workgroup (4, or 8 when the operand rows need > 64 KiB of LDS)
 };
 
 #ifdef __cplusplus

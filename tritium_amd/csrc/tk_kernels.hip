@@ -477,8 +477,8 @@ __device__ __forceinline__ void flow_epilogue(const TkProblem &pr, int n, int ro
   }
 }
 
-template <int P, int RT, int TW, int D, bool TABLE>
-__global__ __launch_bounds__(TK_WG) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+template <int P, int RT, int TW, int D, int NW, bool TABLE>
+__global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                         const int *__restrict__ wg_prob) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
@@ -486,7 +486,7 @@ __global__ __launch_bounds__(TK_WG) void tk_flow_kernel(const TkProblem single, 
   const int i = lane & 15, g = lane >> 4;
   const int nb = pr.nb, R = pr.R, S = pr.run_tiles;
   const int nbpad = (nb + D - 1) / D * D;
-  const int first = ((blockIdx.x - pr.group_begin) * 4 + wave) * TW * S;  // first tile of this wave
+  const int first = ((blockIdx.x - pr.group_begin) * NW + wave) * TW * S;  // first tile of this wave
   const unsigned last_chunk = (unsigned)pr.n_tiles * (unsigned)nb - 1u;   // clamp: stay inside the plane
 
   // the stream position is a chunk index inside the plane; lane offset is added at the load
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(TK_WG) void tk_flow_kernel(const TkProblem single, 
     const uint4 *ap4 = (const uint4 *)pr.ap;
     uint4 *lds4w = (uint4 *)smem;
     const int cnt = nb * 16 * R;
-    for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4w[idx] = ap4[idx];
+    for (int idx = threadIdx.x; idx < cnt; idx += NW * 64) lds4w[idx] = ap4[idx];
   }
   RowConst rc[RT];
 #pragma unroll
@@ -1058,18 +1058,36 @@ hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProb
   }
 }
 
+template <typename K>
+static hipError_t flow_launch_one(K kernel, hipStream_t s, const TkProblem &sg, const TkProblem *table,
+                                  const int *wg_prob, const TkLaunchCfg &cfg, int threads) {
+  if (cfg.lds_bytes > 64 * 1024) {
+    // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+    static thread_local const void *raised[64];
+    static thread_local int nraised = 0;
+    bool done = false;
+    for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
+    if (!done) {
+      hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      if (nraised < 64) raised[nraised++] = (const void *)kernel;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(cfg.grid), dim3(threads), cfg.lds_bytes, s, sg, table, wg_prob);
+  return hipGetLastError();
+}
+
 template <int P, int RT>
 static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                  const TkLaunchCfg &cfg) {
   constexpr int TW = (RT >= 4 && P <= 2) ? 2 : 1;
   constexpr int D = (P * TW >= 4) ? 2 : 4;
-  if (table)
-    hipLaunchKernelGGL((tk_flow_kernel<P, RT, TW, D, true>), dim3(cfg.grid), dim3(TK_WG), cfg.lds_bytes, s, sg, table,
-                       wg_prob);
-  else
-    hipLaunchKernelGGL((tk_flow_kernel<P, RT, TW, D, false>), dim3(cfg.grid), dim3(TK_WG), cfg.lds_bytes, s, sg, table,
-                       wg_prob);
-  return hipGetLastError();
+  if (cfg.waves == 8) {
+    if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 8, true>, s, sg, table, wg_prob, cfg, 512);
+    return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 8, false>, s, sg, table, wg_prob, cfg, 512);
+  }
+  if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 4, true>, s, sg, table, wg_prob, cfg, 256);
+  return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 4, false>, s, sg, table, wg_prob, cfg, 256);
 }
 
 template <int P>
