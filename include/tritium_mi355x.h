@@ -193,6 +193,9 @@ int tk_get_gemm_min_m(const tk_ctx *ctx);
  * through LDS), 3 flow (all of K resident in LDS; falls back to 2 when it does not fit). All give
  * identical bits; the knob exists for tests and tuning. */
 int tk_set_decode_kernel(tk_ctx *ctx, int variant);
+/* Consecutive output tiles a wave of the flow kernel walks as one stream; 0 = chosen from the size
+ * of the launch. A tuning knob: results do not depend on it. */
+int tk_set_flow_run_tiles(tk_ctx *ctx, int tiles);
 int tk_set_stream_min_groups(tk_ctx *ctx, int groups);
 int tk_get_stream_min_groups(const tk_ctx *ctx);
 

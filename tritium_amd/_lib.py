@@ -6,7 +6,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libtritium_mi355x.so")
+LIB_PATH = os.environ.get("TRITIUM_MI355X_LIB") or os.path.join(HERE, "libtritium_mi355x.so")
 
 TK_OK, TK_ERR_SHAPE_MISMATCH, TK_ERR_UNSUPPORTED_FORMAT, TK_ERR_OUT_OF_MEMORY, TK_ERR_INVALID_INPUT, TK_ERR_BACKEND = range(6)
 TK_F32, TK_BF16, TK_I8, TK_I32 = range(4)
@@ -64,6 +64,7 @@ SIGNATURES = {
     "tk_set_gemm_min_m": (C.c_int, [vp, C.c_int]),
     "tk_get_gemm_min_m": (C.c_int, [vp]),
     "tk_set_decode_kernel": (C.c_int, [vp, C.c_int]),
+    "tk_set_flow_run_tiles": (C.c_int, [vp, C.c_int]),
     "tk_set_stream_min_groups": (C.c_int, [vp, C.c_int]),
     "tk_get_stream_min_groups": (C.c_int, [vp]),
     "tk_set_exact_max_macs": (C.c_int, [vp, sz]),

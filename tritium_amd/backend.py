@@ -387,6 +387,9 @@ class Mi355xBackend:
         """0 automatic, 1 K-split, 2 streaming, 3 flow."""
         _check(self._lib.tk_set_decode_kernel(self._ctx, variant))
 
+    def set_flow_run_tiles(self, tiles):
+        _check(self._lib.tk_set_flow_run_tiles(self._ctx, tiles))
+
     def set_stream_min_groups(self, groups):
         _check(self._lib.tk_set_stream_min_groups(self._ctx, groups))
 

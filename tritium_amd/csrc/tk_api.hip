@@ -72,6 +72,7 @@ struct tk_ctx {
   size_t exact_max_macs = (size_t)1 << 20;
   int stream_min_groups = 0;  // set at init to the CU count
   int decode_force = 0;  // DECODE_AUTO
+  int flow_run_tiles = 0;  // 0 = automatic
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
   int *d_invalid = nullptr;
 };
@@ -245,6 +246,14 @@ extern "C" int tk_set_stream_min_groups(tk_ctx *ctx, int groups) {
 }
 extern "C" int tk_get_stream_min_groups(const tk_ctx *ctx) { return ctx ? ctx->stream_min_groups : 0; }
 
+extern "C" int tk_set_flow_run_tiles(tk_ctx *ctx, int tiles) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_run_tiles: null context");
+  if (tiles < 0 || tiles > 1024) return tk_fail(TK_ERR_INVALID_INPUT, "flow_run_tiles=%d - use 0 (automatic) .. 1024", tiles);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->flow_run_tiles = tiles;
+  return TK_OK;
+}
+
 extern "C" int tk_set_decode_kernel(tk_ctx *ctx, int variant) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_decode_kernel: null context");
   if (variant < 0 || variant > 3) return tk_fail(TK_ERR_INVALID_INPUT, "decode kernel %d - use 0..3", variant);
@@ -402,16 +411,25 @@ struct Plan {
 
 enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3 };
 
-// Consecutive tiles per run of the flow kernel: enough workgroups to give every CU several, few
-// enough that a workgroup's start-up (descriptor, operand staging) is amortised.
 static const size_t kLdsFlowMax = 160 * 1024;
 static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
 
-static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves) {
-  const unsigned per_s = (unsigned)waves * (unsigned)tk_flow_runs_per_wave(planes, rt);
-  unsigned s = total_tiles / (per_s * (unsigned)ctx->info.compute_units * 6u);
-  if (s < 1) s = 1;
-  if (s > 16) s = 16;
+// Consecutive tiles per run of the flow kernel. A workgroup pays for staging its operand rows
+// (lds_bytes) once, so it should stream several times that in weights; beyond that, shorter runs
+// win (more, shorter-lived workgroups keep more loads in flight and balance the tail). Measured on
+// K=2048 N=8192 x 2 planes over 128 layer copies: 4-16 operand rows peak at 2 tiles per run
+// (128 KiB of weights per workgroup), 32 and 64 rows at 8 (8x the staged bytes).
+static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
+                          size_t nb) {
+  if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
+  const size_t per_s = (size_t)waves * (size_t)tk_flow_runs_per_wave(planes, rt);
+  const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
+  size_t target = 8 * lds_bytes * (size_t)(waves / 4);
+  if (target < 128 * 1024) target = 128 * 1024;
+  size_t s = 1;
+  while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
+  // keep at least two workgroups per CU
+  while (s > 1 && total_tiles / (per_s * s) < 2u * (unsigned)ctx->info.compute_units) --s;
   return (int)s;
 }
 
@@ -529,7 +547,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   unsigned flow_groups = 0;
   if (pl.skinny) {
     const int fw = flow_waves(pl.flow_lds);
-    run_tiles = flow_run_tiles(ctx, (unsigned)pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw);
+    run_tiles = flow_run_tiles(ctx, (unsigned)pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, pl.flow_lds, pr.nb);
     const unsigned per_wg = (unsigned)fw * (unsigned)tk_flow_runs_per_wave(pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
     variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
@@ -802,7 +820,10 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     flow_ok = flow_ok && plans[i].flow_ok;
   }
   const int fw = flow_waves(flds);
-  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw);
+  size_t nb_max = 1;
+  for (size_t i = 0; i < count; ++i)
+    if ((size_t)plans[i].pr.nb > nb_max) nb_max = plans[i].pr.nb;
+  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max);
   const unsigned fper = (unsigned)fw * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)run_tiles;
   unsigned fgroups = 0;
   for (size_t i = 0; i < count; ++i) {

@@ -21,6 +21,13 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 #define TK_WG 256
+// prefetch ring depth of the flow kernel, in K blocks: narrow (planes*runs < 4) and wide streams
+#ifndef TK_FLOW_DEPTH
+#define TK_FLOW_DEPTH 4
+#endif
+#ifndef TK_FLOW_DEPTH_WIDE
+#define TK_FLOW_DEPTH_WIDE 2
+#endif
 
 // ------------------------------------------------------------------------------------------
 // small helpers
@@ -1081,7 +1088,7 @@ template <int P, int RT>
 static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                  const TkLaunchCfg &cfg) {
   constexpr int TW = (RT >= 4 && P <= 2) ? 2 : 1;
-  constexpr int D = (P * TW >= 4) ? 2 : 4;
+  constexpr int D = (P * TW >= 4) ? TK_FLOW_DEPTH_WIDE : TK_FLOW_DEPTH;
   if (cfg.waves == 8) {
     if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 8, true>, s, sg, table, wg_prob, cfg, 512);
     return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 8, false>, s, sg, table, wg_prob, cfg, 512);
