@@ -481,10 +481,11 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->flow_lds = nb * 256 * R;
     pl->flow_ok = pl->flow_lds <= kLdsFlowMax;
   } else {
-    pl->cfg.rt = 8;
-    pl->cfg.lds_bytes = 16 * 8 * 16 * 16;
-    pl->grid_m = (unsigned)((R + 127) / 128);
-    pl->grid_n = (unsigned)((pr.n_tiles + 7) / 8);
+    pl->cfg.rt = 4;
+    pl->cfg.lds_bytes = 2 * 16 * 64 * 16;  // two 64-row blocks of 256 k
+    pl->grid_m = (unsigned)((R + 63) / 64);
+    const unsigned per_wg = 4u * (unsigned)tk_gemm_tiles_per_wave(layer->n_planes);
+    pl->grid_n = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
   }
 }
 

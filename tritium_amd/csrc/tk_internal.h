@@ -91,6 +91,7 @@ hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProb
 int tk_flow_runs_per_wave(int planes, int rt);
 hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
+int tk_gemm_tiles_per_wave(int planes);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

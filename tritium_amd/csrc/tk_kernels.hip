@@ -399,6 +399,20 @@ struct RowConst {
   unsigned flag;   // any of the rows takes the exact fallback
 };
 
+// fallback flags of the 4 operand rows starting at rowbase (bit r = row r; DIGITS: bit 0 = the token)
+__device__ __forceinline__ unsigned row_flags(const TkProblem &pr, int rowbase) {
+  unsigned fl = 0;
+  if (!pr.flags) return 0;
+  if (pr.mode == TK_MODE_INT8) {
+    for (int r = 0; r < 4; ++r)
+      if (rowbase + r < pr.R && pr.flags[rowbase + r]) fl |= 1u << r;
+  } else {
+    const int tok = rowbase >> 2;
+    if (tok < pr.M && pr.flags[tok]) fl = 1u;
+  }
+  return fl;
+}
+
 __device__ __forceinline__ RowConst load_row_const(const TkProblem &pr, int rowbase) {
   RowConst rc;
   rc.exp = 0;
@@ -428,7 +442,8 @@ __device__ __forceinline__ RowConst load_row_const(const TkProblem &pr, int rowb
   return rc;
 }
 
-// Finish one lane's 4 accumulator registers for every plane, with preloaded constants.
+// Finish one lane's 4 accumulator registers for every plane, with preloaded constants. Rows that
+// take the exact fallback are left alone here: exact_rows() writes them afterwards.
 template <int P>
 __device__ __forceinline__ void flow_epilogue(const TkProblem &pr, int n, int rowbase, const v4i (&acc)[P],
                                               const float (&sc)[P], const RowConst &rc) {
@@ -444,41 +459,54 @@ __device__ __forceinline__ void flow_epilogue(const TkProblem &pr, int n, int ro
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = rowbase + r;
-      if (m >= pr.R) continue;
+      if (m >= pr.R || (rc.flag & (1u << r))) continue;
       float f = 0.0f;
-      if (rc.flag & (1u << r)) {
-        for (int p = 0; p < P; ++p) {
-          float t = __fmul_rn(seq_dot(pr, p, n, m, 1), sc[p]);
-          f = p == 0 ? t : __fadd_rn(f, t);
-        }
-      } else {
 #pragma unroll
-        for (int p = 0; p < P; ++p) {
-          float t = __fmul_rn((float)(acc[p][r] - rc.rs[r]), sc[p]);
-          f = p == 0 ? t : __fadd_rn(f, t);
-        }
+      for (int p = 0; p < P; ++p) {
+        float t = __fmul_rn((float)(acc[p][r] - rc.rs[r]), sc[p]);
+        f = p == 0 ? t : __fadd_rn(f, t);
       }
       if (pr.act_scale) f = __fmul_rn(f, rc.as[r]);
       store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
     }
   } else {
     const int tok = rowbase >> 2;
-    if (tok >= pr.M) return;
+    if (tok >= pr.M || rc.flag) return;
     float f = 0.0f;
-    if (rc.flag) {
-      for (int p = 0; p < P; ++p) {
-        float t = __fmul_rn(seq_dot(pr, p, n, tok, 0), sc[p]);
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      long long V = 0;
+#pragma unroll
+      for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(acc[p][r] - rc.rs[r]);
+      float t = __fmul_rn((float)ldexp((double)V, rc.exp), sc[p]);
+      f = p == 0 ? t : __fadd_rn(f, t);
+    }
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
+  }
+}
+
+// The rows of one lane that hold NaN/Inf: recomputed in the reference's order (needs no accumulator).
+__device__ __forceinline__ void exact_rows(const TkProblem &pr, int n, int rowbase, unsigned flag) {
+  if (pr.out_dtype == TK_I32) return;
+  if (pr.mode == TK_MODE_INT8) {
+    for (int r = 0; r < 4; ++r) {
+      const int m = rowbase + r;
+      if (m >= pr.R || !(flag & (1u << r))) continue;
+      float f = 0.0f;
+      for (int p = 0; p < pr.planes; ++p) {
+        float t = __fmul_rn(seq_dot(pr, p, n, m, 1), pr.scales[p][n]);
         f = p == 0 ? t : __fadd_rn(f, t);
       }
-    } else {
-#pragma unroll
-      for (int p = 0; p < P; ++p) {
-        long long V = 0;
-#pragma unroll
-        for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(acc[p][r] - rc.rs[r]);
-        float t = __fmul_rn((float)ldexp((double)V, rc.exp), sc[p]);
-        f = p == 0 ? t : __fadd_rn(f, t);
-      }
+      if (pr.act_scale) f = __fmul_rn(f, pr.act_scale[m]);
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
+    }
+  } else {
+    const int tok = rowbase >> 2;
+    if (tok >= pr.M || !flag) return;
+    float f = 0.0f;
+    for (int p = 0; p < pr.planes; ++p) {
+      float t = __fmul_rn(seq_dot(pr, p, n, tok, 0), pr.scales[p][n]);
+      f = p == 0 ? t : __fadd_rn(f, t);
     }
     store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
   }
@@ -527,8 +555,12 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
     for (int idx = threadIdx.x; idx < cnt; idx += NW * 64) lds4w[idx] = ap4[idx];
   }
   RowConst rc[RT];
+  unsigned any_flag = 0;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) rc[rt] = load_row_const(pr, rt * 16 + 4 * g);
+  for (int rt = 0; rt < RT; ++rt) {
+    rc[rt] = load_row_const(pr, rt * 16 + 4 * g);
+    any_flag |= rc[rt].flag;
+  }
   __syncthreads();
   const uint4 *lds4 = (const uint4 *)smem;
 
@@ -605,98 +637,159 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
         for (int rt = 0; rt < RT; ++rt) flow_epilogue<P>(pr, n, rt * 16 + 4 * g, acc[tw][rt], sc[tw], rc[rt]);
       }
     }
+    if (any_flag) {
+      for (int tw = 0; tw < TW; ++tw) {
+        const int t = first + tw * S + s;
+        const int n = t * 16 + i;
+        if (t >= pr.n_tiles || n >= pr.n) continue;
+        for (int rt = 0; rt < RT; ++rt) {
+          const int rowbase = rt * 16 + 4 * g;
+          const unsigned fl = row_flags(pr, rowbase);
+          if (fl) exact_rows(pr, n, rowbase, fl);
+        }
+      }
+    }
   }
 }
 
 // ------------------------------------------------------------------------------------------
-// prefill GEMM: workgroup tile = (RT*16 operand rows) x (4 waves * NT * 16 outputs).
-// A operands are staged per K block in LDS and shared by the four waves; weights are never
-// staged: each wave streams the 2-bit chunks of its own output tiles straight into registers and
-// expands them when the MFMA operand is formed.
+// prefill GEMM, pipelined form. Workgroup tile = 64 operand rows x (4 waves * NT tiles * 16 outputs),
+// all P planes of a tile in the same wave (P*NT = 8 accumulator tiles per row tile, so one LDS read
+// of an A operand feeds 8 MFMAs). A blocks of 256 k are double-buffered in LDS: while the MFMAs of
+// block kb run, the global loads of block kb+1 (A rows into registers, 2-bit weight chunks into
+// registers) are in flight; one barrier per block.
 // ------------------------------------------------------------------------------------------
 
-template <int P, int RT, int NT>
-__global__ __launch_bounds__(TK_WG) void tk_gemm_kernel(TkProblem pr) {
+template <int P, int NT>
+__global__ __launch_bounds__(TK_WG) void tk_gemm2_kernel(const TkProblem pr) {
+  constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, PER_T = A4 / TK_WG;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int i = lane & 15, g = lane >> 4;
   const int nb = pr.nb, R = pr.R;
-  const int row0 = blockIdx.x * RT * 16;
-  const int tile0 = (blockIdx.y * 4 + wave) * NT;  // first output tile of this wave
+  const int row0 = blockIdx.x * ROWS;
+  const int tile0 = (blockIdx.y * 4 + wave) * NT;
   uint4 *lds4 = (uint4 *)smem;
   const uint4 *ap4 = (const uint4 *)pr.ap;
 
-  float outf[RT][NT][4];
-  v4i acc[RT][NT];
-
-#pragma unroll 1
-  for (int p = 0; p < P; ++p) {
+  // weight chunk pointers (tiles past the end re-read the last tile; their results are dropped)
+  const uint8_t *wp[NT][P];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+  for (int nt = 0; nt < NT; ++nt) {
+    const int t = min(tile0 + nt, pr.n_tiles - 1);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = v4i{0, 0, 0, 0};
-
-    const uint8_t *codes = pr.codes[p];
-    for (int kb = 0; kb < nb; ++kb) {
-      uint4 w[NT];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const int tl = tile0 + nt;
-        w[nt] = make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
-        if (tl < pr.n_tiles) w[nt] = *(const uint4 *)(codes + (((size_t)tl * nb + kb) * 64 + lane) * 16);
-      }
-      __syncthreads();
-      // stage A: 16 (j,g) segments of RT*16 rows each
-      for (int idx = threadIdx.x; idx < 16 * RT * 16; idx += TK_WG) {
-        const int seg = idx / (RT * 16), rr = idx % (RT * 16);
-        uint4 q = make_uint4(0, 0, 0, 0);
-        if (row0 + rr < R) q = ap4[((size_t)kb * 16 + seg) * R + row0 + rr];
-        lds4[idx] = q;
-      }
-      __syncthreads();
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v4i b[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const uint32_t wj = j == 0 ? w[nt].x : (j == 1 ? w[nt].y : (j == 2 ? w[nt].z : w[nt].w));
-          b[nt] = expand_codes(wj);
-        }
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          const uint4 q = lds4[(j * 4 + g) * (RT * 16) + rt * 16 + i];
-          const v4i a = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            acc[rt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b[nt], acc[rt][nt], 0, 0, 0);
-        }
-      }
-    }
-    // fold this plane
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const int n = (tile0 + nt) * 16 + i;
-        const int rowbase = row0 + rt * 16 + 4 * g;
-        if (n < pr.n) {
-          if (pr.out_dtype == TK_I32) {
-            if (p == 0) store_raw(pr, n, rowbase, acc[rt][nt]);
-          } else {
-            fold_plane(pr, p, n, rowbase, acc[rt][nt], outf[rt][nt], p == 0);
-          }
-        }
-      }
+    for (int p = 0; p < P; ++p) wp[nt][p] = pr.codes[p] + ((size_t)t * nb * 64 + lane) * 16;
   }
-  if (pr.out_dtype == TK_I32) return;
+  // this thread's share of an A block: PER_T pieces of 16 bytes
+  int a_src[PER_T];
+  bool a_ok[PER_T];
+#pragma unroll
+  for (int u = 0; u < PER_T; ++u) {
+    const int idx = threadIdx.x + u * TK_WG;
+    const int seg = idx / ROWS, rr = idx % ROWS;
+    a_ok[u] = row0 + rr < R;
+    a_src[u] = seg * R + row0 + rr;
+  }
+
+  v4i acc[RT][NT][P];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int n = (tile0 + nt) * 16 + i;
-      const int rowbase = row0 + rt * 16 + 4 * g;
-      if (n < pr.n) finish_lane(pr, n, rowbase, outf[rt][nt]);
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int p = 0; p < P; ++p) acc[rt][nt][p] = v4i{0, 0, 0, 0};
+
+  uint4 wc[NT][P], wn[NT][P], areg[PER_T];
+  if (nb > 0) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int p = 0; p < P; ++p) wc[nt][p] = *(const uint4 *)(wp[nt][p]);
+#pragma unroll
+    for (int u = 0; u < PER_T; ++u) {
+      uint4 q = make_uint4(0, 0, 0, 0);
+      if (a_ok[u]) q = ap4[a_src[u]];
+      lds4[threadIdx.x + u * TK_WG] = q;
     }
+  }
+  __syncthreads();
+
+  for (int kb = 0; kb < nb; ++kb) {
+    const bool more = kb + 1 < nb;
+    if (more) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int p = 0; p < P; ++p) wn[nt][p] = *(const uint4 *)(wp[nt][p] + (size_t)(kb + 1) * TK_CHUNK_BYTES);
+#pragma unroll
+      for (int u = 0; u < PER_T; ++u) {
+        areg[u] = make_uint4(0, 0, 0, 0);
+        if (a_ok[u]) areg[u] = ap4[(size_t)(kb + 1) * 16 * R + a_src[u]];
+      }
+    }
+    const uint4 *buf = lds4 + (kb & 1) * A4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v4i a[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const uint4 q = buf[(j * 4 + g) * ROWS + rt * 16 + i];
+        a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          const uint4 w = wc[nt][p];
+          const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
+          const v4i b = expand_codes(wj);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][nt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[rt][nt][p], 0, 0, 0);
+        }
+    }
+    if (more) {
+      uint4 *nbuf = lds4 + ((kb + 1) & 1) * A4;
+#pragma unroll
+      for (int u = 0; u < PER_T; ++u) nbuf[threadIdx.x + u * TK_WG] = areg[u];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int p = 0; p < P; ++p) wc[nt][p] = wn[nt][p];
+    }
+    __syncthreads();
+  }
+
+  RowConst rc[RT];
+  unsigned any_flag = 0;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    rc[rt] = load_row_const(pr, row0 + rt * 16 + 4 * g);
+    any_flag |= rc[rt].flag;
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int t = tile0 + nt;
+    const int n = t * 16 + i;
+    if (t >= pr.n_tiles || n >= pr.n) continue;
+    float sc[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) sc[p] = pr.scales[p][n];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) flow_epilogue<P>(pr, n, row0 + rt * 16 + 4 * g, acc[rt][nt], sc, rc[rt]);
+  }
+  if (any_flag) {
+    for (int nt = 0; nt < NT; ++nt) {
+      const int t = tile0 + nt;
+      const int n = t * 16 + i;
+      if (t >= pr.n_tiles || n >= pr.n) continue;
+      for (int rt = 0; rt < RT; ++rt) {
+        const int rowbase = row0 + rt * 16 + 4 * g;
+        const unsigned fl = row_flags(pr, rowbase);
+        if (fl) exact_rows(pr, n, rowbase, fl);
+      }
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1125,15 +1218,17 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
   }
 }
 
+int tk_gemm_tiles_per_wave(int planes) { return planes == 1 ? 8 : (planes == 2 ? 4 : 2); }
+
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n) {
   if (!grid_m || !grid_n) return hipSuccess;
   dim3 grid(grid_m, grid_n), block(TK_WG);
   switch (cfg.planes) {
-    case 1: hipLaunchKernelGGL((tk_gemm_kernel<1, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 2: hipLaunchKernelGGL((tk_gemm_kernel<2, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 3: hipLaunchKernelGGL((tk_gemm_kernel<3, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 4: hipLaunchKernelGGL((tk_gemm_kernel<4, 8, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 1: hipLaunchKernelGGL((tk_gemm2_kernel<1, 8>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 2: hipLaunchKernelGGL((tk_gemm2_kernel<2, 4>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 3: hipLaunchKernelGGL((tk_gemm2_kernel<3, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 4: hipLaunchKernelGGL((tk_gemm2_kernel<4, 2>), grid, block, cfg.lds_bytes, s, *single); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
