@@ -484,8 +484,26 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->cfg.rt = 4;
     pl->cfg.lds_bytes = 2 * 16 * 64 * 16;  // two 64-row blocks of 256 k
     pl->grid_m = (unsigned)((R + 63) / 64);
-    const unsigned per_wg = 4u * (unsigned)tk_gemm_tiles_per_wave(layer->n_planes);
+    const unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(layer->n_planes);
     pl->grid_n = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
+    // split the tile grid over the 8 XCDs so that each L2 holds few A row blocks and few weight
+    // column blocks: minimise bytes touched per XCD = K·(64·sub_m + 4·tiles_per_wg·planes·sub_n)
+    pr.grid_m = (int)pl->grid_m;
+    pr.grid_n = (int)pl->grid_n;
+    size_t best = (size_t)-1;
+    for (int xr = 1; xr <= 8; xr *= 2) {
+      const int xc = 8 / xr;
+      const int sm = ((int)pl->grid_m + xr - 1) / xr, sn = ((int)pl->grid_n + xc - 1) / xc;
+      const size_t cost = (size_t)64 * sm + (size_t)4 * per_wg * layer->n_planes * sn;
+      const size_t waste = (size_t)8 * sm * sn;  // launched workgroups, some of them empty
+      const size_t score = cost * 1024 + waste;
+      if (score < best) {
+        best = score;
+        pr.xr = xr;
+        pr.sub_m = sm;
+        pr.sub_n = sn;
+      }
+    }
   }
 }
 

@@ -43,6 +43,8 @@ struct TkProblem {
   int kc;                    // K blocks staged in LDS per pass (decode kernels)
   int group_begin;           // streaming / flow kernels: first workgroup index of this problem
   int run_tiles;             // flow kernel: consecutive tiles per run (S)
+  int grid_m, grid_n;        // GEMM: row blocks and column blocks
+  int xr, sub_m, sub_n;      // GEMM: XCDs along M, and the tile sub-grid one XCD owns
 };
 
 enum { TK_PREP_A8 = 0, TK_PREP_DIGITS = 1, TK_PREP_I8 = 2 };
@@ -91,7 +93,7 @@ hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProb
 int tk_flow_runs_per_wave(int planes, int rt);
 hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
-int tk_gemm_tiles_per_wave(int planes);
+int tk_gemm_tiles_per_wg(int planes);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

@@ -653,63 +653,73 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
 }
 
 // ------------------------------------------------------------------------------------------
-// prefill GEMM, pipelined form. Workgroup tile = 64 operand rows x (4 waves * NT tiles * 16 outputs),
-// all P planes of a tile in the same wave (P*NT = 8 accumulator tiles per row tile, so one LDS read
-// of an A operand feeds 8 MFMAs). A blocks of 256 k are double-buffered in LDS: while the MFMAs of
-// block kb run, the global loads of block kb+1 (A rows into registers, 2-bit weight chunks into
-// registers) are in flight; one barrier per block.
+// prefill GEMM. Workgroup tile = 64 operand rows x (TK_GEMM_WAVES waves * NT tiles * 16 outputs),
+// all P planes of a tile in the same wave (P*NT = 4 accumulator tiles per row tile, so one LDS read
+// of an A operand feeds 4 MFMAs). A blocks of 256 k are double-buffered in LDS: while the MFMAs of
+// block kb run, the global loads of block kb+1 (A rows, and the 2-bit weight chunks, both into
+// registers) are in flight; one barrier per block. Weights never pass through LDS: each wave
+// streams the chunks of its own output tiles and expands a dword into an MFMA operand when needed.
+// A single wave cannot keep the MFMA pipe full (measured: ~25 cycles per 16x16x64 issue from one
+// wave, ~18 from two), and waves of one workgroup stall together at its barrier, so the kernel is
+// sized for several independent workgroups per CU.
 // ------------------------------------------------------------------------------------------
 
+#ifndef TK_GEMM_WAVES
+#define TK_GEMM_WAVES 4
+#endif
+#define TK_GEMM_THREADS (TK_GEMM_WAVES * 64)
+
 template <int P, int NT>
-__global__ __launch_bounds__(TK_WG) void tk_gemm2_kernel(const TkProblem pr) {
-  constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, PER_T = A4 / TK_WG;
+__global__ __launch_bounds__(TK_GEMM_THREADS) void tk_gemm_kernel(const TkProblem pr) {
+  constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, PER_T = A4 / TK_GEMM_THREADS, NB = NT * P;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int i = lane & 15, g = lane >> 4;
   const int nb = pr.nb, R = pr.R;
-  const int row0 = blockIdx.x * ROWS;
-  const int tile0 = (blockIdx.y * 4 + wave) * NT;
+  // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, each with its own
+  // L2. XCD x = id % 8 gets a compact sub-grid of sub_m x sub_n tiles, so the A row blocks and the
+  // weight column blocks it touches stay resident in that L2 instead of every XCD streaming all.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int bm = (xcd % pr.xr) * pr.sub_m + slot % pr.sub_m;
+  const int bn = (xcd / pr.xr) * pr.sub_n + slot / pr.sub_m;
+  if (bm >= pr.grid_m || bn >= pr.grid_n) return;
+  const int row0 = bm * ROWS;
+  const int tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
   uint4 *lds4 = (uint4 *)smem;
   const uint4 *ap4 = (const uint4 *)pr.ap;
 
-  // weight chunk pointers (tiles past the end re-read the last tile; their results are dropped)
-  const uint8_t *wp[NT][P];
+  // weight chunk offsets inside a plane (tiles past the end re-read the last tile; results dropped)
+  unsigned woff[NT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    const int t = min(tile0 + nt, pr.n_tiles - 1);
-#pragma unroll
-    for (int p = 0; p < P; ++p) wp[nt][p] = pr.codes[p] + ((size_t)t * nb * 64 + lane) * 16;
-  }
-  // this thread's share of an A block: PER_T pieces of 16 bytes
+  for (int nt = 0; nt < NT; ++nt) woff[nt] = ((unsigned)min(tile0 + nt, pr.n_tiles - 1) * (unsigned)nb * 64u + lane) * 16u;
+  // this thread's share of an A block
   int a_src[PER_T];
   bool a_ok[PER_T];
 #pragma unroll
   for (int u = 0; u < PER_T; ++u) {
-    const int idx = threadIdx.x + u * TK_WG;
+    const int idx = threadIdx.x + u * TK_GEMM_THREADS;
     const int seg = idx / ROWS, rr = idx % ROWS;
     a_ok[u] = row0 + rr < R;
     a_src[u] = seg * R + row0 + rr;
   }
 
-  v4i acc[RT][NT][P];
+  v4i acc[RT][NB];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int p = 0; p < P; ++p) acc[rt][nt][p] = v4i{0, 0, 0, 0};
+    for (int x = 0; x < NB; ++x) acc[rt][x] = v4i{0, 0, 0, 0};
 
-  uint4 wc[NT][P], wn[NT][P], areg[PER_T];
+  uint4 wc[NB], wn[NB], areg[PER_T];
   if (nb > 0) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int p = 0; p < P; ++p) wc[nt][p] = *(const uint4 *)(wp[nt][p]);
+      for (int p = 0; p < P; ++p) wc[nt * P + p] = *(const uint4 *)(pr.codes[p] + woff[nt]);
 #pragma unroll
     for (int u = 0; u < PER_T; ++u) {
       uint4 q = make_uint4(0, 0, 0, 0);
       if (a_ok[u]) q = ap4[a_src[u]];
-      lds4[threadIdx.x + u * TK_WG] = q;
+      lds4[threadIdx.x + u * TK_GEMM_THREADS] = q;
     }
   }
   __syncthreads();
@@ -720,7 +730,8 @@ __global__ __launch_bounds__(TK_WG) void tk_gemm2_kernel(const TkProblem pr) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int p = 0; p < P; ++p) wn[nt][p] = *(const uint4 *)(wp[nt][p] + (size_t)(kb + 1) * TK_CHUNK_BYTES);
+        for (int p = 0; p < P; ++p)
+          wn[nt * P + p] = *(const uint4 *)(pr.codes[p] + woff[nt] + (size_t)(kb + 1) * TK_CHUNK_BYTES);
 #pragma unroll
       for (int u = 0; u < PER_T; ++u) {
         areg[u] = make_uint4(0, 0, 0, 0);
@@ -737,25 +748,20 @@ __global__ __launch_bounds__(TK_WG) void tk_gemm2_kernel(const TkProblem pr) {
         a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
       }
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
+      for (int x = 0; x < NB; ++x) {
+        const uint32_t wj = j == 0 ? wc[x].x : (j == 1 ? wc[x].y : (j == 2 ? wc[x].z : wc[x].w));
+        const v4i b = expand_codes(wj);
 #pragma unroll
-        for (int p = 0; p < P; ++p) {
-          const uint4 w = wc[nt][p];
-          const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
-          const v4i b = expand_codes(wj);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            acc[rt][nt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[rt][nt][p], 0, 0, 0);
-        }
+        for (int rt = 0; rt < RT; ++rt)
+          acc[rt][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[rt][x], 0, 0, 0);
+      }
     }
     if (more) {
       uint4 *nbuf = lds4 + ((kb + 1) & 1) * A4;
 #pragma unroll
-      for (int u = 0; u < PER_T; ++u) nbuf[threadIdx.x + u * TK_WG] = areg[u];
+      for (int u = 0; u < PER_T; ++u) nbuf[threadIdx.x + u * TK_GEMM_THREADS] = areg[u];
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int p = 0; p < P; ++p) wc[nt][p] = wn[nt][p];
+      for (int x = 0; x < NB; ++x) wc[x] = wn[x];
     }
     __syncthreads();
   }
@@ -776,7 +782,12 @@ __global__ __launch_bounds__(TK_WG) void tk_gemm2_kernel(const TkProblem pr) {
 #pragma unroll
     for (int p = 0; p < P; ++p) sc[p] = pr.scales[p][n];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) flow_epilogue<P>(pr, n, row0 + rt * 16 + 4 * g, acc[rt][nt], sc, rc[rt]);
+    for (int rt = 0; rt < RT; ++rt) {
+      v4i av[P];
+#pragma unroll
+      for (int p = 0; p < P; ++p) av[p] = acc[rt][nt * P + p];
+      flow_epilogue<P>(pr, n, row0 + rt * 16 + 4 * g, av, sc, rc[rt]);
+    }
   }
   if (any_flag) {
     for (int nt = 0; nt < NT; ++nt) {
@@ -1218,17 +1229,18 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
   }
 }
 
-int tk_gemm_tiles_per_wave(int planes) { return planes == 1 ? 8 : (planes == 2 ? 4 : 2); }
+// output tiles per workgroup of the GEMM for a plane count
+int tk_gemm_tiles_per_wg(int planes) { return TK_GEMM_WAVES * (planes == 1 ? 4 : (planes == 2 ? 2 : 1)); }
 
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n) {
   if (!grid_m || !grid_n) return hipSuccess;
-  dim3 grid(grid_m, grid_n), block(TK_WG);
+  dim3 grid(8u * (unsigned)single->sub_m * (unsigned)single->sub_n), block(TK_GEMM_THREADS);
   switch (cfg.planes) {
-    case 1: hipLaunchKernelGGL((tk_gemm2_kernel<1, 8>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 2: hipLaunchKernelGGL((tk_gemm2_kernel<2, 4>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 3: hipLaunchKernelGGL((tk_gemm2_kernel<3, 2>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 4: hipLaunchKernelGGL((tk_gemm2_kernel<4, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 1: hipLaunchKernelGGL((tk_gemm_kernel<1, 4>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 2: hipLaunchKernelGGL((tk_gemm_kernel<2, 2>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 3: hipLaunchKernelGGL((tk_gemm_kernel<3, 1>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 4: hipLaunchKernelGGL((tk_gemm_kernel<4, 1>), grid, block, cfg.lds_bytes, s, *single); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
