@@ -27,6 +27,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+# HBM bytes per launch of the decode kernel (sweep average), from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration against a 1 GiB copy kernel):
+# profiles/decode_flow_c2_sweep_traffic.txt
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_157_498_880
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 
 K2, N2, PLANES2 = 2048, 8192, 2
@@ -214,21 +218,26 @@ def cpu_baseline(rng):
     planes = [orc.pack_matrix(ternary(rng, N2, K2, p0), N2, K2, oracle_lib.FMT_TQ2_0) for p0 in (0.4, 0.7)]
     scs = [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)]
     threads = min(os.cpu_count() or 1, 16)
-    used_max, total_bytes = 0, 0
-    t0 = time.perf_counter()
+    used_max, total_bytes, passes = 0, 0, 0
+    acts = []
     for m in SWEEP:
         bits = f32_to_bf16_bits(rng.standard_normal((m, K2)).astype(np.float32))
-        act = (bits.astype(np.uint32) << 16).view(np.float32).reshape(m, K2)
-        out = None
-        for p in range(PLANES2):
-            o, used, _ = orc.cpu_mpgemm_fast(planes[p], oracle_lib.FMT_TQ2_0, act, scs[p], m, N2, K2, threads)
-            out = o if out is None else out + o
-            used_max = max(used_max, used)
-        total_bytes += algorithmic_bytes(m, N2, K2, PLANES2, 2, 4)
+        acts.append((bits.astype(np.uint32) << 16).view(np.float32).reshape(m, K2))
+    t0 = time.perf_counter()
+    while passes < 60 and time.perf_counter() - t0 < 12.0:  # a bounded sample: about 12 s of CPU work
+        for m, act in zip(SWEEP, acts):
+            out = None
+            for p in range(PLANES2):
+                o, used, _ = orc.cpu_mpgemm_fast(planes[p], oracle_lib.FMT_TQ2_0, act, scs[p], m, N2, K2, threads)
+                out = o if out is None else out + o
+                used_max = max(used_max, used)
+            total_bytes += algorithmic_bytes(m, N2, K2, PLANES2, 2, 4)
+        passes += 1
     dt = time.perf_counter() - t0
     return {"value": round(total_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": used_max, "kind": "port",
-            "sample": f"one pass of the sweep (batch {','.join(map(str, SWEEP))}) over ONE layer copy, "
-                      f"{dt:.2f} s; tritium-cpu's row chunking gives batch 1 a single worker"}
+            "sample": f"{passes} passes of the sweep (batch {','.join(map(str, SWEEP))}) over ONE layer copy, "
+                      f"{dt:.1f} s; C restatement of tritium-cpu (unpack per call, AVX-512 k-order f32 fold, rows "
+                      f"chunked over threads: batch 1 gets a single worker, batch 16 gets {used_max})"}
 
 
 def main():
@@ -238,6 +247,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM and projection-stack legs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a plain 1 GiB device copy kernel 3 times (scale for hardware traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards over output channels without any "
@@ -265,14 +276,22 @@ def main():
                                f"each batch one launch over {COPIES} resident layer copies",
                    "copies": COPIES, "bytes_per_step": int(dec["bytes_per_launch_avg"] * len(SWEEP))},
         "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "tk_skinny_kernel<2,*>", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
+                     "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "tk_flow_kernel<2,*>", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
                      "algorithmic_bytes_per_launch": int(dec["bytes_per_launch_avg"])},
         "per_batch": dec["per_batch"],
         "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
                    "clock_mhz": info.clock_khz / 1000, "memory_clock_mhz": info.memory_clock_khz / 1000,
                    "memory_bus_bits": info.memory_bus_bits},
     }
+    if args.copy_calibration:
+        n = 1 << 30
+        src, dst = be.empty(n // 4, "f32"), be.empty(n // 4, "f32")
+        for _ in range(3):
+            be.copy_kernel(dst, src, n)
+        be.sync()
+        src.free()
+        dst.free()
     if not args.no_extra:
         out["extra"] = {"prefill_gemm": bench_prefill(T, be, rng), "projection_stack": bench_stack(T, be, rng)}
     if not args.no_cpu:

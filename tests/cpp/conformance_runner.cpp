@@ -1,0 +1,108 @@
+// Conformance of the C++ adapter (tritium_amd/csrc/tritium_backend.hpp) through the TernaryBackend
+// interface, as the reference's harness drives any backend (crates/tritium-testkit/src/runner.rs:171-267,
+// 288-420). Test infrastructure: links the CPU oracle for the vectors and expected values.
+//   conformance_runner           run on device 0, print a report, exit 0 on success
+//   conformance_runner --nogpu   only the host-side checks (registry skips an unavailable device)
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../oracle/tritium_oracle.h"
+#include "../../tritium_amd/csrc/tritium_backend.hpp"
+
+using namespace tritium;
+
+static int failures = 0;
+#define CHECK(cond, ...)                     \
+  do {                                       \
+    if (!(cond)) {                           \
+      ++failures;                            \
+      std::printf("FAIL %s:%d: ", __FILE__, __LINE__); \
+      std::printf(__VA_ARGS__);              \
+      std::printf("\n");                     \
+    }                                        \
+  } while (0)
+
+static bool same_bits(const float *a, const float *b, size_t n) { return std::memcmp(a, b, n * 4) == 0; }
+
+int main(int argc, char **argv) {
+  const bool nogpu = argc > 1 && !std::strcmp(argv[1], "--nogpu");
+  Registry reg;
+  if (nogpu) {
+    // no device in this container: the entry fails to initialise, is logged and skipped
+    CHECK(reg.is_empty() || reg.get("mi355x") != nullptr, "registry state");
+    CHECK(backends().size() == 1 && backends()[0].name == "mi355x", "registration record");
+    std::printf("%s\n", failures ? "FAILED" : "OK (host-side only)");
+    return failures != 0;
+  }
+  TernaryBackend *be = reg.get("mi355x");
+  if (!be) {
+    std::printf("FAILED: backend mi355x did not initialise\n");
+    return 1;
+  }
+  CHECK(be->device_id() == "mi355x:0", "device_id %s", be->device_id().c_str());
+  CHECK(be->capabilities().backend == "mi355x" && be->capabilities().supports_imma, "capabilities");
+  CHECK(be->mpgemm_projected_vjp().has_value(), "vjp must be refused");
+  CHECK(be->as_concrete() != nullptr, "as_concrete");
+
+  to_vector_set *set = to_generate_vectors(0xC0FFEE, 64);
+  size_t passed = 0;
+  for (size_t i = 0; i < set->count; ++i) {
+    const to_vector &v = set->v[i];
+    const size_t len = v.n * to_row_bytes(v.k, v.format);
+    std::vector<uint8_t> packed(len);
+    to_pack_matrix(v.weights, v.n, v.k, v.format, packed.data(), len);
+    std::unique_ptr<DeviceBuffer> buf;
+    GemmShape shape{v.m, v.n, v.k};
+    Status e = be->upload_weights(packed.data(), len, shape, (TernaryFormat)v.format, &buf);
+    CHECK(!e, "%s upload: %s", v.id, e ? e->message.c_str() : "");
+    if (e) continue;
+    CHECK(buf->len_bytes() == len, "%s len_bytes", v.id);
+    std::vector<float> out(v.m * v.n, -1.0f), want(v.m * v.n);
+    MpGemm p{v.activation, v.m * v.k, buf.get(), v.scales, v.n, shape, (TernaryFormat)v.format, out.data(), out.size()};
+    e = be->mpgemm(p);
+    CHECK(!e, "%s mpgemm: %s", v.id, e ? e->message.c_str() : "");
+    bool ok = true;
+    for (size_t j = 0; j < out.size(); ++j) ok &= to_accepts_with_floor(out[j], v.expected[j], 1e-4f, 0, 1.0f) != 0;
+    CHECK(ok, "%s beyond 1e-4", v.id);
+    // fused path == the trait's host default, bit for bit
+    e = be->mpgemm_with_act_quant(p);
+    CHECK(!e, "%s fused: %s", v.id, e ? e->message.c_str() : "");
+    to_cpu_mpgemm_with_act_quant(packed.data(), len, v.format, v.activation, v.m * v.k, v.scales, v.n, v.m, v.n, v.k,
+                                 want.data(), want.size());
+    CHECK(same_bits(out.data(), want.data(), out.size()), "%s fused bits", v.id);
+    // and the base class's default composition over this backend's mpgemm gives the same bits
+    std::vector<float> viadefault(v.m * v.n);
+    MpGemm pd = p;
+    pd.out = viadefault.data();
+    e = be->TernaryBackend::mpgemm_with_act_quant(pd);
+    CHECK(!e && same_bits(viadefault.data(), want.data(), want.size()), "%s default composition", v.id);
+    passed += ok;
+  }
+  // error paths (crates/tritium-cpu/src/lib.rs:801-886)
+  {
+    std::vector<uint8_t> shortbuf(2 * 66 - 1);
+    std::unique_ptr<DeviceBuffer> buf;
+    Status e = be->upload_weights(shortbuf.data(), shortbuf.size(), GemmShape{1, 2, 256}, TernaryFormat::Tq2_0, &buf);
+    CHECK(e && e->kind == BackendError::InvalidInput, "short upload");
+    e = be->upload_weights(shortbuf.data(), 64, GemmShape{1, 1, 256}, TernaryFormat::I2sInt8, &buf);
+    CHECK(e && e->kind == BackendError::UnsupportedFormat, "unsupported format");
+    std::vector<uint8_t> ok(66, 0x55);
+    e = be->upload_weights(ok.data(), 66, GemmShape{0, 1, 256}, TernaryFormat::Tq2_0, &buf);
+    CHECK(!e, "upload");
+    std::vector<float> act(256), sc(1, 1.0f), out(2);
+    MpGemm p{act.data(), 256, buf.get(), sc.data(), 1, GemmShape{2, 1, 256}, TernaryFormat::Tq2_0, out.data(), 2};
+    e = be->mpgemm(p);
+    CHECK(e && e->kind == BackendError::ShapeMismatch && e->expected == 512 && e->got == 256, "operand length");
+    struct Foreign : DeviceBuffer {
+      size_t len_bytes() const override { return 0; }
+    } foreign;
+    p.weights = &foreign;
+    e = be->mpgemm(p);
+    CHECK(e && e->kind == BackendError::InvalidInput, "foreign buffer");
+  }
+  std::printf("conformance: %zu/%zu vectors passed, %d failures\n", passed, set->count, failures);
+  to_free_vectors(set);
+  std::printf("%s\n", failures ? "FAILED" : "OK");
+  return failures != 0;
+}

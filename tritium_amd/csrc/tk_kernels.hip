@@ -669,8 +669,13 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
 #endif
 #define TK_GEMM_THREADS (TK_GEMM_WAVES * 64)
 
+#ifndef TK_GEMM_OCC
+#define TK_GEMM_OCC 3
+#endif
+
 template <int P, int NT>
-__global__ __launch_bounds__(TK_GEMM_THREADS) void tk_gemm_kernel(const TkProblem pr) {
+__global__ __launch_bounds__(TK_GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(TK_GEMM_OCC, TK_GEMM_OCC))) void
+tk_gemm_kernel(const TkProblem pr) {
   constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, PER_T = A4 / TK_GEMM_THREADS, NB = NT * P;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
