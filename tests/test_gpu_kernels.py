@@ -256,6 +256,61 @@ def test_gemm_crossover_is_bit_neutral(backend, oracle):
     assert same_bits(a, b) and same_bits(a, want)
 
 
+@pytest.mark.parametrize("m,n,k", [(65, 64, 512), (150, 136, 768), (130, 131, 512), (300, 520, 256)])
+def test_gemm_epilogue_variants(backend, oracle, m, n, k, decode_kernel):
+    """The prefill kernel's two ways out -- rows staged through LDS when the output rows are 16-byte
+    aligned, direct stores otherwise -- for every output type, both activation contracts, and with
+    tokens that take the exact NaN/Inf path in the middle of a tile."""
+    if decode_kernel != "ksplit":
+        pytest.skip("the prefill kernel does not depend on the decode kernel choice")
+    print("case gemm-epilogue", m, n, k, flush=True)
+    rng = np.random.default_rng(m * 7 + n)
+    ws = [ternary(rng, n, k, 0.4), ternary(rng, n, k, 0.7)]
+    scs = [scales(rng, n), scales(rng, n)]
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[3, 5] = np.nan
+    act[m - 2, k - 1] = np.inf
+    act[40] = 0.0
+    packed, layer = _layer(backend, oracle, ws, scs)
+    dact = backend.to_device(act, "f32")
+    want_a8 = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k).reshape(m, n)
+    want_f = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k).reshape(m, n)
+    fin = np.isfinite(want_f)
+    for dtype in ("f32", "bf16"):
+        dout = backend.empty(m * n, dtype)
+        backend.linear_a8(layer, dact, m, dout)
+        got = dout.to_host().reshape(m, n)
+        if dtype == "bf16":
+            ok = ~np.isnan(want_a8)
+            assert (np.isnan(bf16_bits_to_f32(got).reshape(m, n)) == ~ok).all()
+            assert (got[ok] == f32_to_bf16_bits(want_a8).reshape(m, n)[ok]).all()
+        else:
+            assert (np.isnan(got) == np.isnan(want_a8)).all()
+            assert same_bits(got[~np.isnan(want_a8)], want_a8[~np.isnan(want_a8)])
+        backend.linear_float(layer, dact, m, dout)
+        got = dout.to_host().reshape(m, n)
+        if dtype == "bf16":
+            got = bf16_bits_to_f32(got).reshape(m, n)
+            assert (np.isnan(got) == np.isnan(want_f)).all()
+            assert accepts(got[fin], want_f[fin], rel=1e-2, floor=1.0).all()  # bf16 keeps 8 bits
+        else:
+            assert (np.isnan(got) == np.isnan(want_f)).all()
+            assert accepts(got[fin], want_f[fin], rel=1e-4, floor=1.0).all()
+            # rows with NaN/Inf are computed in the reference's order: bits equal the CPU's
+            assert same_bits(got[3][fin[3]], want_f[3][fin[3]]) and same_bits(got[m - 2][fin[m - 2]], want_f[m - 2][fin[m - 2]])
+        dout.free()
+    # raw accumulators of one plane
+    q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    single = backend.linear([packed[0]], [scs[0]], n, k, T.TernaryFormat(FMT_TQ2_0))
+    dq, dacc = backend.to_device(q, "i8"), backend.empty(m * n, "i32")
+    backend.linear_i8(single, dq, None, m, dacc)
+    assert (dacc.to_host().reshape(m, n) == oracle.int8_accumulators(packed[0], FMT_TQ2_0, q, m, n, k)).all()
+    for a in (dact, dq, dacc):
+        a.free()
+    single.free()
+    layer.free()
+
+
 def test_group_launch_equals_single_launches(backend, oracle):
     rng = np.random.default_rng(29)
     k = 768

@@ -453,6 +453,7 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
   pr.k = (int)k;
   pr.nb = (int)nb;
   pr.R = (int)R;
+  pr.rs = (int)R;
   pr.M = (int)m;
   pr.mode = mode;
   pr.out_dtype = out_dtype;
@@ -481,8 +482,12 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->flow_lds = nb * 256 * R;
     pl->flow_ok = pl->flow_lds <= kLdsFlowMax;
   } else {
+    // The GEMM reads, per K block, 16 segments of the operand rows that are exactly rs*16 bytes apart,
+    // and all workgroups do so in step: with a power-of-two stride they would all land on the same
+    // few memory channels. 16 rows (256 bytes) of padding walk the segments across the channels.
+    pr.rs = (int)(R + 16);
     pl->cfg.rt = 4;
-    pl->cfg.lds_bytes = 2 * 16 * 64 * 16;  // two 64-row blocks of 256 k
+    pl->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();  // three 64-row blocks of 256 k
     pl->grid_m = (unsigned)((R + 63) / 64);
     const unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(layer->n_planes);
     pl->grid_n = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
@@ -522,7 +527,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   Plan pl;
   plan_shape(ctx, layer, n, k, m, mode, out_dtype, &pl);
   const size_t nb = pl.pr.nb, R = pl.pr.R;
-  TKCHK(ensure(ctx, ctx->ap, R * nb * 256));
+  TKCHK(ensure(ctx, ctx->ap, (size_t)pl.pr.rs * nb * 256));
   TKCHK(ensure(ctx, ctx->rowsum, R * 4));
   TKCHK(ensure(ctx, ctx->fscale, m * 4));
   TKCHK(ensure(ctx, ctx->aux, m * 4));
@@ -540,6 +545,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   pp.k = k;
   pp.nb = nb;
   pp.R = R;
+  pp.rs = (size_t)pl.pr.rs;
   pp.act_dtype = act_dtype;
   pp.m = (int)m;
   HIPCHK(tk_launch_prep(ctx->stream, prep_kind, &pp, nullptr, 0, (unsigned)m));
@@ -673,6 +679,7 @@ extern "C" int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size
   pp.k = k;
   pp.nb = num_blocks(k);
   pp.R = m;
+  pp.rs = m;
   pp.act_dtype = act_dtype;
   pp.m = (int)m;
   HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_A8, &pp, nullptr, 0, (unsigned)m));
@@ -816,6 +823,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       pp.k = k;
       pp.nb = nb;
       pp.R = R;
+      pp.rs = R;
       pp.act_dtype = act_dtype;
       pp.m = (int)m;
       pp.row_begin = (int)rows;

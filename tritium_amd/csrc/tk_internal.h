@@ -37,6 +37,7 @@ struct TkProblem {
   const void *raw_act;       // original activations [M,K] for the fallback (or null)
   void *out;                 // [M,N]
   int n, k, nb, R, M;
+  int rs;                    // row stride of `ap` in rows (>= R; the GEMM pads it, see tk_api.hip)
   int mode, raw_dtype, out_dtype, planes;
   int tile_begin;            // first launch-wide tile index of this problem
   int n_tiles;               // ceil(n/16)
@@ -60,6 +61,7 @@ struct TkPrep {
   uint32_t *flags;      // [m]
   int8_t *q_rowmajor;   // A8: optional plain [m,k] int8 copy
   size_t k, nb, R;
+  size_t rs;            // row stride of `ap` in rows (>= R)
   int act_dtype;
   int row_begin;        // first launch-wide token index of this tensor
   int m;
@@ -94,6 +96,7 @@ int tk_flow_runs_per_wave(int planes, int rt);
 hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
 int tk_gemm_tiles_per_wg(int planes);
+int tk_gemm_lds_bytes(void);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

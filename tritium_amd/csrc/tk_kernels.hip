@@ -442,6 +442,35 @@ __device__ __forceinline__ RowConst load_row_const(const TkProblem &pr, int rowb
   return rc;
 }
 
+// One finished output of the int8 contract from the accumulator registers r of every plane.
+template <int P>
+__device__ __forceinline__ float int8_value(const v4i (&acc)[P], int r, const float (&sc)[P], const RowConst &rc,
+                                            bool has_act_scale) {
+  float f = 0.0f;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    float t = __fmul_rn((float)(acc[p][r] - rc.rs[r]), sc[p]);
+    f = p == 0 ? t : __fadd_rn(f, t);
+  }
+  if (has_act_scale) f = __fmul_rn(f, rc.as[r]);
+  return f;
+}
+
+// One finished output of the float contract: the four digit rows of a token recombined exactly.
+template <int P>
+__device__ __forceinline__ float digits_value(const v4i (&acc)[P], const float (&sc)[P], const RowConst &rc) {
+  float f = 0.0f;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    long long V = 0;
+#pragma unroll
+    for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(acc[p][r] - rc.rs[r]);
+    float t = __fmul_rn((float)ldexp((double)V, rc.exp), sc[p]);
+    f = p == 0 ? t : __fadd_rn(f, t);
+  }
+  return f;
+}
+
 // Finish one lane's 4 accumulator registers for every plane, with preloaded constants. Rows that
 // take the exact fallback are left alone here: exact_rows() writes them afterwards.
 template <int P>
@@ -460,28 +489,12 @@ __device__ __forceinline__ void flow_epilogue(const TkProblem &pr, int n, int ro
     for (int r = 0; r < 4; ++r) {
       const int m = rowbase + r;
       if (m >= pr.R || (rc.flag & (1u << r))) continue;
-      float f = 0.0f;
-#pragma unroll
-      for (int p = 0; p < P; ++p) {
-        float t = __fmul_rn((float)(acc[p][r] - rc.rs[r]), sc[p]);
-        f = p == 0 ? t : __fadd_rn(f, t);
-      }
-      if (pr.act_scale) f = __fmul_rn(f, rc.as[r]);
-      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, int8_value<P>(acc, r, sc, rc, pr.act_scale != nullptr));
     }
   } else {
     const int tok = rowbase >> 2;
     if (tok >= pr.M || rc.flag) return;
-    float f = 0.0f;
-#pragma unroll
-    for (int p = 0; p < P; ++p) {
-      long long V = 0;
-#pragma unroll
-      for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(acc[p][r] - rc.rs[r]);
-      float t = __fmul_rn((float)ldexp((double)V, rc.exp), sc[p]);
-      f = p == 0 ? t : __fadd_rn(f, t);
-    }
-    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, digits_value<P>(acc, sc, rc));
   }
 }
 
@@ -673,11 +686,19 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
 #define TK_GEMM_OCC 3
 #endif
 
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding: vmcnt[3:0] | [15:14])
+#define TK_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
+template <int P, int NT>
+__device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)[4][NT * P], uint8_t *smem, int tid, int bm,
+                                                 int bn);
+
 template <int P, int NT>
 __global__ __launch_bounds__(TK_GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(TK_GEMM_OCC, TK_GEMM_OCC))) void
 tk_gemm_kernel(const TkProblem pr) {
-  constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, PER_T = A4 / TK_GEMM_THREADS, NB = NT * P;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, NB = NT * P;
+  constexpr int SEGS = 16 / TK_GEMM_WAVES;  // 1-KiB A segments (one (j,g) pair x 64 rows) per wave per block
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // three A blocks of 16 KiB
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int i = lane & 15, g = lane >> 4;
   const int nb = pr.nb, R = pr.R;
@@ -690,22 +711,44 @@ tk_gemm_kernel(const TkProblem pr) {
   if (bm >= pr.grid_m || bn >= pr.grid_n) return;
   const int row0 = bm * ROWS;
   const int tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
-  uint4 *lds4 = (uint4 *)smem;
-  const uint4 *ap4 = (const uint4 *)pr.ap;
 
   // weight chunk offsets inside a plane (tiles past the end re-read the last tile; results dropped)
   unsigned woff[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) woff[nt] = ((unsigned)min(tile0 + nt, pr.n_tiles - 1) * (unsigned)nb * 64u + lane) * 16u;
-  // this thread's share of an A block
-  int a_src[PER_T];
-  bool a_ok[PER_T];
+
+  // A rows travel global -> LDS directly (no registers): one wave-wide 16-byte-per-lane load lands
+  // as 1 KiB at a wave-uniform LDS address, which is exactly one (j,g) segment of 64 rows. Rows past
+  // R are clamped to the last row (their results are never stored).
+  const unsigned a_lane = (unsigned)min(row0 + lane, R - 1) * 16u;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto dma_block = [&](int kb, int slot3) {
 #pragma unroll
-  for (int u = 0; u < PER_T; ++u) {
-    const int idx = threadIdx.x + u * TK_GEMM_THREADS;
-    const int seg = idx / ROWS, rr = idx % ROWS;
-    a_ok[u] = row0 + rr < R;
-    a_src[u] = seg * R + row0 + rr;
+    for (int u = 0; u < SEGS; ++u) {
+      const int seg = wave_u * SEGS + u;
+      const uint8_t *seg_base = (const uint8_t *)pr.ap + ((size_t)kb * 16 + seg) * (size_t)pr.rs * 16;  // wave-uniform
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(seg_base + a_lane),
+                                       (__attribute__((address_space(3))) void *)(smem + ((size_t)slot3 * A4 + (size_t)seg * ROWS) * 16),
+                                       16, 0, 0);
+    }
+  };
+
+  // Per-row constants of the tile (row sums, activation scales or grid exponents, fallback flags)
+  // travel to LDS by DMA now, one kind per wave, into 1 KiB past the A slots: the epilogue reads
+  // them from there, so they neither wait on memory then nor occupy registers during the main loop.
+  // Indices past the end are clamped; what is read for them is never used.
+  constexpr int CST = 3 * A4 * 16;  // int rs[64] | float as[64] | int exp[64] | uint flag[64]
+  {
+    const bool int8_in = pr.mode == TK_MODE_INT8;
+    const int row_c = min(row0 + lane, R - 1), tok_c = min((row0 >> 2) + lane, pr.M - 1);
+    const void *src = nullptr;
+    if (wave_u == 0) src = pr.rowsum + row_c;
+    else if (wave_u == 1) src = (int8_in && pr.act_scale) ? (const void *)(pr.act_scale + row_c) : nullptr;
+    else if (wave_u == 2) src = int8_in ? nullptr : (const void *)(pr.exps + tok_c);
+    else if (wave_u == 3) src = pr.flags ? (const void *)(pr.flags + (int8_in ? row_c : tok_c)) : nullptr;
+    if (src && wave_u < 4)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                       (__attribute__((address_space(3))) void *)(smem + CST + wave_u * 256), 4, 0, 0);
   }
 
   v4i acc[RT][NB];
@@ -714,87 +757,229 @@ tk_gemm_kernel(const TkProblem pr) {
 #pragma unroll
     for (int x = 0; x < NB; ++x) acc[rt][x] = v4i{0, 0, 0, 0};
 
-  uint4 wc[NB], wn[NB], areg[PER_T];
-  if (nb > 0) {
+  // The operand loads of the main loop are written as asm, with explicit waits. The compiler's own
+  // wait insertion cannot keep loads in flight across this loop: it does not see that an LDS read
+  // of slot `cur` never aliases the DMA into another slot, and with DMA and register loads pending
+  // together it drains the whole vector-memory counter at the first use of a loaded register --
+  // right after the prefetches were issued. An empty asm with a "+v" operand after each wait ties
+  // every later use of a loaded register to that wait.
+  // one address register for every read: slot, k step and row tile all sit in the 16-bit offset field
+  auto lds_read = [&](v4i (&a)[RT], unsigned addr, int off) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[rt]) : "v"(addr), "n"(off + rt * 256));
+  };
+  auto lds_wait = [&](v4i (&a)[RT]) {
+    asm volatile("s_waitcnt lgkmcnt(0)");
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) asm volatile("" : "+v"(a[rt]));
+  };
+  auto load_w = [&](v4i (&w)[NB], int kb) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int p = 0; p < P; ++p) wc[nt * P + p] = *(const uint4 *)(pr.codes[p] + woff[nt]);
+      for (int p = 0; p < P; ++p)
+        asm volatile("global_load_dwordx4 %0, %1, %2"
+                     : "=v"(w[nt * P + p])
+                     : "v"(woff[nt] + (unsigned)kb * (unsigned)TK_CHUNK_BYTES), "s"(pr.codes[p]));
+  };
+  auto tie_w = [&](v4i (&w)[NB]) {
 #pragma unroll
-    for (int u = 0; u < PER_T; ++u) {
-      uint4 q = make_uint4(0, 0, 0, 0);
-      if (a_ok[u]) q = ap4[a_src[u]];
-      lds4[threadIdx.x + u * TK_GEMM_THREADS] = q;
-    }
-  }
-  __syncthreads();
+    for (int x = 0; x < NB; ++x) asm volatile("" : "+v"(w[x]));
+  };
 
-  for (int kb = 0; kb < nb; ++kb) {
-    const bool more = kb + 1 < nb;
-    if (more) {
+  // Prefetch distance is two blocks for both operands: at the top of block kb the weight chunks and
+  // the A DMA of block kb+2 are issued; by the end of block kb everything of block kb+1 has landed.
+  v4i wc[NB], wn[NB], wf[NB];
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int p = 0; p < P; ++p)
-          wn[nt * P + p] = *(const uint4 *)(pr.codes[p] + woff[nt] + (size_t)(kb + 1) * TK_CHUNK_BYTES);
-#pragma unroll
-      for (int u = 0; u < PER_T; ++u) {
-        areg[u] = make_uint4(0, 0, 0, 0);
-        if (a_ok[u]) areg[u] = ap4[(size_t)(kb + 1) * 16 * R + a_src[u]];
-      }
+  for (int x = 0; x < NB; ++x) wc[x] = wn[x] = wf[x] = v4i{0, 0, 0, 0};
+  if (nb > 0) {
+    load_w(wc, 0);
+    dma_block(0, 0);
+    if (nb > 1) {
+      load_w(wn, 1);
+      dma_block(1, 1);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SEGS + NB));  // block 0 has landed; block 1 may be in flight
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)");
     }
-    const uint4 *buf = lds4 + (kb & 1) * A4;
+    tie_w(wc);
+  }
+  __builtin_amdgcn_s_barrier();
+
+  const unsigned lds_lane = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t *)smem + (unsigned)(g * ROWS + i) * 16u;
+  // One block: `w` holds its weight chunks, `w1` those of block kb+1 (in flight or landed), `w2` is
+  // free and receives block kb+2. The three register sets and the three LDS slots rotate by name
+  // (the loop below is unrolled by three), never by copying: a register with a load in flight must
+  // not be read.
+  auto block = [&](v4i (&w)[NB], v4i (&w1)[NB], v4i (&w2)[NB], int kb, int cur) {
+    const bool more2 = kb + 2 < nb;
+    const int nxt2 = cur == 0 ? 2 : cur - 1;  // slot of block kb+2 == slot of block kb-1, free since the last barrier
+    if (more2) {
+      load_w(w2, kb + 2);
+      dma_block(kb + 2, nxt2);
+    }
+    v4i a[RT];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      v4i a[RT];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const uint4 q = buf[(j * 4 + g) * ROWS + rt * 16 + i];
-        a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
-      }
+      lds_read(a, lds_lane, cur * (A4 * 16) + j * (4 * ROWS * 16));
+      lds_wait(a);
 #pragma unroll
       for (int x = 0; x < NB; ++x) {
-        const uint32_t wj = j == 0 ? wc[x].x : (j == 1 ? wc[x].y : (j == 2 ? wc[x].z : wc[x].w));
-        const v4i b = expand_codes(wj);
+        const v4i b = expand_codes((uint32_t)w[x][j]);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
           acc[rt][x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[rt][x], 0, 0, 0);
       }
     }
-    if (more) {
-      uint4 *nbuf = lds4 + ((kb + 1) & 1) * A4;
-#pragma unroll
-      for (int u = 0; u < PER_T; ++u) nbuf[threadIdx.x + u * TK_GEMM_THREADS] = areg[u];
-#pragma unroll
-      for (int x = 0; x < NB; ++x) wc[x] = wn[x];
-    }
-    __syncthreads();
+    // Everything of block kb+1 (issued one block ago) must have landed before the barrier lets anyone
+    // read it; the loads of block kb+2, the youngest of this wave, stay in flight.
+    if (more2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SEGS + NB)); else asm volatile("s_waitcnt vmcnt(0)");
+    tie_w(w1);
+    __builtin_amdgcn_s_barrier();
+  };
+  int kb = 0;
+  for (; kb + 3 <= nb; kb += 3) {  // one exit only: the accumulators keep their registers
+    block(wc, wn, wf, kb, 0);
+    block(wn, wf, wc, kb + 1, 1);
+    block(wf, wc, wn, kb + 2, 2);
+  }
+  if (kb < nb) {
+    block(wc, wn, wf, kb, 0);
+    if (kb + 1 < nb) block(wn, wf, wc, kb + 1, 1);
   }
 
-  RowConst rc[RT];
-  unsigned any_flag = 0;
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    rc[rt] = load_row_const(pr, row0 + rt * 16 + 4 * g);
-    any_flag |= rc[rt].flag;
+  // The epilogue derives its lane coordinates afresh from a laundered thread id: sharing them with
+  // the prologue would keep a dozen registers alive across the main loop, which has none to spare.
+  unsigned tid_e = threadIdx.x;
+  asm volatile("" : "+v"(tid_e));
+  tk_gemm_epilogue<P, NT>(pr, acc, smem, (int)tid_e, bm, bn);
+}
+
+template <int P, int NT>
+__device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)[4][NT * P], uint8_t *smem, int tid, int bm,
+                                                 int bn) {
+  constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, CST = 3 * A4 * 16;
+  const int wave = tid >> 6, lane = tid & 63, i = lane & 15, g = lane >> 4;
+  const int R = pr.R, row0 = bm * ROWS, tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+  // Epilogue. The row constants are in LDS since the prologue: one 16-byte read per row tile.
+  const int *cst_rs = (const int *)(smem + CST);
+  const float *cst_as = (const float *)(smem + CST + 256);
+  const int *cst_exp = (const int *)(smem + CST + 512);
+  const int *cst_flag = (const int *)(smem + CST + 768);
+  unsigned my_flag = 0;
+  if (pr.flags && tid < ROWS) {
+    const bool in_range = pr.mode == TK_MODE_INT8 ? row0 + tid < R : (row0 >> 2) + tid < pr.M;
+    if (in_range) my_flag = cst_flag[tid] ? 1u : 0u;
   }
+  float sc[NT][P];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const int t = tile0 + nt;
-    const int n = t * 16 + i;
-    if (t >= pr.n_tiles || n >= pr.n) continue;
-    float sc[P];
+    const int n = (tile0 + nt) * 16 + i;
 #pragma unroll
-    for (int p = 0; p < P; ++p) sc[p] = pr.scales[p][n];
+    for (int p = 0; p < P; ++p) sc[nt][p] = (tile0 + nt < pr.n_tiles && n < pr.n) ? pr.scales[p][n] : 0.0f;
+  }
+  const int wg_flag = __syncthreads_or((int)my_flag);
+  auto row_const = [&](int rt) {
+    RowConst rc;
+    const v4i rs4 = *(const v4i *)(cst_rs + rt * 16 + 4 * g);
+    const float4 as4 = *(const float4 *)(cst_as + rt * 16 + 4 * g);
+    rc.rs[0] = rs4.x; rc.rs[1] = rs4.y; rc.rs[2] = rs4.z; rc.rs[3] = rs4.w;
+    rc.as[0] = as4.x; rc.as[1] = as4.y; rc.as[2] = as4.z; rc.as[3] = as4.w;
+    rc.exp = cst_exp[rt * 4 + g];
+    rc.flag = 0;
+    if (wg_flag) {
+      if (pr.mode == TK_MODE_INT8) {
+        const v4i f4 = *(const v4i *)(cst_flag + rt * 16 + 4 * g);
+        rc.flag = (f4.x ? 1u : 0u) | (f4.y ? 2u : 0u) | (f4.z ? 4u : 0u) | (f4.w ? 8u : 0u);
+      } else {
+        rc.flag = cst_flag[rt * 4 + g] ? 1u : 0u;
+      }
+    }
+    return rc;
+  };
+
+  // The MFMA result layout gives a lane 16 outputs of one column, four rows apart, so a direct
+  // store instruction writes 32-byte pieces of four different output rows. When the rows of the
+  // output are 16-byte aligned, the finished values are staged through LDS instead (free after the
+  // last barrier of the main loop) and leave as whole 16-byte pieces of contiguous row segments:
+  // every store instruction of a wave then covers full cache lines.
+  const int esz = pr.out_dtype == TK_BF16 ? 2 : 4;
+  const bool staged = (((size_t)pr.n * esz) & 15) == 0 && (((size_t)pr.out) & 15) == 0;
+  if (staged) {
+    constexpr int WG_COLS = TK_GEMM_WAVES * NT * 16;
+    const bool int8_mode = pr.mode == TK_MODE_INT8 || pr.out_dtype == TK_I32;
+    const int halves = esz == 4 ? 2 : 1;            // 4-byte outputs take the 64 rows in two halves
+    const int rt_per_half = RT / halves;
+    const int orows_rt = int8_mode ? 16 : 4;        // output rows per row tile (4 digit rows = 1 token)
+    const int stride = WG_COLS * esz + 16;          // padded: the 4 lane groups of a wave hit different banks
+    const int pieces_row = WG_COLS * esz / 16;      // 16-byte pieces per staged row (a power of two)
+    const int out_row0 = int8_mode ? row0 : (row0 >> 2);
+    const int out_rows = int8_mode ? pr.R : pr.M;
+    const int col0 = bn * WG_COLS;
+    const bool has_as = pr.act_scale != nullptr;
+    for (int h = 0; h < halves; ++h) {
+      if (h > 0) __syncthreads();
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (rt / rt_per_half != h) continue;
+        const int rl = rt - h * rt_per_half;
+        const RowConst rc = row_const(rt);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const int cl = (wave * NT + nt) * 16 + i;
+          v4i av[P];
+#pragma unroll
+          for (int p = 0; p < P; ++p) av[p] = acc[rt][nt * P + p];
+          if (pr.out_dtype == TK_I32) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              *(int32_t *)(smem + (size_t)(rl * 16 + 4 * g + r) * stride + cl * 4) = av[0][r] - rc.rs[r];
+          } else if (pr.mode == TK_MODE_INT8) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float f = int8_value<P>(av, r, sc[nt], rc, has_as);
+              uint8_t *dst = smem + (size_t)(rl * 16 + 4 * g + r) * stride + cl * esz;
+              if (esz == 2) *(uint16_t *)dst = f32_to_bf16_rne(f); else *(float *)dst = f;
+            }
+          } else {
+            const float f = digits_value<P>(av, sc[nt], rc);
+            uint8_t *dst = smem + (size_t)(rl * 4 + g) * stride + cl * esz;
+            if (esz == 2) *(uint16_t *)dst = f32_to_bf16_rne(f); else *(float *)dst = f;
+          }
+        }
+      }
+      __syncthreads();
+      const int rows_h = rt_per_half * orows_rt;
+      const int per16 = 16 / esz;
+      for (int pc = tid; pc < rows_h * pieces_row; pc += TK_GEMM_THREADS) {
+        const int rl = pc / pieces_row, piece = pc - rl * pieces_row;
+        const int orow = out_row0 + h * rows_h + rl;
+        const int c = col0 + piece * per16;
+        if (orow >= out_rows || c >= pr.n) continue;
+        if (wg_flag && pr.out_dtype != TK_I32 && pr.flags[orow]) continue;  // written by exact_rows below
+        const uint8_t *src = smem + (size_t)rl * stride + piece * 16;
+        uint8_t *dst = (uint8_t *)pr.out + ((size_t)orow * pr.n + c) * esz;
+        *(uint4 *)dst = *(const uint4 *)src;  // n is a multiple of per16 here, so a piece never straddles the row end
+      }
+    }
+  } else {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      v4i av[P];
+      const RowConst rc = row_const(rt);
 #pragma unroll
-      for (int p = 0; p < P; ++p) av[p] = acc[rt][nt * P + p];
-      flow_epilogue<P>(pr, n, row0 + rt * 16 + 4 * g, av, sc, rc[rt]);
+      for (int nt = 0; nt < NT; ++nt) {
+        const int t = tile0 + nt;
+        const int n = t * 16 + i;
+        if (t >= pr.n_tiles || n >= pr.n) continue;
+        v4i av[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) av[p] = acc[rt][nt * P + p];
+        flow_epilogue<P>(pr, n, row0 + rt * 16 + 4 * g, av, sc[nt], rc);
+      }
     }
   }
-  if (any_flag) {
+  if (wg_flag) {
     for (int nt = 0; nt < NT; ++nt) {
       const int t = tile0 + nt;
       const int n = t * 16 + i;
@@ -960,7 +1145,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
   __shared__ int shi[4];
   int rowi;
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
-  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.R;
+  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = row * k;
   float gamma;
   int nonfinite;
@@ -1000,7 +1185,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
   __shared__ int shi[4];
   int rowi;
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
-  const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.R;
+  const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = tok * k;
   float gamma;
   int nonfinite;
@@ -1044,7 +1229,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_i8_kernel(TkPrep single, const 
   __shared__ int shi[4];
   int rowi;
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
-  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.R;
+  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const int8_t *q = (const int8_t *)pp.act;
   const size_t base = row * k;
   int sum = 0;
@@ -1235,6 +1420,7 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
 }
 
 // output tiles per workgroup of the GEMM for a plane count
+int tk_gemm_lds_bytes(void) { return 3 * 16 * 64 * 16 + 1024; }  // three A blocks + the row constants
 int tk_gemm_tiles_per_wg(int planes) { return TK_GEMM_WAVES * (planes == 1 ? 4 : (planes == 2 ? 2 : 1)); }
 
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
