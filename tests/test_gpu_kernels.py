@@ -311,6 +311,37 @@ def test_gemm_epilogue_variants(backend, oracle, m, n, k, decode_kernel):
     layer.free()
 
 
+@pytest.mark.parametrize("nb", [1, 2, 3, 4, 5, 6, 7, 9, 27])
+@pytest.mark.parametrize("planes", [1, 2])
+def test_flow_runs_of_several_tiles(backend, oracle, nb, planes, decode_kernel):
+    """A wave of the flow kernel walks runs of consecutive tiles as one stream behind a prefetch
+    ring; every K block count relative to the ring size, runs of 2 and 5 tiles, ragged last run."""
+    if decode_kernel != "flow":
+        pytest.skip("flow kernel only")
+    k = nb * 256 - 13
+    n = 16 * 37 + 5
+    rng = np.random.default_rng(1000 + nb * 10 + planes)
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7)[:planes]]
+    scs = [np.ones(n, np.float32) for _ in range(planes)]
+    packed, layer = _layer(backend, oracle, ws, scs)
+    try:
+        for run_tiles in (2, 5):
+            backend.set_flow_run_tiles(run_tiles)
+            for m in (1, 16):
+                print("case flow-runs", nb, planes, run_tiles, m, flush=True)
+                q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+                dq, dout = backend.to_device(q, "i8"), backend.empty(m * n, "f32")
+                backend.linear_i8(layer, dq, None, m, dout)
+                got = dout.to_host().reshape(m, n)
+                want = sum(q.astype(np.int32) @ w.T.astype(np.int32) for w in ws).astype(np.float32)
+                assert same_bits(got, want)  # exact: the sums stay far below 2^24
+                dq.free()
+                dout.free()
+    finally:
+        backend.set_flow_run_tiles(0)
+        layer.free()
+
+
 def test_group_launch_equals_single_launches(backend, oracle):
     rng = np.random.default_rng(29)
     k = 768

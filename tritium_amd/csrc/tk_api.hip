@@ -582,6 +582,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.grid = flow_groups;
     cfg.lds_bytes = pl.flow_lds;
     cfg.waves = flow_waves(pl.flow_lds);
+    cfg.ring = tk_flow_ring(&pr.nb, nullptr, 1);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -937,6 +938,15 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
   g->cfg.grid = variant == DECODE_KSPLIT ? tiles : groups_total;
   g->cfg.waves = fw;
+  {
+    std::vector<int> nbs(count);
+    std::vector<double> wts(count);
+    for (size_t i = 0; i < count; ++i) {
+      nbs[i] = plans[i].pr.nb;
+      wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
+    }
+    g->cfg.ring = tk_flow_ring(nbs.data(), wts.data(), (int)count);
+  }
   *out = g;
   return TK_OK;
 }

@@ -21,13 +21,6 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 #define TK_WG 256
-// prefetch ring depth of the flow kernel, in K blocks: narrow (planes*runs < 4) and wide streams
-#ifndef TK_FLOW_DEPTH
-#define TK_FLOW_DEPTH 4
-#endif
-#ifndef TK_FLOW_DEPTH_WIDE
-#define TK_FLOW_DEPTH_WIDE 2
-#endif
 
 // ------------------------------------------------------------------------------------------
 // small helpers
@@ -42,15 +35,33 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
   return (uint16_t)(u >> 16);
 }
 
+// Every pointer a kernel receives is device memory. Where the compiler cannot see that (a pointer
+// read from a problem table), it would emit flat accesses, which also count on the LDS counter and
+// serialise against LDS reads; these helpers state the address space.
+#define TK_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ T gload(const T *p) {
+  return *(const TK_GLOBAL T *)p;
+}
+template <typename T>
+__device__ __forceinline__ void gstore(T *p, T v) {
+  *(TK_GLOBAL T *)p = v;
+}
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 gload16(const void *p) {
+  const v4u v = *(const TK_GLOBAL v4u *)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ __forceinline__ float load_act(const void *p, int dtype, size_t idx) {
-  return dtype == TK_BF16 ? bf16_to_f32(((const uint16_t *)p)[idx]) : ((const float *)p)[idx];
+  return dtype == TK_BF16 ? bf16_to_f32(gload((const uint16_t *)p + idx)) : gload((const float *)p + idx);
 }
 
 __device__ __forceinline__ void store_out(void *out, int dtype, size_t idx, float v) {
   if (dtype == TK_BF16)
-    ((uint16_t *)out)[idx] = f32_to_bf16_rne(v);
+    gstore((uint16_t *)out + idx, f32_to_bf16_rne(v));
   else
-    ((float *)out)[idx] = v;
+    gstore((float *)out + idx, v);
 }
 
 __device__ __forceinline__ v4i expand_codes(uint32_t w) {
@@ -392,6 +403,31 @@ __global__ __launch_bounds__(TK_WG) void tk_stream_kernel(TkProblem single, cons
 // epilogue of a tile waits on nothing that was issued behind the stream's prefetches.
 // ------------------------------------------------------------------------------------------
 
+// The fields of a problem that the epilogues read, copied into registers once per kernel: read through
+// a pointer into a problem table they would be fetched again after every store.
+struct TkHot {
+  void *out;
+  const int32_t *rowsum;
+  const float *act_scale;
+  const int32_t *exps;
+  const uint32_t *flags;
+  int n, R, M, mode, out_dtype;
+};
+__device__ __forceinline__ TkHot make_hot(const TkProblem &pr) {
+  TkHot h;
+  h.out = pr.out;
+  h.rowsum = pr.rowsum;
+  h.act_scale = pr.act_scale;
+  h.exps = pr.exps;
+  h.flags = pr.flags;
+  h.n = pr.n;
+  h.R = pr.R;
+  h.M = pr.M;
+  h.mode = pr.mode;
+  h.out_dtype = pr.out_dtype;
+  return h;
+}
+
 struct RowConst {
   int rs[4];       // row sums of the 4 operand rows this lane finishes
   float as[4];     // INT8: per-token activation scale (1.0 when absent)
@@ -405,22 +441,23 @@ __device__ __forceinline__ unsigned row_flags(const TkProblem &pr, int rowbase) 
   if (!pr.flags) return 0;
   if (pr.mode == TK_MODE_INT8) {
     for (int r = 0; r < 4; ++r)
-      if (rowbase + r < pr.R && pr.flags[rowbase + r]) fl |= 1u << r;
+      if (rowbase + r < pr.R && gload(pr.flags + rowbase + r)) fl |= 1u << r;
   } else {
     const int tok = rowbase >> 2;
-    if (tok < pr.M && pr.flags[tok]) fl = 1u;
+    if (tok < pr.M && gload(pr.flags + tok)) fl = 1u;
   }
   return fl;
 }
 
-__device__ __forceinline__ RowConst load_row_const(const TkProblem &pr, int rowbase) {
+template <typename PR>
+__device__ __forceinline__ RowConst load_row_const(const PR &pr, int rowbase) {
   RowConst rc;
   rc.exp = 0;
   rc.flag = 0;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int m = rowbase + r;
-    rc.rs[r] = m < pr.R ? pr.rowsum[m] : 0;
+    rc.rs[r] = m < pr.R ? gload(pr.rowsum + m) : 0;
     rc.as[r] = 1.0f;
   }
   if (pr.mode == TK_MODE_INT8) {
@@ -428,15 +465,15 @@ __device__ __forceinline__ RowConst load_row_const(const TkProblem &pr, int rowb
     for (int r = 0; r < 4; ++r) {
       const int m = rowbase + r;
       if (m < pr.R) {
-        if (pr.act_scale) rc.as[r] = pr.act_scale[m];
-        if (pr.flags && pr.flags[m]) rc.flag |= 1u << r;
+        if (pr.act_scale) rc.as[r] = gload(pr.act_scale + m);
+        if (pr.flags && gload(pr.flags + m)) rc.flag |= 1u << r;
       }
     }
   } else {
     const int tok = rowbase >> 2;
     if (tok < pr.M) {
-      rc.exp = pr.exps[tok];
-      if (pr.flags && pr.flags[tok]) rc.flag = 1u;
+      rc.exp = gload(pr.exps + tok);
+      if (pr.flags && gload(pr.flags + tok)) rc.flag = 1u;
     }
   }
   return rc;
@@ -462,10 +499,11 @@ __device__ __forceinline__ float digits_value(const v4i (&acc)[P], const float (
   float f = 0.0f;
 #pragma unroll
   for (int p = 0; p < P; ++p) {
-    long long V = 0;
+    // Horner in double: every step is exact (|digit sum| < 2^28 for K < 2^20, so |V| < 2^53)
+    double V = (double)(acc[p][3] - rc.rs[3]);
 #pragma unroll
-    for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(acc[p][r] - rc.rs[r]);
-    float t = __fmul_rn((float)ldexp((double)V, rc.exp), sc[p]);
+    for (int r = 2; r >= 0; --r) V = __builtin_fma(V, 256.0, (double)(acc[p][r] - rc.rs[r]));
+    float t = __fmul_rn((float)ldexp(V, rc.exp), sc[p]);
     f = p == 0 ? t : __fadd_rn(f, t);
   }
   return f;
@@ -473,14 +511,14 @@ __device__ __forceinline__ float digits_value(const v4i (&acc)[P], const float (
 
 // Finish one lane's 4 accumulator registers for every plane, with preloaded constants. Rows that
 // take the exact fallback are left alone here: exact_rows() writes them afterwards.
-template <int P>
-__device__ __forceinline__ void flow_epilogue(const TkProblem &pr, int n, int rowbase, const v4i (&acc)[P],
+template <int P, typename PR>
+__device__ __forceinline__ void flow_epilogue(const PR &pr, int n, int rowbase, const v4i (&acc)[P],
                                               const float (&sc)[P], const RowConst &rc) {
   if (pr.out_dtype == TK_I32) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = rowbase + r;
-      if (m < pr.R) ((int32_t *)pr.out)[(size_t)m * pr.n + n] = acc[0][r] - rc.rs[r];
+      if (m < pr.R) gstore((int32_t *)pr.out + (size_t)m * pr.n + n, acc[0][r] - rc.rs[r]);
     }
     return;
   }
@@ -525,66 +563,84 @@ __device__ __forceinline__ void exact_rows(const TkProblem &pr, int n, int rowba
   }
 }
 
-template <int P, int RT, int TW, int D, int NW, bool TABLE>
-__global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
-                                                        const int *__restrict__ wg_prob) {
+template <int P, int RT, int TW, int DR, bool TABLE>
+__global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+                                                      const int *__restrict__ wg_prob) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
+  const int NW = (int)(blockDim.x >> 6);  // 4 or 8 waves
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int i = lane & 15, g = lane >> 4;
-  const int nb = pr.nb, R = pr.R, S = pr.run_tiles;
-  const int nbpad = (nb + D - 1) / D * D;
-  const int first = ((blockIdx.x - pr.group_begin) * NW + wave) * TW * S;  // first tile of this wave
-  const unsigned last_chunk = (unsigned)pr.n_tiles * (unsigned)nb - 1u;   // clamp: stay inside the plane
-
-  // the stream position is a chunk index inside the plane; lane offset is added at the load
-  unsigned cbase[TW];
+  const int nb = pr.nb, R = pr.R, S = pr.run_tiles, n_tiles = pr.n_tiles;
+  // local copies: a field read through the table pointer would be fetched again after every store
+  const TkHot hot = make_hot(pr);
+  const uint8_t *codes[P];
+  const float *scales[P];
 #pragma unroll
-  for (int tw = 0; tw < TW; ++tw) cbase[tw] = (unsigned)(first + tw * S) * (unsigned)nb;
-
-  auto load_chunk = [&](int tw, int p, int s, int kb) -> uint4 {
-    unsigned c = cbase[tw] + (unsigned)s * (unsigned)nb + (unsigned)kb;
-    c = c < last_chunk ? c : last_chunk;
-    return *(const uint4 *)(pr.codes[p] + ((size_t)c * 64 + lane) * 16);
-  };
-
-  uint4 ring[D][TW][P];
-  if (nb > 0) {
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-      if (d < nb) {
-#pragma unroll
-        for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-          for (int p = 0; p < P; ++p) ring[d][tw][p] = load_chunk(tw, p, 0, d);
-      }
+  for (int p = 0; p < P; ++p) {
+    codes[p] = pr.codes[p];
+    scales[p] = pr.scales[p];
   }
+  // The weight stream of a run is walked in positions q = s*nbpad + kb, nbpad = nb rounded up to a
+  // multiple of the ring size DR (positions kb >= nb are padding: nothing is computed there). Slot =
+  // kb % DR. At EVERY position, padding included, the chunks D = DR-1 positions ahead are requested
+  // into the slot consumed one position ago: no register is copied, no chunk is overwritten before
+  // its use, and because each position issues the same number of loads the wait in front of a
+  // chunk's first use leaves exactly the D younger positions in flight. The chunks of a run are
+  // consecutive in memory, so a request is one running byte offset per run, advanced by 1 KiB when
+  // the requested position is a real one; a padding position asks again for the chunk the next real
+  // position will get, and requests past the end of the plane are clamped to its last chunk. The
+  // host picks DR so that padding is rare.
+  constexpr int D = DR - 1;
+  const int nbpad = (nb + DR - 1) / DR * DR;
+  const int first = ((blockIdx.x - pr.group_begin) * NW + wave) * TW * S;  // first tile of this wave
+  const unsigned last_off = ((unsigned)n_tiles * (unsigned)nb - 1u) * 1024u + (unsigned)lane * 16u;
+  unsigned roff[TW];  // byte offset inside a plane of this lane's piece of the next chunk to request
+#pragma unroll
+  for (int tw = 0; tw < TW; ++tw) roff[tw] = (unsigned)(first + tw * S) * (unsigned)nb * 1024u + (unsigned)lane * 16u;
+
+  uint4 ring[DR][TW][P];
+  auto request = [&](int slot, bool real) {
+#pragma unroll
+    for (int tw = 0; tw < TW; ++tw) {
+      const unsigned off = min(roff[tw], last_off);
+#pragma unroll
+      for (int p = 0; p < P; ++p) ring[slot][tw][p] = gload16(codes[p] + (size_t)off);
+      roff[tw] += real ? 1024u : 0u;
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) request(d, d < nb);
 
   // stage every operand row of the problem in LDS
   {
     const uint4 *ap4 = (const uint4 *)pr.ap;
     uint4 *lds4w = (uint4 *)smem;
     const int cnt = nb * 16 * R;
-    for (int idx = threadIdx.x; idx < cnt; idx += NW * 64) lds4w[idx] = ap4[idx];
+    for (int idx = threadIdx.x; idx < cnt; idx += (int)blockDim.x) lds4w[idx] = gload16(ap4 + idx);
   }
   RowConst rc[RT];
   unsigned any_flag = 0;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    rc[rt] = load_row_const(pr, rt * 16 + 4 * g);
+    rc[rt] = load_row_const(hot, rt * 16 + 4 * g);
     any_flag |= rc[rt].flag;
   }
   __syncthreads();
   const uint4 *lds4 = (const uint4 *)smem;
+  // operand rows past R re-read the last row: their results are never stored
+  int arow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) arow[rt] = min(rt * 16 + i, R - 1);
 
   for (int s = 0; s < S; ++s) {
     // per-tile scales, issued now, consumed in the epilogue
     float sc[TW][P];
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
-      const int n = min((first + tw * S + s) * 16 + i, pr.n - 1);
+      const int n = min((first + tw * S + s) * 16 + i, hot.n - 1);
 #pragma unroll
-      for (int p = 0; p < P; ++p) sc[tw][p] = pr.scales[p][n];
+      for (int p = 0; p < P; ++p) sc[tw][p] = gload(scales[p] + n);
     }
     v4i acc[TW][RT][P];
 #pragma unroll
@@ -594,42 +650,29 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
 #pragma unroll
         for (int p = 0; p < P; ++p) acc[tw][rt][p] = v4i{0, 0, 0, 0};
 
-    for (int kbg = 0; kbg < nbpad; kbg += D) {
+    for (int kbg = 0; kbg < nbpad; kbg += DR) {
 #pragma unroll
-      for (int d = 0; d < D; ++d) {
+      for (int d = 0; d < DR; ++d) {
         const int kb = kbg + d;
+        {  // request the position D ahead (slot (d + D) % DR, consumed at the previous position)
+          int kb2 = kb + D;
+          if (kb2 >= nbpad) kb2 -= nbpad;
+          request((d + D) % DR, kb2 < nb);
+        }
         if (kb < nb) {
-          uint4 cur[TW][P];
-#pragma unroll
-          for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-            for (int p = 0; p < P; ++p) cur[tw][p] = ring[d][tw][p];
-          // refill this ring slot with the chunk D positions ahead in the padded stream
-          {
-            int kb2 = kb + D, s2 = s;
-            if (kb2 >= nbpad) { kb2 -= nbpad; s2 += 1; }
-            if (kb2 < nb && s2 < S) {
-#pragma unroll
-              for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-                for (int p = 0; p < P; ++p) ring[d][tw][p] = load_chunk(tw, p, s2, kb2);
-            }
-          }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             v4i a[RT];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-              const int row = rt * 16 + i;
-              uint4 q = make_uint4(0, 0, 0, 0);
-              if (row < R) q = lds4[((kb * 4 + j) * 4 + g) * R + row];
+              const uint4 q = lds4[((kb * 4 + j) * 4 + g) * R + arow[rt]];
               a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
             }
 #pragma unroll
             for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
               for (int p = 0; p < P; ++p) {
-                const uint4 w = cur[tw][p];
+                const uint4 w = ring[d][tw][p];
                 const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
                 const v4i b = expand_codes(wj);
 #pragma unroll
@@ -645,9 +688,9 @@ __global__ __launch_bounds__(NW * 64) void tk_flow_kernel(const TkProblem single
     for (int tw = 0; tw < TW; ++tw) {
       const int t = first + tw * S + s;
       const int n = t * 16 + i;
-      if (t < pr.n_tiles && n < pr.n) {
+      if (t < n_tiles && n < hot.n) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) flow_epilogue<P>(pr, n, rt * 16 + 4 * g, acc[tw][rt], sc[tw], rc[rt]);
+        for (int rt = 0; rt < RT; ++rt) flow_epilogue<P>(hot, n, rt * 16 + 4 * g, acc[tw][rt], sc[tw], rc[rt]);
       }
     }
     if (any_flag) {
@@ -1364,14 +1407,14 @@ static hipError_t flow_launch_one(K kernel, hipStream_t s, const TkProblem &sg, 
                                   const int *wg_prob, const TkLaunchCfg &cfg, int threads) {
   if (cfg.lds_bytes > 64 * 1024) {
     // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    static thread_local const void *raised[64];
+    static thread_local const void *raised[128];
     static thread_local int nraised = 0;
     bool done = false;
     for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
     if (!done) {
       hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
-      if (nraised < 64) raised[nraised++] = (const void *)kernel;
+      if (nraised < 128) raised[nraised++] = (const void *)kernel;
     }
   }
   hipLaunchKernelGGL(kernel, dim3(cfg.grid), dim3(threads), cfg.lds_bytes, s, sg, table, wg_prob);
@@ -1382,13 +1425,19 @@ template <int P, int RT>
 static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                  const TkLaunchCfg &cfg) {
   constexpr int TW = (RT >= 4 && P <= 2) ? 2 : 1;
-  constexpr int D = (P * TW >= 4) ? TK_FLOW_DEPTH_WIDE : TK_FLOW_DEPTH;
-  if (cfg.waves == 8) {
-    if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 8, true>, s, sg, table, wg_prob, cfg, 512);
-    return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 8, false>, s, sg, table, wg_prob, cfg, 512);
+  const int threads = cfg.waves * 64;
+  switch (cfg.ring) {
+    case 3:
+      if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, 3, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow_kernel<P, RT, TW, 3, false>, s, sg, table, wg_prob, cfg, threads);
+    case 4:
+      if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, 4, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow_kernel<P, RT, TW, 4, false>, s, sg, table, wg_prob, cfg, threads);
+    case 5:
+      if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, 5, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow_kernel<P, RT, TW, 5, false>, s, sg, table, wg_prob, cfg, threads);
+    default: return hipErrorInvalidValue;
   }
-  if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 4, true>, s, sg, table, wg_prob, cfg, 256);
-  return flow_launch_one(tk_flow_kernel<P, RT, TW, D, 4, false>, s, sg, table, wg_prob, cfg, 256);
 }
 
 template <int P>
@@ -1404,6 +1453,27 @@ static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProb
 
 // lock-step runs per wave of the flow kernel for a (planes, rt) pair
 int tk_flow_runs_per_wave(int planes, int rt) { return (rt >= 4 && planes <= 2) ? 2 : 1; }
+
+// Ring size of the flow kernel for launches whose K block counts are nbs[0..count): the compiled
+// size (3, 4 or 5 positions) that pads the fewest positions, weighted by each problem's chunk count;
+// ties go to the deeper ring.
+int tk_flow_ring(const int *nbs, const double *weights, int count) {
+  int best = 4;
+  double best_waste = -1.0;
+  const int cand[3] = {5, 4, 3};
+  for (int c = 0; c < 3; ++c) {
+    double waste = 0.0;
+    for (int x = 0; x < count; ++x) {
+      const int nb = nbs[x], pad = (nb + cand[c] - 1) / cand[c] * cand[c];
+      waste += (weights ? weights[x] : 1.0) * (double)(pad - nb) / (double)(nb > 0 ? nb : 1);
+    }
+    if (best_waste < 0.0 || waste < best_waste - 1e-12) {
+      best_waste = waste;
+      best = cand[c];
+    }
+  }
+  return best;
+}
 
 hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg) {
