@@ -115,6 +115,22 @@ __device__ __forceinline__ float seq_dot(const TkProblem &pr, int p, int n, int 
 
 // Fold one plane's accumulators of one lane (4 consecutive operand rows starting at rowbase,
 // output column n) into the running float outputs.
+// The four digit rows of a token recombined: V = x3*2^24 + x2*2^16 + x1*2^8 + x0 (exact integers
+// x_r = sum of trit*digit, |x_r| <= 128*K), scaled by the token's grid exponent. Three
+// single-precision FMAs: the pairs (x3,x2) and (x1,x0) first, then their combination. The high pair
+// is a multiple of 2^16 and the low pair is below 2^33, so whenever the two nearly cancel the high
+// pair is small enough to be exact; otherwise the result has the magnitude of the high pair and each
+// rounding is half an ulp of it: the value returned is within 1.5 ulp of the exact dot product (and
+// equal to it when that is representable, e.g. for integer-valued activations), where a k-ordered
+// f32 accumulation drifts by ~sqrt(K) ulp. Every kernel finishes through this one function, so
+// their float results are bit-identical to each other. Double precision would round once, but runs
+// at a fraction of the rate, and this sits on the decode path of every output.
+__device__ __forceinline__ float digits_to_float(int x3, int x2, int x1, int x0, int exp) {
+  const float hi = __builtin_fmaf((float)x3, 256.0f, (float)x2);
+  const float lo = __builtin_fmaf((float)x1, 256.0f, (float)x0);
+  return ldexpf(__builtin_fmaf(hi, 65536.0f, lo), exp);
+}
+
 __device__ __forceinline__ void fold_plane(const TkProblem &pr, int p, int n, int rowbase, v4i v,
                                            float out[4], bool first) {
   const float sc = pr.scales[p][n];
@@ -130,10 +146,8 @@ __device__ __forceinline__ void fold_plane(const TkProblem &pr, int p, int n, in
   } else {
     int tok = rowbase >> 2;
     if (tok < pr.M) {
-      long long V = 0;
-#pragma unroll
-      for (int r = 3; r >= 0; --r) V = V * 256 + (long long)(v[r] - pr.rowsum[rowbase + r]);
-      float val = (float)ldexp((double)V, pr.exps[tok]);
+      const int32_t *rs = pr.rowsum + rowbase;
+      float val = digits_to_float(v[3] - rs[3], v[2] - rs[2], v[1] - rs[1], v[0] - rs[0], pr.exps[tok]);
       float f = __fmul_rn(val, sc);
       out[0] = first ? f : __fadd_rn(out[0], f);
     }
@@ -493,17 +507,15 @@ __device__ __forceinline__ float int8_value(const v4i (&acc)[P], int r, const fl
   return f;
 }
 
-// One finished output of the float contract: the four digit rows of a token recombined exactly.
+// One finished output of the float contract from the accumulator registers of every plane.
 template <int P>
 __device__ __forceinline__ float digits_value(const v4i (&acc)[P], const float (&sc)[P], const RowConst &rc) {
   float f = 0.0f;
 #pragma unroll
   for (int p = 0; p < P; ++p) {
-    // Horner in double: every step is exact (|digit sum| < 2^28 for K < 2^20, so |V| < 2^53)
-    double V = (double)(acc[p][3] - rc.rs[3]);
-#pragma unroll
-    for (int r = 2; r >= 0; --r) V = __builtin_fma(V, 256.0, (double)(acc[p][r] - rc.rs[r]));
-    float t = __fmul_rn((float)ldexp(V, rc.exp), sc[p]);
+    const float val = digits_to_float(acc[p][3] - rc.rs[3], acc[p][2] - rc.rs[2], acc[p][1] - rc.rs[1],
+                                      acc[p][0] - rc.rs[0], rc.exp);
+    float t = __fmul_rn(val, sc[p]);
     f = p == 0 ? t : __fadd_rn(f, t);
   }
   return f;
@@ -595,14 +607,20 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
   const int nbpad = (nb + DR - 1) / DR * DR;
   const int first = ((blockIdx.x - pr.group_begin) * NW + wave) * TW * S;  // first tile of this wave
   const unsigned last_off = ((unsigned)n_tiles * (unsigned)nb - 1u) * 1024u + (unsigned)lane * 16u;
+  // The TW runs of a wave interleave tile by tile (run tw takes tiles first+tw, first+tw+TW, ...), so
+  // that what the wave finishes together is TW*16 adjacent output columns (its stores then fill
+  // whole cache lines between them); at the first position of a tile a run therefore skips the
+  // (TW-1) tiles of its siblings.
+  const unsigned skip = (unsigned)(TW - 1) * (unsigned)nb * 1024u;
   unsigned roff[TW];  // byte offset inside a plane of this lane's piece of the next chunk to request
 #pragma unroll
-  for (int tw = 0; tw < TW; ++tw) roff[tw] = (unsigned)(first + tw * S) * (unsigned)nb * 1024u + (unsigned)lane * 16u;
+  for (int tw = 0; tw < TW; ++tw) roff[tw] = (unsigned)(first + tw) * (unsigned)nb * 1024u + (unsigned)lane * 16u - skip;
 
   uint4 ring[DR][TW][P];
-  auto request = [&](int slot, bool real) {
+  auto request = [&](int slot, bool real, bool tile_start) {
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
+      roff[tw] += tile_start ? skip : 0u;
       const unsigned off = min(roff[tw], last_off);
 #pragma unroll
       for (int p = 0; p < P; ++p) ring[slot][tw][p] = gload16(codes[p] + (size_t)off);
@@ -610,7 +628,7 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
     }
   };
 #pragma unroll
-  for (int d = 0; d < D; ++d) request(d, d < nb);
+  for (int d = 0; d < D; ++d) request(d, d < nb, d == 0);
 
   // stage every operand row of the problem in LDS
   {
@@ -638,7 +656,7 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
     float sc[TW][P];
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
-      const int n = min((first + tw * S + s) * 16 + i, hot.n - 1);
+      const int n = min((first + s * TW + tw) * 16 + i, hot.n - 1);
 #pragma unroll
       for (int p = 0; p < P; ++p) sc[tw][p] = gload(scales[p] + n);
     }
@@ -650,14 +668,17 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
 #pragma unroll
         for (int p = 0; p < P; ++p) acc[tw][rt][p] = v4i{0, 0, 0, 0};
 
-    for (int kbg = 0; kbg < nbpad; kbg += DR) {
+    // a do-while: K has at least one block, and without a way round the loop the waits of the epilogue
+    // (for the scales requested above) can leave the ring's youngest requests in flight
+    int kbg = 0;
+    do {
 #pragma unroll
       for (int d = 0; d < DR; ++d) {
         const int kb = kbg + d;
         {  // request the position D ahead (slot (d + D) % DR, consumed at the previous position)
           int kb2 = kb + D;
           if (kb2 >= nbpad) kb2 -= nbpad;
-          request((d + D) % DR, kb2 < nb);
+          request((d + D) % DR, kb2 < nb, kb2 == 0);
         }
         if (kb < nb) {
 #pragma unroll
@@ -682,11 +703,12 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
           }
         }
       }
-    }
+      kbg += DR;
+    } while (kbg < nbpad);
 
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
-      const int t = first + tw * S + s;
+      const int t = first + s * TW + tw;
       const int n = t * 16 + i;
       if (t < n_tiles && n < hot.n) {
 #pragma unroll
@@ -695,7 +717,7 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
     }
     if (any_flag) {
       for (int tw = 0; tw < TW; ++tw) {
-        const int t = first + tw * S + s;
+        const int t = first + s * TW + tw;
         const int n = t * 16 + i;
         if (t >= pr.n_tiles || n >= pr.n) continue;
         for (int rt = 0; rt < RT; ++rt) {
