@@ -12,8 +12,11 @@ COPIES distinct resident copies of the layer (1.07 GB of 2-bit codes per launch,
 Prints ONE JSON line. `value` is algorithmic GB/s of the whole timed region (activation prep
 launches included); `roofline` is the decode kernel alone, timed with events on the stream it runs
 on; `cpu_baseline` is the CPU oracle's restatement of tritium-cpu timed on this host on one pass
-of the same sweep. `extra` carries the prefill GEMM (configs[2]) and the projection-stack
-tokens/s (configs[3]) measured in the same run.
+of the same sweep. `extra` carries the other configs measured in the same run: the batch-1 f32
+layer (configs[0]), the prefill GEMM (configs[2]), the projection-stack tokens/s (configs[3]) and
+the three-plane decode and prefill (configs[4]). Every timed region follows an untimed pre-warm of
+PREWARM_S seconds of the same work: from idle the clocks take tens of milliseconds to settle, and a
+cold first few milliseconds under-report a kernel by 10-25%.
 """
 import argparse
 import json
@@ -56,9 +59,24 @@ def algorithmic_bytes(m, n, k, planes, act_bytes, out_bytes, a8=False):
     return planes * n * nb * 64 + m * k * act_bytes + planes * n * 4 + m * n * out_bytes + (4 * m if a8 else 0)
 
 
+PREWARM_S = 0.25  # untimed: the clock governor needs some tens of milliseconds of load to settle
+
+
+def prewarm(be, fn, seconds=PREWARM_S):
+    """Run fn() untimed until `seconds` of wall clock have passed (at least once)."""
+    t0 = time.perf_counter()
+    while True:
+        fn()
+        be.sync()
+        if time.perf_counter() - t0 >= seconds:
+            return
+
+
 def time_steps(be, steps, warmup, step_fn):
-    """W untimed steps, then exactly K steps between two events on the library's stream."""
+    """Untimed: a fixed pre-warm, then W steps. Timed: exactly K steps between two events on the
+    library's stream."""
     start, stop = be.event(), be.event()
+    prewarm(be, lambda: step_fn(None))
     for _ in range(warmup):
         step_fn(None)
     be.sync()
@@ -109,13 +127,15 @@ def bench_decode(T, be, steps, warmup, rng):
     for m in SWEEP:
         g = groups[m]
         g.launch_parts(True, False)
+        for _ in range(20):
+            g.launch_parts(False, True)
         be.sync()
         a = be.event().record()
-        for _ in range(5):
+        for _ in range(50):
             g.launch_parts(False, True)
         b = be.event().record()
         be.sync()
-        ms = a.elapsed_ms(b) / 5
+        ms = a.elapsed_ms(b) / 50
         per_m[str(m)] = {"GB/s": round(per_launch[m] / ms / 1e6, 1), "us_per_layer": round(ms * 1e3 / COPIES, 3)}
     res = {
         "ms_per_step": total_ms / steps,
@@ -134,32 +154,101 @@ def bench_decode(T, be, steps, warmup, rng):
     return res
 
 
-def bench_prefill(T, be, rng, iters=10):
-    """configs[2]: M=2048, K=2560, N=6912, one plane, bf16 activations quantized per token to int8,
-    int32 accumulation, bf16 output."""
-    m, k, n = 2048, 2560, 6912
-    layers = [be.linear([T.pack_rows(ternary(rng, n, k, 0.4), n, k)], [rng.uniform(0.01, 0.1, n).astype(np.float32)],
-                        n, k) for _ in range(2)]
-    act = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32)), "bf16")
-    out = be.empty(m * n, "bf16")
-    q, s = be.empty(m * k, "i8"), be.empty(m, "f32")
-    be.act_quant_i8(act, m, k, q, s)
-    for i in range(3):
-        be.linear_a8(layers[i % 2], act, m, out)
-    be.sync()
+def time_calls(be, fn, iters):
+    """Pre-warm, then `iters` calls of fn(i) between two events; returns ms per call."""
+    prewarm(be, lambda: fn(0))
     a = be.event().record()
     for i in range(iters):
-        be.linear_a8(layers[i % 2], act, m, out)
+        fn(i)
     b = be.event().record()
     be.sync()
-    ms = a.elapsed_ms(b) / iters
-    ops = 2.0 * m * n * k
-    return {"workload": "prefill GEMM M=2048 K=2560 N=6912 1 plane, bf16 act -> int8 per token -> int32 acc -> bf16",
+    return a.elapsed_ms(b) / iters
+
+
+def bench_prefill(T, be, rng, m, k, n, planes=1, iters=100):
+    """Prefill GEMM: bf16 activations quantized per token to int8 (fused prep launch), int8 MFMA with
+    int32 accumulation over `planes` additive planes, bf16 output after per-channel x per-token scale."""
+    p0s = (0.4, 0.7, 0.85)[:planes]
+    layers = [be.linear([T.pack_rows(ternary(rng, n, k, p0), n, k) for p0 in p0s],
+                        [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in p0s], n, k) for _ in range(2)]
+    act = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32)), "bf16")
+    out = be.empty(m * n, "bf16")
+    ms = time_calls(be, lambda i: be.linear_a8(layers[i % 2], act, m, out), iters)
+    ops = 2.0 * m * n * k * planes
+    for l in layers:
+        l.free()
+    act.free()
+    out.free()
+    return {"workload": f"prefill GEMM M={m} K={k} N={n} {planes} plane(s), bf16 act -> int8 per token -> int32 acc -> bf16",
             "ms_per_call_incl_quant": round(ms, 4), "TOPS": round(ops / ms / 1e9, 1),
             "frac_of_int8_peak": round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4)}
 
 
-def bench_stack(T, be, rng, iters=10):
+def bench_config1(T, be, rng, iters=200):
+    """configs[0]: one ternary linear, K=2560 N=6912, one plane, f32 N(0,1) activation, batch 1.
+    Through the adapter call on host slices (upload, kernel, download, sync per call) and through the
+    device-resident call (one launch of prep + decode kernel, back to back)."""
+    n, k = 6912, 2560
+    w = T.pack_rows(ternary(rng, n, k, 0.4), n, k)
+    sc = rng.uniform(0.01, 0.1, n).astype(np.float32)
+    act = rng.standard_normal((1, k)).astype(np.float32)
+    buf = be.upload_weights(w, T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0)
+    out = np.zeros(n, np.float32)
+    call = T.MpGemm(act.reshape(-1), buf, sc, T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0, out)
+    for _ in range(20):
+        be.mpgemm(call)
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        be.mpgemm(call)
+    host_us = (time.perf_counter() - t0) / iters * 1e6
+    layer = be.linear([w], [sc], n, k)
+    dact, dout = be.to_device(act, "f32"), be.empty(n, "f32")
+    ms = time_calls(be, lambda i: be.linear_float(layer, dact, 1, dout), iters)
+    by = algorithmic_bytes(1, n, k, 1, 4, 4)
+    layer.free()
+    dact.free()
+    dout.free()
+    return {"workload": "K=2560 N=6912 1 plane, f32 activation, batch 1 (a single 4.4 MB layer: launch-bound)",
+            "adapter_call_on_host_slices_us": round(host_us, 1), "device_resident_call_us": round(ms * 1e3, 2),
+            "device_resident_GB/s": round(by / ms / 1e6, 1)}
+
+
+def bench_config5(T, be, rng):
+    """configs[4]: three additive planes (P(0)=0.4/0.7/0.85), hidden 5120, FFN 17408. Decode at batch
+    64 over the up and down projections of 8 distinct layers in one grouped launch (W1.58A8, bf16 in
+    and out), and the 4096-token prefill GEMM of the up projection."""
+    h, f, layers_n, m = 5120, 17408, 8, 64
+    shapes = {"up": (f, h), "down": (h, f)}
+    lins = []
+    for _ in range(layers_n):
+        lins.append({name: be.linear([T.pack_rows(ternary(rng, n, k, p0), n, k) for p0 in (0.4, 0.7, 0.85)],
+                                     [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in range(3)], n, k)
+                     for name, (n, k) in shapes.items()})
+    hid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
+    mid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, f)).astype(np.float32)), "bf16")
+    members, outs = [], []
+    for L in lins:
+        for name, src in (("up", hid), ("down", mid)):
+            o = be.empty(m * shapes[name][0], "bf16")
+            outs.append(o)
+            members.append((L[name], src, m, o))
+    g = be.group(members, 1, "bf16", "bf16")
+    ms = time_calls(be, lambda i: g.launch(), 30)
+    by = layers_n * sum(algorithmic_bytes(m, n, k, 3, 2, 2, a8=True) for n, k in shapes.values())
+    res = {"decode_batch64": {"workload": f"{layers_n} layers x (up, down), 3 planes, batch 64, one grouped launch incl. quantization",
+                              "ms_per_step": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+                              "frac_of_hbm_peak": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}}
+    g.destroy()
+    for x in outs + [hid, mid]:
+        x.free()
+    for L in lins:
+        for l in L.values():
+            l.free()
+    res["prefill_4096"] = bench_prefill(T, be, rng, 4096, h, f, planes=3, iters=30)
+    return res
+
+
+def bench_stack(T, be, rng, iters=100):
     """configs[3]: the 7 ternary projections of 30 decoder layers (hidden 2560, FFN 6912, 20 query
     heads and 5 KV heads of 128), W1.58A8, one launch for the whole stack with given inputs.
     tokens/s = batch / time of the projection path only."""
@@ -186,15 +275,7 @@ def bench_stack(T, be, rng, iters=10):
                 outs.append(o)
                 members.append((L[name], src, m, o))
         g = be.group(members, 1, "bf16", "bf16")
-        for _ in range(3):
-            g.launch()
-        be.sync()
-        a = be.event().record()
-        for _ in range(iters):
-            g.launch()
-        b = be.event().record()
-        be.sync()
-        ms = a.elapsed_ms(b) / iters
+        ms = time_calls(be, lambda i: g.launch(), iters)
         res[f"batch{m}"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1),
                             "code_GB/s": round(code_bytes / ms / 1e6, 1)}
         g.destroy()
@@ -243,8 +324,8 @@ def cpu_baseline(rng):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM and projection-stack legs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -265,6 +346,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "prewarm_s": PREWARM_S,
         "ms_per_step": round(dec["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -293,7 +375,10 @@ def main():
         src.free()
         dst.free()
     if not args.no_extra:
-        out["extra"] = {"prefill_gemm": bench_prefill(T, be, rng), "projection_stack": bench_stack(T, be, rng)}
+        out["extra"] = {"config1_f32_batch1": bench_config1(T, be, rng),
+                        "prefill_gemm": bench_prefill(T, be, rng, 2048, 2560, 6912),
+                        "projection_stack": bench_stack(T, be, rng),
+                        "config5_three_planes": bench_config5(T, be, rng)}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np.random.default_rng(1))
     be.close()

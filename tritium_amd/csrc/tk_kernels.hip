@@ -1153,14 +1153,6 @@ __global__ void tk_decode_trits_kernel(const uint8_t *__restrict__ codes, size_t
 // activation prep: one workgroup per token
 // ------------------------------------------------------------------------------------------
 
-__device__ __forceinline__ size_t ap_offset(size_t k0, size_t R, size_t row) {
-  // k0 is a multiple of 4: the dword (s, b=0..3) of piece (kb, j, g)
-  size_t kb = k0 >> 8, e = k0 & 255;
-  size_t c = e >> 7, s = (e & 127) >> 5, mm = e & 31;
-  size_t g = c * 2 + (mm >> 4), j = (mm & 15) >> 2;
-  return ((((kb * 4 + j) * 4 + g) * R + row) * 16 + s * 4);
-}
-
 __device__ float block_max(float v, float *sh) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
   if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
@@ -1178,18 +1170,64 @@ __device__ int block_sum(int v, int *sh) {
   return r;
 }
 
+// Four consecutive activations starting at element e (a multiple of 4) as floats; elements at or
+// past k read as 0. `vec` says the row starts are aligned for one 8- or 16-byte load.
+__device__ __forceinline__ void load_act4(const void *act, int dtype, size_t base, size_t e, size_t k, bool vec, float (&v)[4]) {
+  if (vec && e + 4 <= k) {
+    if (dtype == TK_BF16) {
+      typedef unsigned v2u __attribute__((ext_vector_type(2)));
+      const v2u u = *(const TK_GLOBAL v2u *)((const uint16_t *)act + base + e);
+      v[0] = __uint_as_float(u.x << 16);
+      v[1] = __uint_as_float(u.x & 0xFFFF0000u);
+      v[2] = __uint_as_float(u.y << 16);
+      v[3] = __uint_as_float(u.y & 0xFFFF0000u);
+    } else {
+      const v4u u = *(const TK_GLOBAL v4u *)((const float *)act + base + e);
+      v[0] = __uint_as_float(u.x);
+      v[1] = __uint_as_float(u.y);
+      v[2] = __uint_as_float(u.z);
+      v[3] = __uint_as_float(u.w);
+    }
+    return;
+  }
+#pragma unroll
+  for (int b = 0; b < 4; ++b) v[b] = e + b < k ? load_act(act, dtype, base + e + b) : 0.0f;
+}
+
+__device__ __forceinline__ bool act_rows_vectorizable(const void *act, int dtype, size_t k) {
+  return (k & 3) == 0 && (((size_t)act) & 15) == 0 && (dtype == TK_BF16 || dtype == TK_F32);
+}
+
 // gamma = max |a| with the reference's `a > gamma` rule (NaN never wins), plus a non-finite flag.
-__device__ void row_absmax(const void *act, int dtype, size_t base, size_t k, float *sh, float &gamma,
+__device__ void row_absmax(const void *act, int dtype, size_t base, size_t k, bool vec, float *sh, float &gamma,
                            int &nonfinite, int *shi) {
   float g = 0.0f;
   int nf = 0;
-  for (size_t c = threadIdx.x; c < k; c += TK_WG) {
-    float a = fabsf(load_act(act, dtype, base + c));
-    if (a > g) g = a;
-    nf |= !(a <= 3.402823466e38f);  // NaN or Inf
+  for (size_t e = (size_t)threadIdx.x * 4; e < k; e += TK_WG * 4) {
+    float v[4];
+    load_act4(act, dtype, base, e, k, vec, v);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const float a = fabsf(v[b]);
+      if (a > g) g = a;
+      nf |= !(a <= 3.402823466e38f);  // NaN or Inf
+    }
   }
   gamma = block_max(g, sh);
   nonfinite = block_sum(nf, shi) != 0;
+}
+
+// A thread of the prep kernels builds whole 16-byte pieces of the operand layout. Piece q of K block
+// kb (q = c*8 + h*4 + j, lane group g = 2c + h) holds the elements kb*256 + c*128 + s*32 + h*16 + j*4
+// + b for s, b = 0..3: consecutive q walk 32 consecutive elements for each s, so the four loads of
+// a wave are contiguous runs.
+__device__ __forceinline__ size_t piece_elem0(size_t kb, int q) {
+  const int c = q >> 3, h = (q >> 2) & 1, j = q & 3;
+  return kb * 256 + (size_t)c * 128 + (size_t)h * 16 + (size_t)j * 4;
+}
+__device__ __forceinline__ size_t piece_offset(size_t kb, int q, size_t R, size_t row) {
+  const int c = q >> 3, h = (q >> 2) & 1, j = q & 3, g = c * 2 + h;
+  return (((kb * 4 + j) * 4 + g) * R + row) * 16;
 }
 
 __device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const TkPrep *table, int nprep, int &row) {
@@ -1212,27 +1250,49 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
   const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = row * k;
+  const void *act = pp.act;
+  const int dtype = pp.act_dtype;
+  int8_t *ap = pp.ap, *qrm = pp.q_rowmajor;
+  const bool vec = act_rows_vectorizable(act, dtype, k);
   float gamma;
   int nonfinite;
-  row_absmax(pp.act, pp.act_dtype, base, k, shf, gamma, nonfinite, shi);
+  row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi);
   const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
+  const bool live = gamma != 0.0f && !nonfinite;
   int sum = 0;
-  for (size_t d = threadIdx.x; d < nb * 64; d += TK_WG) {
-    const size_t k0 = d * 4;
-    uint32_t packed = 0;
-    for (int b = 0; b < 4; ++b) {
-      int q = 0;
-      if (k0 + b < k && gamma != 0.0f && !nonfinite) {
-        float a = load_act(pp.act, pp.act_dtype, base + k0 + b);
-        float r = rintf(__fmul_rn(a, s));  // one multiply, ties to even
-        r = r < -128.0f ? -128.0f : (r > 127.0f ? 127.0f : r);
-        q = (int)r;
+  for (size_t pc = threadIdx.x; pc < nb * 16; pc += TK_WG) {
+    const size_t kb = pc >> 4;
+    const int q16 = (int)(pc & 15);
+    const size_t e0 = piece_elem0(kb, q16);
+    v4u piece;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const size_t e = e0 + (size_t)sl * 32;
+      float v[4];
+      load_act4(act, dtype, base, e, k, vec, v);
+      uint32_t packed = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        int q = 0;
+        if (live && e + b < k) {
+          float r = rintf(__fmul_rn(v[b], s));  // one multiply, ties to even
+          r = r < -128.0f ? -128.0f : (r > 127.0f ? 127.0f : r);
+          q = (int)r;
+        }
+        sum += q;
+        packed |= ((uint32_t)q & 0xFFu) << (8 * b);
       }
-      sum += q;
-      packed |= ((uint32_t)q & 0xFFu) << (8 * b);
-      if (pp.q_rowmajor && k0 + b < k) pp.q_rowmajor[base + k0 + b] = (int8_t)q;
+      piece[sl] = packed;
+      if (qrm) {
+        if (vec && e + 4 <= k) {
+          *(TK_GLOBAL uint32_t *)(qrm + base + e) = packed;
+        } else {
+          for (int b = 0; b < 4; ++b)
+            if (e + b < k) qrm[base + e + b] = (int8_t)(packed >> (8 * b));
+        }
+      }
     }
-    if (pp.ap) *(uint32_t *)(pp.ap + ap_offset(k0, R, row)) = packed;
+    if (ap) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, row)) = piece;
   }
   sum = block_sum(sum, shi);
   if (threadIdx.x == 0) {
@@ -1243,7 +1303,9 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
   }
 }
 
-// Float token -> four balanced base-256 digit rows of round(a · 2^(30-E)), 2^(E-1) <= max|a| < 2^E.
+// Float token -> four balanced base-256 digit rows of round(a * 2^(30-E)), 2^(E-1) <= max|a| < 2^E.
+// Scaling a float by a power of two is exact, so the rounding to an integer happens once, in
+// single precision.
 __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                                int nprep) {
   __shared__ float shf[4];
@@ -1252,35 +1314,51 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
   const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = tok * k;
+  const void *act = pp.act;
+  const int dtype = pp.act_dtype;
+  int8_t *ap = pp.ap;
+  const bool vec = act_rows_vectorizable(act, dtype, k);
   float gamma;
   int nonfinite;
-  row_absmax(pp.act, pp.act_dtype, base, k, shf, gamma, nonfinite, shi);
+  row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi);
   int E = 0;
   if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
   const int shift = 30 - E;
+  const bool live = gamma != 0.0f && !nonfinite;
   int sums[4] = {0, 0, 0, 0};
-  for (size_t d = threadIdx.x; d < nb * 64; d += TK_WG) {
-    const size_t k0 = d * 4;
-    uint32_t packed[4] = {0, 0, 0, 0};
-    for (int b = 0; b < 4; ++b) {
-      int q = 0;
-      if (k0 + b < k && gamma != 0.0f && !nonfinite)
-        q = __double2int_rn(ldexp((double)load_act(pp.act, pp.act_dtype, base + k0 + b), shift));  // |q| <= 2^30
+  for (size_t pc = threadIdx.x; pc < nb * 16; pc += TK_WG) {
+    const size_t kb = pc >> 4;
+    const int q16 = (int)(pc & 15);
+    const size_t e0 = piece_elem0(kb, q16);
+    v4u piece[4];
 #pragma unroll
-      for (int dg = 0; dg < 4; ++dg) {
-        int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
-        q = (q - dv) >> 8;
-        sums[dg] += dv;
-        packed[dg] |= ((uint32_t)dv & 0xFFu) << (8 * b);
+    for (int sl = 0; sl < 4; ++sl) {
+      const size_t e = e0 + (size_t)sl * 32;
+      float v[4];
+      load_act4(act, dtype, base, e, k, vec, v);
+      uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        int q = 0;
+        if (live && e + b < k) q = __float2int_rn(ldexpf(v[b], shift));  // |q| <= 2^30
+#pragma unroll
+        for (int dg = 0; dg < 4; ++dg) {
+          int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
+          q = (q - dv) >> 8;
+          sums[dg] += dv;
+          packed[dg] |= ((uint32_t)dv & 0xFFu) << (8 * b);
+        }
       }
+#pragma unroll
+      for (int dg = 0; dg < 4; ++dg) piece[dg][sl] = packed[dg];
     }
 #pragma unroll
-    for (int dg = 0; dg < 4; ++dg) *(uint32_t *)(pp.ap + ap_offset(k0, R, tok * 4 + dg)) = packed[dg];
+    for (int dg = 0; dg < 4; ++dg) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, tok * 4 + dg)) = piece[dg];
   }
 #pragma unroll
   for (int dg = 0; dg < 4; ++dg) {
-    int s = block_sum(sums[dg], shi);
-    if (threadIdx.x == 0) pp.rowsum[tok * 4 + dg] = s;
+    int sm = block_sum(sums[dg], shi);
+    if (threadIdx.x == 0) pp.rowsum[tok * 4 + dg] = sm;
   }
   if (threadIdx.x == 0) {
     pp.exps[tok] = -shift;
@@ -1296,17 +1374,29 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_i8_kernel(TkPrep single, const 
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
   const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const int8_t *q = (const int8_t *)pp.act;
+  int8_t *ap = pp.ap;
   const size_t base = row * k;
+  const bool vec = (k & 3) == 0 && (((size_t)q) & 3) == 0;
   int sum = 0;
-  for (size_t d = threadIdx.x; d < nb * 64; d += TK_WG) {
-    const size_t k0 = d * 4;
-    uint32_t packed = 0;
-    for (int b = 0; b < 4; ++b) {
-      int v = k0 + b < k ? (int)q[base + k0 + b] : 0;
-      sum += v;
-      packed |= ((uint32_t)v & 0xFFu) << (8 * b);
+  for (size_t pc = threadIdx.x; pc < nb * 16; pc += TK_WG) {
+    const size_t kb = pc >> 4;
+    const int q16 = (int)(pc & 15);
+    const size_t e0 = piece_elem0(kb, q16);
+    v4u piece;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const size_t e = e0 + (size_t)sl * 32;
+      uint32_t packed = 0;
+      if (vec && e + 4 <= k) {
+        packed = *(const TK_GLOBAL uint32_t *)(q + base + e);
+      } else {
+        for (int b = 0; b < 4; ++b)
+          if (e + b < k) packed |= ((uint32_t)q[base + e + b] & 0xFFu) << (8 * b);
+      }
+      sum += (int)(int8_t)(packed) + (int)(int8_t)(packed >> 8) + (int)(int8_t)(packed >> 16) + (int)(int8_t)(packed >> 24);
+      piece[sl] = packed;
     }
-    *(uint32_t *)(pp.ap + ap_offset(k0, R, row)) = packed;
+    *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, row)) = piece;
   }
   sum = block_sum(sum, shi);
   if (threadIdx.x == 0) pp.rowsum[row] = sum;
