@@ -196,6 +196,9 @@ int tk_set_decode_kernel(tk_ctx *ctx, int variant);
 /* Consecutive output tiles a wave of the flow kernel walks as one stream; 0 = chosen from the size
  * of the launch. A tuning knob: results do not depend on it. */
 int tk_set_flow_run_tiles(tk_ctx *ctx, int tiles);
+/* Positions in the flow kernel's prefetch ring: 0 = chosen per launch (fewest padded positions for
+ * the K block counts of the launch), or 2..5. A tuning knob: results do not depend on it. */
+int tk_set_flow_ring(tk_ctx *ctx, int positions);
 int tk_set_stream_min_groups(tk_ctx *ctx, int groups);
 int tk_get_stream_min_groups(const tk_ctx *ctx);
 

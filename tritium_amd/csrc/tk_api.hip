@@ -73,6 +73,7 @@ struct tk_ctx {
   int stream_min_groups = 0;  // set at init to the CU count
   int decode_force = 0;  // DECODE_AUTO
   int flow_run_tiles = 0;  // 0 = automatic
+  int flow_ring = 0;       // 0 = automatic
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
   int *d_invalid = nullptr;
 };
@@ -254,6 +255,15 @@ extern "C" int tk_set_flow_run_tiles(tk_ctx *ctx, int tiles) {
   return TK_OK;
 }
 
+extern "C" int tk_set_flow_ring(tk_ctx *ctx, int positions) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_ring: null context");
+  if (positions != 0 && (positions < 2 || positions > 5))
+    return tk_fail(TK_ERR_INVALID_INPUT, "flow_ring=%d - use 0 (automatic) or 2..5", positions);
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  ctx->flow_ring = positions;
+  return TK_OK;
+}
+
 extern "C" int tk_set_decode_kernel(tk_ctx *ctx, int variant) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_decode_kernel: null context");
   if (variant < 0 || variant > 3) return tk_fail(TK_ERR_INVALID_INPUT, "decode kernel %d - use 0..3", variant);
@@ -418,13 +428,14 @@ static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
 // (lds_bytes) once, so it should stream several times that in weights; beyond that, shorter runs
 // win (more, shorter-lived workgroups keep more loads in flight and balance the tail). Measured on
 // K=2048 N=8192 x 2 planes over 128 layer copies: 4-16 operand rows peak at 2 tiles per run
-// (128 KiB of weights per workgroup), 32 and 64 rows at 8 (8x the staged bytes).
+// (128 KiB of weights per workgroup), 32 rows at 4 (4x the staged bytes, four-wave workgroups), 64
+// rows at 8 (16x, eight-wave workgroups, one per CU).
 static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
                           size_t nb) {
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)tk_flow_runs_per_wave(planes, rt);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
-  size_t target = 8 * lds_bytes * (size_t)(waves / 4);
+  size_t target = lds_bytes * (size_t)waves * (size_t)waves / 4;
   if (target < 128 * 1024) target = 128 * 1024;
   size_t s = 1;
   while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
@@ -582,7 +593,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.grid = flow_groups;
     cfg.lds_bytes = pl.flow_lds;
     cfg.waves = flow_waves(pl.flow_lds);
-    cfg.ring = tk_flow_ring(&pr.nb, nullptr, 1);
+    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -945,7 +956,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       nbs[i] = plans[i].pr.nb;
       wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
     }
-    g->cfg.ring = tk_flow_ring(nbs.data(), wts.data(), (int)count);
+    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt);
   }
   *out = g;
   return TK_OK;

@@ -73,7 +73,7 @@ struct TkLaunchCfg {
   size_t lds_bytes;
   unsigned grid;
   int waves;    // flow kernel: waves per workgroup (4, or 8 when the operand rows need > 64 KiB of LDS)
-  int ring;     // flow kernel: positions in the prefetch ring (3, 4 or 5)
+  int ring;     // flow kernel: positions in the prefetch ring (2..5)
 };
 
 #ifdef __cplusplus
@@ -98,7 +98,7 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
                           const TkLaunchCfg &cfg);
 int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
-int tk_flow_ring(const int *nbs, const double *weights, int count);
+int tk_flow_ring(const int *nbs, const double *weights, int count, int rt);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
                           unsigned grid_n);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

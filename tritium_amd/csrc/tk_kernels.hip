@@ -1519,14 +1519,14 @@ static hipError_t flow_launch_one(K kernel, hipStream_t s, const TkProblem &sg, 
                                   const int *wg_prob, const TkLaunchCfg &cfg, int threads) {
   if (cfg.lds_bytes > 64 * 1024) {
     // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    static thread_local const void *raised[128];
+    static thread_local const void *raised[256];
     static thread_local int nraised = 0;
     bool done = false;
     for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
     if (!done) {
       hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
-      if (nraised < 128) raised[nraised++] = (const void *)kernel;
+      if (nraised < 256) raised[nraised++] = (const void *)kernel;
     }
   }
   hipLaunchKernelGGL(kernel, dim3(cfg.grid), dim3(threads), cfg.lds_bytes, s, sg, table, wg_prob);
@@ -1539,6 +1539,9 @@ static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkPro
   constexpr int TW = (RT >= 4 && P <= 2) ? 2 : 1;
   const int threads = cfg.waves * 64;
   switch (cfg.ring) {
+    case 2:
+      if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, 2, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow_kernel<P, RT, TW, 2, false>, s, sg, table, wg_prob, cfg, threads);
     case 3:
       if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, 3, true>, s, sg, table, wg_prob, cfg, threads);
       return flow_launch_one(tk_flow_kernel<P, RT, TW, 3, false>, s, sg, table, wg_prob, cfg, threads);
@@ -1567,13 +1570,16 @@ static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProb
 int tk_flow_runs_per_wave(int planes, int rt) { return (rt >= 4 && planes <= 2) ? 2 : 1; }
 
 // Ring size of the flow kernel for launches whose K block counts are nbs[0..count): the compiled
-// size (3, 4 or 5 positions) that pads the fewest positions, weighted by each problem's chunk count;
-// ties go to the deeper ring.
-int tk_flow_ring(const int *nbs, const double *weights, int count) {
-  int best = 4;
+// size (2..5 positions) that pads the fewest positions, weighted by each problem's chunk count.
+// Ties go to the shallow ring, which costs the fewest registers (more waves per SIMD did more for
+// the measured bandwidth than more loads per wave), except at two row tiles, where 64 KiB of LDS
+// per workgroup caps the CU at eight waves and the deeper ring measured better.
+int tk_flow_ring(const int *nbs, const double *weights, int count, int rt) {
+  const int shallow[4] = {2, 4, 3, 5}, deep[4] = {4, 2, 3, 5};
+  const int *cand = rt == 2 ? deep : shallow;
+  int best = cand[0];
   double best_waste = -1.0;
-  const int cand[3] = {5, 4, 3};
-  for (int c = 0; c < 3; ++c) {
+  for (int c = 0; c < 4; ++c) {
     double waste = 0.0;
     for (int x = 0; x < count; ++x) {
       const int nb = nbs[x], pad = (nb + cand[c] - 1) / cand[c] * cand[c];
