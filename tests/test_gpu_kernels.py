@@ -364,6 +364,46 @@ def test_group_launch_equals_single_launches(backend, oracle):
         grp.destroy()
 
 
+def test_group_with_rows_beyond_lds_takes_the_prefill_kernel(backend, oracle, decode_kernel):
+    """Grouped decode whose operand rows do not fit in LDS (40 tokens x K=4500 int8, 12 tokens x 4
+    digit rows x K=4500) runs as one grouped launch of the prefill kernel; bits equal the single
+    launches and the CPU composition. Two projections share an activation, a third has its own."""
+    if decode_kernel != "ksplit":
+        pytest.skip("automatic kernel choice only")
+    backend.set_decode_kernel(0)
+    rng = np.random.default_rng(37)
+    for mode, m, fn in ((1, 40, backend.linear_a8), (0, 12, backend.linear_float)):
+        k = 4500
+        act_a = rng.standard_normal((m, k)).astype(np.float32)
+        act_b = rng.standard_normal((m, k)).astype(np.float32)
+        act_c = rng.standard_normal((m, 768)).astype(np.float32)  # these rows do fit: the flow kernel's share
+        da, db, dc = backend.to_device(act_a, "f32"), backend.to_device(act_b, "f32"), backend.to_device(act_c, "f32")
+        members, singles, hosts = [], [], []
+        for n, src, act in ((136, da, act_a), (200, dc, act_c), (72, da, act_a), (257, db, act_b), (48, dc, act_c)):
+            k = act.shape[1]
+            ws = [ternary(rng, n, k, 0.4), ternary(rng, n, k, 0.7)]
+            scs = [scales(rng, n), scales(rng, n)]
+            packed, layer = _layer(backend, oracle, ws, scs)
+            out_g, out_s = backend.empty(m * n, "f32"), backend.empty(m * n, "f32")
+            members.append((layer, src, m, out_g))
+            singles.append((layer, src, out_s))
+            hosts.append((packed, scs, act, n))
+        grp = backend.group(members, mode, "f32", "f32")
+        grp.launch()
+        grp.launch()
+        for (layer, src, _, out_g), (_, _, out_s), (packed, scs, act, n) in zip(members, singles, hosts):
+            k = act.shape[1]
+            fn(layer, src, m, out_s)
+            got = out_g.to_host()
+            assert same_bits(got, out_s.to_host())
+            if mode == 1:
+                assert same_bits(got, oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+            else:
+                want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+                assert accepts(got.reshape(m, n), want.reshape(m, n), rel=1e-4, floor=1.0).all()
+        grp.destroy()
+
+
 def test_ternary_linear_forward(backend, oracle):
     """tritium-nn/tests/layers.rs:138+ : TernaryLinear on the backend vs the inline reference, ragged K."""
     rng = np.random.default_rng(31)

@@ -419,7 +419,7 @@ struct Plan {
   size_t flow_lds;
 };
 
-enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3 };
+enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3, DECODE_GEMM = 4 };
 
 static const size_t kLdsFlowMax = 160 * 1024;
 static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
@@ -450,6 +450,39 @@ static const size_t kLdsStreamBudget = 64 * 1024;
 static bool prefer_stream(const tk_ctx *ctx, unsigned groups);
 
 // Fills everything of a plan that does not depend on workspace addresses.
+// GEMM form of a planned problem: padded operand row stride, tile grid and its split over the XCDs.
+static void plan_gemm(Plan *pl) {
+  TkProblem &pr = pl->pr;
+  const size_t R = (size_t)pr.R;
+  // The GEMM reads, per K block, 16 segments of the operand rows that are exactly rs*16 bytes apart,
+  // and all workgroups do so in step: with a power-of-two stride they would all land on the same
+  // few memory channels. 16 rows (256 bytes) of padding walk the segments across the channels.
+  pr.rs = (int)(R + 16);
+  pl->cfg.rt = 4;
+  pl->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();  // three 64-row blocks of 256 k + the row constants
+  pl->grid_m = (unsigned)((R + 63) / 64);
+  const unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(pr.planes);
+  pl->grid_n = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
+  // split the tile grid over the 8 XCDs so that each L2 holds few A row blocks and few weight
+  // column blocks: minimise bytes touched per XCD = K*(64*sub_m + 4*tiles_per_wg*planes*sub_n)
+  pr.grid_m = (int)pl->grid_m;
+  pr.grid_n = (int)pl->grid_n;
+  size_t best = (size_t)-1;
+  for (int xr = 1; xr <= 8; xr *= 2) {
+    const int xc = 8 / xr;
+    const int sm = ((int)pl->grid_m + xr - 1) / xr, sn = ((int)pl->grid_n + xc - 1) / xc;
+    const size_t cost = (size_t)64 * sm + (size_t)4 * per_wg * pr.planes * sn;
+    const size_t waste = (size_t)8 * sm * sn;  // launched workgroups, some of them empty
+    const size_t score = cost * 1024 + waste;
+    if (score < best) {
+      best = score;
+      pr.xr = xr;
+      pr.sub_m = sm;
+      pr.sub_n = sn;
+    }
+  }
+}
+
 static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_t k, size_t m, int mode,
                        int out_dtype, Plan *pl) {
   memset(pl, 0, sizeof *pl);
@@ -493,33 +526,7 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->flow_lds = nb * 256 * R;
     pl->flow_ok = pl->flow_lds <= kLdsFlowMax;
   } else {
-    // The GEMM reads, per K block, 16 segments of the operand rows that are exactly rs*16 bytes apart,
-    // and all workgroups do so in step: with a power-of-two stride they would all land on the same
-    // few memory channels. 16 rows (256 bytes) of padding walk the segments across the channels.
-    pr.rs = (int)(R + 16);
-    pl->cfg.rt = 4;
-    pl->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();  // three 64-row blocks of 256 k
-    pl->grid_m = (unsigned)((R + 63) / 64);
-    const unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(layer->n_planes);
-    pl->grid_n = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
-    // split the tile grid over the 8 XCDs so that each L2 holds few A row blocks and few weight
-    // column blocks: minimise bytes touched per XCD = K·(64·sub_m + 4·tiles_per_wg·planes·sub_n)
-    pr.grid_m = (int)pl->grid_m;
-    pr.grid_n = (int)pl->grid_n;
-    size_t best = (size_t)-1;
-    for (int xr = 1; xr <= 8; xr *= 2) {
-      const int xc = 8 / xr;
-      const int sm = ((int)pl->grid_m + xr - 1) / xr, sn = ((int)pl->grid_n + xc - 1) / xc;
-      const size_t cost = (size_t)64 * sm + (size_t)4 * per_wg * layer->n_planes * sn;
-      const size_t waste = (size_t)8 * sm * sn;  // launched workgroups, some of them empty
-      const size_t score = cost * 1024 + waste;
-      if (score < best) {
-        best = score;
-        pr.xr = xr;
-        pr.sub_m = sm;
-        pr.sub_n = sn;
-      }
-    }
+    plan_gemm(pl);
   }
 }
 
@@ -607,7 +614,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else if (pl.skinny) {
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
   } else {
-    HIPCHK(tk_launch_gemm(ctx->stream, &pr, pl.cfg, pl.grid_m, pl.grid_n));
+    HIPCHK(tk_launch_gemm(ctx->stream, &pr, nullptr, nullptr, pl.cfg));
   }
   return TK_OK;
 }
@@ -784,6 +791,11 @@ struct tk_group {
   int variant = 1;
   size_t wg_prob_off = 0;
   TkLaunchCfg cfg{};
+  // a second launch: the members of a prefill-form group whose operand rows do fit in LDS go
+  // through the flow kernel
+  bool has_flow_part = false;
+  size_t flow_wg_prob_off = 0;
+  TkLaunchCfg flow_cfg{};
 };
 
 extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size_t count, int mode, int act_dtype,
@@ -842,7 +854,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       rows += (unsigned)m;
       prep_of[i] = (int)preps.size();
       preps.push_back(pp);
-      prep_off.push_back(take(R * nb * 256));
+      prep_off.push_back(take((R + 16) * nb * 256));  // room for the GEMM form's padded row stride
       take(R * 4); take(m * 4); take(m * 4); take(m * 4); take(m * 4);
     }
     plans[i].pr.tile_begin = (int)tiles;
@@ -870,10 +882,58 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     fgroups += ((unsigned)plans[i].pr.n_tiles + fper - 1) / fper;
     if (plans[i].stream_lds > slds) slds = plans[i].stream_lds;
   }
-  const int variant = choose_decode(ctx, flow_ok, fgroups, sgroups);
+  int variant = choose_decode(ctx, flow_ok, fgroups, sgroups);
+  // Operand rows that do not fit in LDS, and more than one row tile of them: the prefill kernel
+  // (operand rows streamed block by block, int8 MFMA over 64-row tiles) beats a decode kernel that
+  // re-stages slices of K behind barriers.
+  if (ctx->decode_force == DECODE_AUTO && !flow_ok && rt >= 2) variant = DECODE_GEMM;
   std::vector<int> wg_prob;
   unsigned groups_total = 0;
-  if (variant != DECODE_KSPLIT) {
+  std::vector<int> flow_wg_prob;
+  TkLaunchCfg flow_cfg{};
+  if (variant == DECODE_GEMM) {
+    // members whose rows fit go through the flow kernel in a launch of their own
+    size_t pflds = 0, pnb_max = 1;
+    unsigned ptiles = 0;
+    std::vector<int> nbs;
+    std::vector<double> wts;
+    for (size_t i = 0; i < count; ++i) {
+      if (!plans[i].flow_ok) continue;
+      if (plans[i].flow_lds > pflds) pflds = plans[i].flow_lds;
+      if ((size_t)plans[i].pr.nb > pnb_max) pnb_max = plans[i].pr.nb;
+      ptiles += (unsigned)plans[i].pr.n_tiles;
+      nbs.push_back(plans[i].pr.nb);
+      wts.push_back((double)plans[i].pr.n_tiles * (double)plans[i].pr.nb);
+    }
+    const int pfw = flow_waves(pflds);
+    const int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max) : 1;
+    const unsigned pper = (unsigned)pfw * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)prun;
+    unsigned flow_total = 0;
+    for (size_t i = 0; i < count; ++i) {
+      if (plans[i].flow_ok) {
+        const unsigned gi = ((unsigned)plans[i].pr.n_tiles + pper - 1) / pper;
+        plans[i].pr.group_begin = (int)flow_total;
+        plans[i].pr.run_tiles = prun;
+        for (unsigned j = 0; j < gi; ++j) flow_wg_prob.push_back((int)i);
+        flow_total += gi;
+        continue;
+      }
+      plan_gemm(&plans[i]);
+      const unsigned gi = 8u * (unsigned)plans[i].pr.sub_m * (unsigned)plans[i].pr.sub_n;
+      plans[i].pr.group_begin = (int)groups_total;
+      for (unsigned j = 0; j < gi; ++j) wg_prob.push_back((int)i);
+      groups_total += gi;
+      preps[prep_of[i]].rs = (size_t)plans[i].pr.rs;
+    }
+    if (flow_total) {
+      flow_cfg.planes = planes;
+      flow_cfg.rt = rt;
+      flow_cfg.lds_bytes = pflds;
+      flow_cfg.grid = flow_total;
+      flow_cfg.waves = pfw;
+      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt);
+    }
+  } else if (variant != DECODE_KSPLIT) {
     const unsigned per = variant == DECODE_FLOW ? fper : tpw;
     for (size_t i = 0; i < count; ++i) {
       const unsigned gi = ((unsigned)plans[i].pr.n_tiles + per - 1) / per;
@@ -889,7 +949,8 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   g->ctx = ctx;
   int rc = dev_malloc(ws_bytes, &g->ws);
   const size_t wg_prob_off = count * sizeof(TkProblem) + preps.size() * sizeof(TkPrep);
-  if (!rc) rc = dev_malloc(wg_prob_off + wg_prob.size() * sizeof(int), &g->tables);
+  const size_t flow_wg_prob_off = wg_prob_off + wg_prob.size() * sizeof(int);
+  if (!rc) rc = dev_malloc(flow_wg_prob_off + flow_wg_prob.size() * sizeof(int), &g->tables);
   if (rc) {
     if (g->ws) (void)hipFree(g->ws);
     delete g;
@@ -900,7 +961,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     const size_t R = preps[j].R, nb = preps[j].nb, m = (size_t)preps[j].m;
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     uint8_t *base = (uint8_t *)g->ws + prep_off[j];
-    preps[j].ap = (int8_t *)base; base += al(R * nb * 256);
+    preps[j].ap = (int8_t *)base; base += al((R + 16) * nb * 256);
     preps[j].rowsum = (int32_t *)base; base += al(R * 4);
     preps[j].act_scale = (float *)base; base += al(m * 4);
     preps[j].aux = (float *)base; base += al(m * 4);
@@ -932,12 +993,18 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   if (e == hipSuccess && !wg_prob.empty())
     e = hipMemcpy((uint8_t *)g->tables + wg_prob_off, wg_prob.data(), wg_prob.size() * sizeof(int),
                   hipMemcpyHostToDevice);
+  if (e == hipSuccess && !flow_wg_prob.empty())
+    e = hipMemcpy((uint8_t *)g->tables + flow_wg_prob_off, flow_wg_prob.data(), flow_wg_prob.size() * sizeof(int),
+                  hipMemcpyHostToDevice);
   if (e != hipSuccess) {
     (void)hipFree(g->ws);
     (void)hipFree(g->tables);
     delete g;
     return tk_fail(TK_ERR_BACKEND, "tk_group_create: %s", hipGetErrorString(e));
   }
+  g->has_flow_part = !flow_wg_prob.empty();
+  g->flow_wg_prob_off = flow_wg_prob_off;
+  g->flow_cfg = flow_cfg;
   g->variant = variant;
   g->wg_prob_off = wg_prob_off;
   g->nprobs = (int)count;
@@ -947,6 +1014,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   g->cfg.planes = planes;
   g->cfg.rt = rt;
   g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
+  if (variant == DECODE_GEMM) g->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();
   g->cfg.grid = variant == DECODE_KSPLIT ? tiles : groups_total;
   g->cfg.waves = fw;
   {
@@ -970,7 +1038,12 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
   if (do_prep) HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_rows));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
-  if (do_main && g->variant == DECODE_FLOW)
+  if (do_main && g->has_flow_part)
+    HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),
+                          g->flow_cfg));
+  if (do_main && g->variant == DECODE_GEMM)
+    HIPCHK(tk_launch_gemm(ctx->stream, nullptr, probs, wg_prob, g->cfg));
+  else if (do_main && g->variant == DECODE_FLOW)
     HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, wg_prob, g->cfg));
   else if (do_main && g->variant == DECODE_STREAM)
     HIPCHK(tk_launch_stream(ctx->stream, nullptr, probs, wg_prob, g->cfg));

@@ -99,8 +99,8 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
 int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
 int tk_flow_ring(const int *nbs, const double *weights, int count, int rt);
-hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
-                          unsigned grid_n);
+hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                          const TkLaunchCfg &cfg);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);
 hipError_t tk_launch_copy(hipStream_t s, void *dst, const void *src, size_t bytes);
 #ifdef __cplusplus

@@ -755,12 +755,27 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
 #define TK_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 
 template <int P, int NT>
-__device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)[4][NT * P], uint8_t *smem, int tid, int bm,
-                                                 int bn);
+__device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
+                                                 v4i (&acc)[4][NT * P], uint8_t *smem, int tid, int bm, int bn);
 
-template <int P, int NT>
+// TABLE: a grouped launch; the workgroup finds its problem through wg_prob and counts its position
+// from the problem's first workgroup (a multiple of 8, so the XCD of a workgroup is unchanged).
+template <int P, int NT, bool TABLE>
 __global__ __launch_bounds__(TK_GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(TK_GEMM_OCC, TK_GEMM_OCC))) void
-tk_gemm_kernel(const TkProblem pr) {
+tk_gemm_kernel(const TkProblem single, const TkProblem *__restrict__ table, const int *__restrict__ wg_prob) {
+  const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
+  // local copies: a field read through the table pointer would be fetched again after every store
+  const TkHot hot = make_hot(pr);
+  const uint8_t *codes[P];
+  const float *scales[P];
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    codes[p] = pr.codes[p];
+    scales[p] = pr.scales[p];
+  }
+  const int8_t *ap = pr.ap;
+  const int rs = pr.rs, n_tiles = pr.n_tiles;
+  const unsigned wg = blockIdx.x - (TABLE ? (unsigned)pr.group_begin : 0u);
   constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, NB = NT * P;
   constexpr int SEGS = 16 / TK_GEMM_WAVES;  // 1-KiB A segments (one (j,g) pair x 64 rows) per wave per block
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // three A blocks of 16 KiB
@@ -770,7 +785,7 @@ tk_gemm_kernel(const TkProblem pr) {
   // XCD-aware tile order: consecutive workgroup ids go round-robin to the 8 XCDs, each with its own
   // L2. XCD x = id % 8 gets a compact sub-grid of sub_m x sub_n tiles, so the A row blocks and the
   // weight column blocks it touches stay resident in that L2 instead of every XCD streaming all.
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int xcd = wg & 7, slot = wg >> 3;
   const int bm = (xcd % pr.xr) * pr.sub_m + slot % pr.sub_m;
   const int bn = (xcd / pr.xr) * pr.sub_n + slot / pr.sub_m;
   if (bm >= pr.grid_m || bn >= pr.grid_n) return;
@@ -780,7 +795,7 @@ tk_gemm_kernel(const TkProblem pr) {
   // weight chunk offsets inside a plane (tiles past the end re-read the last tile; results dropped)
   unsigned woff[NT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) woff[nt] = ((unsigned)min(tile0 + nt, pr.n_tiles - 1) * (unsigned)nb * 64u + lane) * 16u;
+  for (int nt = 0; nt < NT; ++nt) woff[nt] = ((unsigned)min(tile0 + nt, n_tiles - 1) * (unsigned)nb * 64u + lane) * 16u;
 
   // A rows travel global -> LDS directly (no registers): one wave-wide 16-byte-per-lane load lands
   // as 1 KiB at a wave-uniform LDS address, which is exactly one (j,g) segment of 64 rows. Rows past
@@ -791,7 +806,7 @@ tk_gemm_kernel(const TkProblem pr) {
 #pragma unroll
     for (int u = 0; u < SEGS; ++u) {
       const int seg = wave_u * SEGS + u;
-      const uint8_t *seg_base = (const uint8_t *)pr.ap + ((size_t)kb * 16 + seg) * (size_t)pr.rs * 16;  // wave-uniform
+      const uint8_t *seg_base = (const uint8_t *)ap + ((size_t)kb * 16 + seg) * (size_t)rs * 16;  // wave-uniform
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(seg_base + a_lane),
                                        (__attribute__((address_space(3))) void *)(smem + ((size_t)slot3 * A4 + (size_t)seg * ROWS) * 16),
                                        16, 0, 0);
@@ -804,13 +819,13 @@ tk_gemm_kernel(const TkProblem pr) {
   // Indices past the end are clamped; what is read for them is never used.
   constexpr int CST = 3 * A4 * 16;  // int rs[64] | float as[64] | int exp[64] | uint flag[64]
   {
-    const bool int8_in = pr.mode == TK_MODE_INT8;
-    const int row_c = min(row0 + lane, R - 1), tok_c = min((row0 >> 2) + lane, pr.M - 1);
+    const bool int8_in = hot.mode == TK_MODE_INT8;
+    const int row_c = min(row0 + lane, R - 1), tok_c = min((row0 >> 2) + lane, hot.M - 1);
     const void *src = nullptr;
-    if (wave_u == 0) src = pr.rowsum + row_c;
-    else if (wave_u == 1) src = (int8_in && pr.act_scale) ? (const void *)(pr.act_scale + row_c) : nullptr;
-    else if (wave_u == 2) src = int8_in ? nullptr : (const void *)(pr.exps + tok_c);
-    else if (wave_u == 3) src = pr.flags ? (const void *)(pr.flags + (int8_in ? row_c : tok_c)) : nullptr;
+    if (wave_u == 0) src = hot.rowsum + row_c;
+    else if (wave_u == 1) src = (int8_in && hot.act_scale) ? (const void *)(hot.act_scale + row_c) : nullptr;
+    else if (wave_u == 2) src = int8_in ? nullptr : (const void *)(hot.exps + tok_c);
+    else if (wave_u == 3) src = hot.flags ? (const void *)(hot.flags + (int8_in ? row_c : tok_c)) : nullptr;
     if (src && wave_u < 4)
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                        (__attribute__((address_space(3))) void *)(smem + CST + wave_u * 256), 4, 0, 0);
@@ -846,7 +861,7 @@ tk_gemm_kernel(const TkProblem pr) {
       for (int p = 0; p < P; ++p)
         asm volatile("global_load_dwordx4 %0, %1, %2"
                      : "=v"(w[nt * P + p])
-                     : "v"(woff[nt] + (unsigned)kb * (unsigned)TK_CHUNK_BYTES), "s"(pr.codes[p]));
+                     : "v"(woff[nt] + (unsigned)kb * (unsigned)TK_CHUNK_BYTES), "s"(codes[p]));
   };
   auto tie_w = [&](v4i (&w)[NB]) {
 #pragma unroll
@@ -918,23 +933,24 @@ tk_gemm_kernel(const TkProblem pr) {
   // the prologue would keep a dozen registers alive across the main loop, which has none to spare.
   unsigned tid_e = threadIdx.x;
   asm volatile("" : "+v"(tid_e));
-  tk_gemm_epilogue<P, NT>(pr, acc, smem, (int)tid_e, bm, bn);
+  tk_gemm_epilogue<P, NT>(pr, hot, scales, acc, smem, (int)tid_e, bm, bn);
 }
 
 template <int P, int NT>
-__device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)[4][NT * P], uint8_t *smem, int tid, int bm,
-                                                 int bn) {
+__device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
+                                                 v4i (&acc)[4][NT * P], uint8_t *smem, int tid, int bm, int bn) {
   constexpr int RT = 4, ROWS = RT * 16, A4 = 16 * ROWS, CST = 3 * A4 * 16;
   const int wave = tid >> 6, lane = tid & 63, i = lane & 15, g = lane >> 4;
-  const int R = pr.R, row0 = bm * ROWS, tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+  const int R = hot.R, row0 = bm * ROWS, tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+  const int n_tiles = (hot.n + 15) >> 4;
   // Epilogue. The row constants are in LDS since the prologue: one 16-byte read per row tile.
   const int *cst_rs = (const int *)(smem + CST);
   const float *cst_as = (const float *)(smem + CST + 256);
   const int *cst_exp = (const int *)(smem + CST + 512);
   const int *cst_flag = (const int *)(smem + CST + 768);
   unsigned my_flag = 0;
-  if (pr.flags && tid < ROWS) {
-    const bool in_range = pr.mode == TK_MODE_INT8 ? row0 + tid < R : (row0 >> 2) + tid < pr.M;
+  if (hot.flags && tid < ROWS) {
+    const bool in_range = hot.mode == TK_MODE_INT8 ? row0 + tid < R : (row0 >> 2) + tid < hot.M;
     if (in_range) my_flag = cst_flag[tid] ? 1u : 0u;
   }
   float sc[NT][P];
@@ -942,7 +958,7 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)
   for (int nt = 0; nt < NT; ++nt) {
     const int n = (tile0 + nt) * 16 + i;
 #pragma unroll
-    for (int p = 0; p < P; ++p) sc[nt][p] = (tile0 + nt < pr.n_tiles && n < pr.n) ? pr.scales[p][n] : 0.0f;
+    for (int p = 0; p < P; ++p) sc[nt][p] = (tile0 + nt < n_tiles && n < hot.n) ? gload(scales[p] + n) : 0.0f;
   }
   const int wg_flag = __syncthreads_or((int)my_flag);
   auto row_const = [&](int rt) {
@@ -954,7 +970,7 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)
     rc.exp = cst_exp[rt * 4 + g];
     rc.flag = 0;
     if (wg_flag) {
-      if (pr.mode == TK_MODE_INT8) {
+      if (hot.mode == TK_MODE_INT8) {
         const v4i f4 = *(const v4i *)(cst_flag + rt * 16 + 4 * g);
         rc.flag = (f4.x ? 1u : 0u) | (f4.y ? 2u : 0u) | (f4.z ? 4u : 0u) | (f4.w ? 8u : 0u);
       } else {
@@ -969,20 +985,20 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)
   // output are 16-byte aligned, the finished values are staged through LDS instead (free after the
   // last barrier of the main loop) and leave as whole 16-byte pieces of contiguous row segments:
   // every store instruction of a wave then covers full cache lines.
-  const int esz = pr.out_dtype == TK_BF16 ? 2 : 4;
-  const bool staged = (((size_t)pr.n * esz) & 15) == 0 && (((size_t)pr.out) & 15) == 0;
+  const int esz = hot.out_dtype == TK_BF16 ? 2 : 4;
+  const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0;
   if (staged) {
     constexpr int WG_COLS = TK_GEMM_WAVES * NT * 16;
-    const bool int8_mode = pr.mode == TK_MODE_INT8 || pr.out_dtype == TK_I32;
+    const bool int8_mode = hot.mode == TK_MODE_INT8 || hot.out_dtype == TK_I32;
     const int halves = esz == 4 ? 2 : 1;            // 4-byte outputs take the 64 rows in two halves
     const int rt_per_half = RT / halves;
     const int orows_rt = int8_mode ? 16 : 4;        // output rows per row tile (4 digit rows = 1 token)
     const int stride = WG_COLS * esz + 16;          // padded: the 4 lane groups of a wave hit different banks
     const int pieces_row = WG_COLS * esz / 16;      // 16-byte pieces per staged row (a power of two)
     const int out_row0 = int8_mode ? row0 : (row0 >> 2);
-    const int out_rows = int8_mode ? pr.R : pr.M;
+    const int out_rows = int8_mode ? hot.R : hot.M;
     const int col0 = bn * WG_COLS;
-    const bool has_as = pr.act_scale != nullptr;
+    const bool has_as = hot.act_scale != nullptr;
     for (int h = 0; h < halves; ++h) {
       if (h > 0) __syncthreads();
 #pragma unroll
@@ -996,11 +1012,11 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)
           v4i av[P];
 #pragma unroll
           for (int p = 0; p < P; ++p) av[p] = acc[rt][nt * P + p];
-          if (pr.out_dtype == TK_I32) {
+          if (hot.out_dtype == TK_I32) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
               *(int32_t *)(smem + (size_t)(rl * 16 + 4 * g + r) * stride + cl * 4) = av[0][r] - rc.rs[r];
-          } else if (pr.mode == TK_MODE_INT8) {
+          } else if (hot.mode == TK_MODE_INT8) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const float f = int8_value<P>(av, r, sc[nt], rc, has_as);
@@ -1021,11 +1037,11 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)
         const int rl = pc / pieces_row, piece = pc - rl * pieces_row;
         const int orow = out_row0 + h * rows_h + rl;
         const int c = col0 + piece * per16;
-        if (orow >= out_rows || c >= pr.n) continue;
-        if (wg_flag && pr.out_dtype != TK_I32 && pr.flags[orow]) continue;  // written by exact_rows below
+        if (orow >= out_rows || c >= hot.n) continue;
+        if (wg_flag && hot.out_dtype != TK_I32 && gload(hot.flags + orow)) continue;  // written by exact_rows below
         const uint8_t *src = smem + (size_t)rl * stride + piece * 16;
-        uint8_t *dst = (uint8_t *)pr.out + ((size_t)orow * pr.n + c) * esz;
-        *(uint4 *)dst = *(const uint4 *)src;  // n is a multiple of per16 here, so a piece never straddles the row end
+        uint8_t *dst = (uint8_t *)hot.out + ((size_t)orow * hot.n + c) * esz;
+        *(TK_GLOBAL v4u *)dst = *(const v4u *)src;  // n is a multiple of per16 here, so a piece never straddles the row end
       }
     }
   } else {
@@ -1036,11 +1052,11 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, v4i (&acc)
       for (int nt = 0; nt < NT; ++nt) {
         const int t = tile0 + nt;
         const int n = t * 16 + i;
-        if (t >= pr.n_tiles || n >= pr.n) continue;
+        if (t >= n_tiles || n >= hot.n) continue;
         v4i av[P];
 #pragma unroll
         for (int p = 0; p < P; ++p) av[p] = acc[rt][nt * P + p];
-        flow_epilogue<P>(pr, n, row0 + rt * 16 + 4 * g, av, sc[nt], rc);
+        flow_epilogue<P>(hot, n, row0 + rt * 16 + 4 * g, av, sc[nt], rc);
       }
     }
   }
@@ -1611,17 +1627,27 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
 int tk_gemm_lds_bytes(void) { return 3 * 16 * 64 * 16 + 1024; }  // three A blocks + the row constants
 int tk_gemm_tiles_per_wg(int planes) { return TK_GEMM_WAVES * (planes == 1 ? 4 : (planes == 2 ? 2 : 1)); }
 
-hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg, unsigned grid_m,
-                          unsigned grid_n) {
-  if (!grid_m || !grid_n) return hipSuccess;
-  dim3 grid(8u * (unsigned)single->sub_m * (unsigned)single->sub_n), block(TK_GEMM_THREADS);
+// single != null: one problem, grid from its XCD split. table != null: a grouped launch of cfg.grid
+// workgroups (every member's share is a multiple of 8).
+hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                          const TkLaunchCfg &cfg) {
+  TkProblem dummy = {};
+  const TkProblem &sg = single ? *single : dummy;
+  const unsigned wgs = table ? cfg.grid : 8u * (unsigned)sg.sub_m * (unsigned)sg.sub_n;
+  if (!wgs) return hipSuccess;
+  dim3 grid(wgs), block(TK_GEMM_THREADS);
+#define TK_GEMM_CASE(PP, NTT)                                                                                 \
+  if (table) hipLaunchKernelGGL((tk_gemm_kernel<PP, NTT, true>), grid, block, cfg.lds_bytes, s, sg, table, wg_prob); \
+  else hipLaunchKernelGGL((tk_gemm_kernel<PP, NTT, false>), grid, block, cfg.lds_bytes, s, sg, table, wg_prob);      \
+  break;
   switch (cfg.planes) {
-    case 1: hipLaunchKernelGGL((tk_gemm_kernel<1, 4>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 2: hipLaunchKernelGGL((tk_gemm_kernel<2, 2>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 3: hipLaunchKernelGGL((tk_gemm_kernel<3, 1>), grid, block, cfg.lds_bytes, s, *single); break;
-    case 4: hipLaunchKernelGGL((tk_gemm_kernel<4, 1>), grid, block, cfg.lds_bytes, s, *single); break;
+    case 1: TK_GEMM_CASE(1, 4)
+    case 2: TK_GEMM_CASE(2, 2)
+    case 3: TK_GEMM_CASE(3, 1)
+    case 4: TK_GEMM_CASE(4, 1)
     default: return hipErrorInvalidValue;
   }
+#undef TK_GEMM_CASE
   return hipGetLastError();
 }
 
