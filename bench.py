@@ -326,7 +326,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--no-extra", action="store_true", help="skip the prefill GEMM and projection-stack legs")
+    ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
+    ap.add_argument("--extra-legs", default="config1,prefill,stack,config5",
+                    help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a plain 1 GiB device copy kernel 3 times (scale for hardware traffic counters)")
@@ -375,10 +377,15 @@ def main():
         src.free()
         dst.free()
     if not args.no_extra:
-        out["extra"] = {"config1_f32_batch1": bench_config1(T, be, rng),
-                        "prefill_gemm": bench_prefill(T, be, rng, 2048, 2560, 6912),
-                        "projection_stack": bench_stack(T, be, rng),
-                        "config5_three_planes": bench_config5(T, be, rng)}
+        legs = {"config1": ("config1_f32_batch1", lambda: bench_config1(T, be, rng)),
+                "prefill": ("prefill_gemm", lambda: bench_prefill(T, be, rng, 2048, 2560, 6912)),
+                "stack": ("projection_stack", lambda: bench_stack(T, be, rng)),
+                "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng))}
+        out["extra"] = {}
+        for leg in [x for x in args.extra_legs.split(",") if x]:
+            if leg not in legs:
+                sys.exit(f"bench.py: unknown leg `{leg}` (choose from {','.join(legs)})")
+            out["extra"][legs[leg][0]] = legs[leg][1]()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np.random.default_rng(1))
     be.close()

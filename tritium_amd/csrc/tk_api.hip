@@ -435,12 +435,14 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)tk_flow_runs_per_wave(planes, rt);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
-  size_t target = lds_bytes * (size_t)waves * (size_t)waves / 4;
+  size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 ? 2 : 4);
   if (target < 128 * 1024) target = 128 * 1024;
   size_t s = 1;
   while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
-  // keep at least two workgroups per CU
-  while (s > 1 && total_tiles / (per_s * s) < 2u * (unsigned)ctx->info.compute_units) --s;
+  // keep every CU supplied: two four-wave workgroups each, or one eight-wave workgroup (those fill
+  // the LDS of a CU alone, and a single round of them has no change-over in the middle of the launch)
+  const unsigned per_cu = waves >= 8 ? 1u : 2u;
+  while (s > 1 && total_tiles / (per_s * s) < per_cu * (unsigned)ctx->info.compute_units) --s;
   return (int)s;
 }
 

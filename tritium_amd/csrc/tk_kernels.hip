@@ -601,27 +601,32 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
   // chunk's first use leaves exactly the D younger positions in flight. The chunks of a run are
   // consecutive in memory, so a request is one running byte offset per run, advanced by 1 KiB when
   // the requested position is a real one; a padding position asks again for the chunk the next real
-  // position will get, and requests past the end of the plane are clamped to its last chunk. The
-  // host picks DR so that padding is rare.
+  // position will get, and requests past the end of the run ask again for its last chunk (a cache
+  // hit: no traffic from memory). The host picks DR so that padding is rare.
   constexpr int D = DR - 1;
   const int nbpad = (nb + DR - 1) / DR * DR;
   const int first = ((blockIdx.x - pr.group_begin) * NW + wave) * TW * S;  // first tile of this wave
-  const unsigned last_off = ((unsigned)n_tiles * (unsigned)nb - 1u) * 1024u + (unsigned)lane * 16u;
+  const unsigned plane_last = (unsigned)n_tiles * (unsigned)nb - 1u;  // last chunk of the plane
   // The TW runs of a wave interleave tile by tile (run tw takes tiles first+tw, first+tw+TW, ...), so
   // that what the wave finishes together is TW*16 adjacent output columns (its stores then fill
   // whole cache lines between them); at the first position of a tile a run therefore skips the
   // (TW-1) tiles of its siblings.
   const unsigned skip = (unsigned)(TW - 1) * (unsigned)nb * 1024u;
-  unsigned roff[TW];  // byte offset inside a plane of this lane's piece of the next chunk to request
+  unsigned roff[TW];      // byte offset inside a plane of this lane's piece of the next chunk to request
+  unsigned last_off[TW];  // ... of the last chunk of the run: requests past it ask for that chunk again
 #pragma unroll
-  for (int tw = 0; tw < TW; ++tw) roff[tw] = (unsigned)(first + tw) * (unsigned)nb * 1024u + (unsigned)lane * 16u - skip;
+  for (int tw = 0; tw < TW; ++tw) {
+    roff[tw] = (unsigned)(first + tw) * (unsigned)nb * 1024u + (unsigned)lane * 16u - skip;
+    const unsigned run_last = (unsigned)(first + (S - 1) * TW + tw) * (unsigned)nb + (unsigned)nb - 1u;
+    last_off[tw] = min(run_last, plane_last) * 1024u + (unsigned)lane * 16u;
+  }
 
   uint4 ring[DR][TW][P];
   auto request = [&](int slot, bool real, bool tile_start) {
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       roff[tw] += tile_start ? skip : 0u;
-      const unsigned off = min(roff[tw], last_off);
+      const unsigned off = min(roff[tw], last_off[tw]);
 #pragma unroll
       for (int p = 0; p < P; ++p) ring[slot][tw][p] = gload16(codes[p] + (size_t)off);
       roff[tw] += real ? 1024u : 0u;
@@ -1585,23 +1590,29 @@ static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProb
 // lock-step runs per wave of the flow kernel for a (planes, rt) pair
 int tk_flow_runs_per_wave(int planes, int rt) { return (rt >= 4 && planes <= 2) ? 2 : 1; }
 
-// Ring size of the flow kernel for launches whose K block counts are nbs[0..count): the compiled
-// size (2..5 positions) that pads the fewest positions, weighted by each problem's chunk count.
-// Ties go to the shallow ring, which costs the fewest registers (more waves per SIMD did more for
-// the measured bandwidth than more loads per wave), except at two row tiles, where 64 KiB of LDS
-// per workgroup caps the CU at eight waves and the deeper ring measured better.
+// Ring size of the flow kernel (2..5 positions) for launches whose K block counts are nbs[0..count).
+// A deeper ring keeps more loads in flight per wave and costs registers, i.e. waves per SIMD.
+// Measured on K=2048 N=8192 x 2 planes: one row tile likes 5 positions, two row tiles 4, four row
+// tiles (250 registers, eight waves per CU whatever the ring) 2. A ring that does not divide a K
+// block count pads that problem's tiles with idle positions; a candidate is taken in the order of
+// preference unless it pads more than a quarter of the positions (weighted by each problem's chunk
+// count), and if all do, the one that pads least.
 int tk_flow_ring(const int *nbs, const double *weights, int count, int rt) {
-  const int shallow[4] = {2, 4, 3, 5}, deep[4] = {4, 2, 3, 5};
-  const int *cand = rt == 2 ? deep : shallow;
+  const int pref1[4] = {5, 4, 3, 2}, pref2[4] = {4, 5, 3, 2}, pref4[4] = {2, 3, 4, 5};
+  const int *cand = rt == 1 ? pref1 : (rt == 2 ? pref2 : pref4);
   int best = cand[0];
   double best_waste = -1.0;
   for (int c = 0; c < 4; ++c) {
-    double waste = 0.0;
+    double waste = 0.0, total = 0.0;
     for (int x = 0; x < count; ++x) {
       const int nb = nbs[x], pad = (nb + cand[c] - 1) / cand[c] * cand[c];
-      waste += (weights ? weights[x] : 1.0) * (double)(pad - nb) / (double)(nb > 0 ? nb : 1);
+      const double w = weights ? weights[x] : 1.0;
+      waste += w * (double)(pad - nb) / (double)(pad > 0 ? pad : 1);
+      total += w;
     }
-    if (best_waste < 0.0 || waste < best_waste - 1e-12) {
+    waste = total > 0.0 ? waste / total : 0.0;
+    if (waste <= 0.25) return cand[c];
+    if (best_waste < 0.0 || waste < best_waste) {
       best_waste = waste;
       best = cand[c];
     }
