@@ -410,11 +410,11 @@ __global__ __launch_bounds__(TK_WG) void tk_stream_kernel(TkProblem single, cons
 
 // ------------------------------------------------------------------------------------------
 // decode GEMV, flow form: the bandwidth kernel. Requirements: all K blocks of the operand rows fit
-// in LDS. A wave owns TW runs of S consecutive output tiles; in the device layout the chunks of
-// consecutive tiles are consecutive in memory, so each run is ONE contiguous byte stream of
-// S*nb KiB, walked with a D-deep ring of 128-bit loads that never drains at tile boundaries.
-// Per-row constants are loaded once per wave, per-tile scales at the start of the tile, so the
-// epilogue of a tile waits on nothing that was issued behind the stream's prefetches.
+// in LDS. A wave owns TW runs of S output tiles; in the device layout the chunks of consecutive
+// tiles are consecutive in memory, so a run is a byte stream with a fixed skip at tile starts,
+// walked with a ring of 128-bit loads that never drains at tile boundaries. Per-row constants are
+// loaded once per wave, per-tile scales at the start of the tile, so the epilogue of a tile waits
+// on nothing that was issued behind the stream's prefetches.
 // ------------------------------------------------------------------------------------------
 
 // The fields of a problem that the epilogues read, copied into registers once per kernel: read through
@@ -738,13 +738,12 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
 // ------------------------------------------------------------------------------------------
 // prefill GEMM. Workgroup tile = 64 operand rows x (TK_GEMM_WAVES waves * NT tiles * 16 outputs),
 // all P planes of a tile in the same wave (P*NT = 4 accumulator tiles per row tile, so one LDS read
-// of an A operand feeds 4 MFMAs). A blocks of 256 k are double-buffered in LDS: while the MFMAs of
-// block kb run, the global loads of block kb+1 (A rows, and the 2-bit weight chunks, both into
-// registers) are in flight; one barrier per block. Weights never pass through LDS: each wave
-// streams the chunks of its own output tiles and expands a dword into an MFMA operand when needed.
-// A single wave cannot keep the MFMA pipe full (measured: ~25 cycles per 16x16x64 issue from one
-// wave, ~18 from two), and waves of one workgroup stall together at its barrier, so the kernel is
-// sized for several independent workgroups per CU.
+// of an A operand feeds 4 MFMAs). A blocks of 256 k travel global -> LDS by DMA into three slots,
+// two blocks ahead of the MFMAs; the 2-bit weight chunks of the wave's own tiles go straight to
+// registers (never through LDS), also two blocks ahead, and a dword is expanded into an MFMA operand
+// when needed; one barrier per block. A single wave cannot keep the MFMA pipe full (measured: ~25
+// cycles per 16x16x64 issue from one wave, ~18 from two), and waves of one workgroup stall
+// together at its barrier, so the kernel is sized for several independent workgroups per CU.
 // ------------------------------------------------------------------------------------------
 
 #ifndef TK_GEMM_WAVES
