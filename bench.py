@@ -213,6 +213,39 @@ def bench_config1(T, be, rng, iters=200):
             "device_resident_GB/s": round(by / ms / 1e6, 1)}
 
 
+def bench_sweep_a8(T, be, rng, iters=100):
+    """The headline sweep again under the other contract: activations quantized per token to int8
+    (what TernaryLinear::forward asks of a backend, mpgemm_with_act_quant), bit-exact to the CPU. One
+    operand row per token instead of the four digit rows of the float contract, so every batch size
+    of the sweep stays in the bandwidth regime. Kernel only, like `per_batch`."""
+    host = []
+    for _ in range(2):
+        planes = [T.pack_rows(ternary(rng, N2, K2, p0), N2, K2) for p0 in (0.4, 0.7)]
+        host.append((planes, [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)]))
+    layers = [be.linear(*host[i % 2], N2, K2) for i in range(COPIES)]
+    mmax = max(SWEEP)
+    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((mmax, K2)).astype(np.float32)), "bf16")
+            for _ in range(COPIES)]
+    outs = [be.empty(mmax * N2, "f32") for _ in range(COPIES)]
+    res, tot_b, tot_ms = {}, 0, 0.0
+    for m in SWEEP:
+        g = be.group([(layers[i], acts[i], m, outs[i]) for i in range(COPIES)], 1, "bf16", "f32")
+        g.launch_parts(True, False)
+        ms = time_calls(be, lambda i: g.launch_parts(False, True), iters)
+        by = COPIES * algorithmic_bytes(m, N2, K2, PLANES2, 2, 4, a8=True)
+        res[str(m)] = {"GB/s": round(by / ms / 1e6, 1), "us_per_layer": round(ms * 1e3 / COPIES, 3)}
+        tot_b += by
+        tot_ms += ms
+        g.destroy()
+    for x in acts + outs:
+        x.free()
+    for l in layers:
+        l.free()
+    return {"workload": "the headline sweep with per-token int8 activations (W1.58A8), decode kernel only",
+            "per_batch": res, "sweep_GB/s": round(tot_b / tot_ms / 1e6, 1),
+            "frac_of_hbm_peak": round(tot_b / tot_ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+
 def bench_config5(T, be, rng):
     """configs[4]: three additive planes (P(0)=0.4/0.7/0.85), hidden 5120, FFN 17408. Decode at batch
     64 over the up and down projections of 8 distinct layers in one grouped launch (W1.58A8, bf16 in
@@ -327,7 +360,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="config1,prefill,stack,config5",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -377,7 +410,8 @@ def main():
         src.free()
         dst.free()
     if not args.no_extra:
-        legs = {"config1": ("config1_f32_batch1", lambda: bench_config1(T, be, rng)),
+        legs = {"sweep_a8": ("decode_sweep_int8_activations", lambda: bench_sweep_a8(T, be, rng)),
+                "config1": ("config1_f32_batch1", lambda: bench_config1(T, be, rng)),
                 "prefill": ("prefill_gemm", lambda: bench_prefill(T, be, rng, 2048, 2560, 6912)),
                 "stack": ("projection_stack", lambda: bench_stack(T, be, rng)),
                 "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng))}
