@@ -1079,6 +1079,366 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, const TkHo
 }
 
 // ------------------------------------------------------------------------------------------
+// prefill GEMM on v_mfma_i32_32x32x32_i8. Same workgroup tile, pipeline and LDS layout as the
+// kernel above; the matrix instruction is the 32x32 one, which this chip sustains at 4.0 POPS where
+// the 16x16x64 form stops at 3.0 (one wave per SIMD is enough to reach it). Operand mapping, with
+// lane L = 32*kappa + 16*h + r:
+//   B (32 weight rows x 32 k): two 16-row tiles side by side. Lane L takes its 16 bytes from tile
+//     h of the pair, row r, 16-byte piece g = 2*l + kappa of that row's 64 code bytes (l = 0,1: two
+//     loads per pair and K block; the device weight layout is unchanged, only the lane -> address
+//     map differs). Dword j of load l expands to the operand of k step (l, j): 8 steps per block.
+//   A (32 operand rows x 32 k): lane L reads piece (kb, j, g = 2*l + kappa) of row 32*rt2 + (L & 31),
+//     the same 16-byte pieces the 16x16x64 kernel reads, so the operand row layout is unchanged too.
+//   D: register i of lane L is row 32*rt2 + 8*(i/4) + 4*kappa + i%4, column (pair, h, r): four
+//     consecutive registers are four consecutive rows, as the epilogues expect.
+// The tiles of a pair belong to the same plane (tile index x = p*NT + nt, pairs (2y, 2y+1)), so the
+// planes of one output meet in one lane; NT is even.
+// ------------------------------------------------------------------------------------------
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int P, int NT>
+__device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
+                                                   v16i (&acc)[2][NT * P / 2], uint8_t *smem, int tid, int bm, int bn);
+
+#ifndef TK_GEMM32_STAGES
+#define TK_GEMM32_STAGES 3
+#endif
+#ifndef TK_GEMM_BAND
+#define TK_GEMM_BAND 8
+#endif
+#ifndef TK_GEMM32_OCC3
+#define TK_GEMM32_OCC(P) ((P) >= 3 ? 2 : 3)
+#endif
+
+template <int P, int NT, bool TABLE>
+__global__ __launch_bounds__(TK_GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(TK_GEMM32_OCC(P), TK_GEMM32_OCC(P)))) void
+tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, const int *__restrict__ wg_prob) {
+  static_assert(NT % 2 == 0, "tiles are processed in pairs");
+  const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
+  const TkHot hot = make_hot(pr);
+  const uint8_t *codes[P];
+  const float *scales[P];
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    codes[p] = pr.codes[p];
+    scales[p] = pr.scales[p];
+  }
+  const int8_t *ap = pr.ap;
+  const int rs = pr.rs, n_tiles = pr.n_tiles;
+  const unsigned wg = blockIdx.x - (TABLE ? (unsigned)pr.group_begin : 0u);
+  constexpr int ROWS = 64, A4 = 16 * ROWS, NB = NT * P, NP = NB / 2, HP = NT / 2;  // HP pairs per plane
+  constexpr int SEGS = 16 / TK_GEMM_WAVES;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // three A blocks of 16 KiB + row constants
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, h = (lane >> 4) & 1, kappa = lane >> 5;
+  const int nb = pr.nb, R = pr.R;
+  // XCD x = id % 8 owns a compact sub-grid of sub_m x sub_n tiles. Inside it the slots walk bands of
+  // TK_GEMM_BAND row tiles: down the band first, then along the columns, so the ~100 workgroups an
+  // XCD holds at a time are a band x 12 patch (8 A row blocks + 12 weight column blocks to keep in
+  // its L2) instead of a full column strip (32 + 3).
+  const int xcd = wg & 7, slot = wg >> 3;
+  const int sub_m = pr.sub_m, sub_n = pr.sub_n;
+  const int band_sz = TK_GEMM_BAND * sub_n;
+  const int band = slot / band_sz, in_band = slot - band * band_sz;
+  const int band_rows = min(TK_GEMM_BAND, sub_m - band * TK_GEMM_BAND);  // the last band may be shorter
+  const int lm = band * TK_GEMM_BAND + in_band % band_rows, ln = in_band / band_rows;
+  const int bm = (xcd % pr.xr) * sub_m + lm;
+  const int bn = (xcd / pr.xr) * sub_n + ln;
+  if (lm >= sub_m || ln >= sub_n || bm >= pr.grid_m || bn >= pr.grid_n) return;
+  const int row0 = bm * ROWS;
+  const int tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+
+  // per pair: this lane's address of load l = 0 in K block 0 (load 1 is 512 bytes further, block kb
+  // kb KiB further); tiles past the end re-read the last tile (results dropped)
+  const uint8_t *wptr[NP];
+#pragma unroll
+  for (int y = 0; y < NP; ++y) {
+    const int p = y / HP, nt = (y % HP) * 2 + h;
+    wptr[y] = codes[p] + ((size_t)min(tile0 + nt, n_tiles - 1) * (size_t)nb * 64 + (size_t)(kappa * 16 + r16)) * 16;
+  }
+
+  const unsigned a_lane = (unsigned)min(row0 + lane, R - 1) * 16u;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto dma_block = [&](int kb, int slot3) {
+#pragma unroll
+    for (int u = 0; u < SEGS; ++u) {
+      const int seg = wave_u * SEGS + u;
+      const uint8_t *seg_base = (const uint8_t *)ap + ((size_t)kb * 16 + seg) * (size_t)rs * 16;  // wave-uniform
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(seg_base + a_lane),
+                                       (__attribute__((address_space(3))) void *)(smem + ((size_t)slot3 * A4 + (size_t)seg * ROWS) * 16),
+                                       16, 0, 0);
+    }
+  };
+
+  constexpr int CST = TK_GEMM32_STAGES * A4 * 16;  // int rs[64] | float as[64] | int exp[64] | uint flag[64]
+  {
+    const bool int8_in = hot.mode == TK_MODE_INT8;
+    const int row_c = min(row0 + lane, R - 1), tok_c = min((row0 >> 2) + lane, hot.M - 1);
+    const void *src = nullptr;
+    if (wave_u == 0) src = hot.rowsum + row_c;
+    else if (wave_u == 1) src = (int8_in && hot.act_scale) ? (const void *)(hot.act_scale + row_c) : nullptr;
+    else if (wave_u == 2) src = int8_in ? nullptr : (const void *)(hot.exps + tok_c);
+    else if (wave_u == 3) src = hot.flags ? (const void *)(hot.flags + (int8_in ? row_c : tok_c)) : nullptr;
+    if (src && wave_u < 4)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                       (__attribute__((address_space(3))) void *)(smem + CST + wave_u * 256), 4, 0, 0);
+  }
+
+  v16i acc[2][NP];
+#pragma unroll
+  for (int rt2 = 0; rt2 < 2; ++rt2)
+#pragma unroll
+    for (int y = 0; y < NP; ++y)
+#pragma unroll
+      for (int c = 0; c < 16; ++c) acc[rt2][y][c] = 0;
+
+  // operand loads as asm with explicit waits, as in the kernel above
+  auto lds_read = [&](v4i (&a)[2], unsigned addr, int off) {
+#pragma unroll
+    for (int rt2 = 0; rt2 < 2; ++rt2)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[rt2]) : "v"(addr), "n"(off + rt2 * 512));
+  };
+  auto lds_wait = [&](v4i (&a)[2]) {
+    asm volatile("s_waitcnt lgkmcnt(0)");
+#pragma unroll
+    for (int rt2 = 0; rt2 < 2; ++rt2) asm volatile("" : "+v"(a[rt2]));
+  };
+  auto load_w = [&](v4i (&w)[NP][2], int kb) {
+#pragma unroll
+    for (int y = 0; y < NP; ++y) {
+      const uint8_t *ptr = wptr[y] + (size_t)kb * TK_CHUNK_BYTES;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(w[y][0]) : "v"(ptr));
+      asm volatile("global_load_dwordx4 %0, %1, off offset:512" : "=v"(w[y][1]) : "v"(ptr));
+    }
+  };
+  auto tie_w = [&](v4i (&w)[NP][2]) {
+#pragma unroll
+    for (int y = 0; y < NP; ++y) {
+      asm volatile("" : "+v"(w[y][0]));
+      asm volatile("" : "+v"(w[y][1]));
+    }
+  };
+
+  // NS register sets and NS LDS slots rotate by name (the loop is unrolled NS times): block kb uses
+  // set and slot kb % NS; at its top the weight chunks and the A DMA of block kb+NS-1 are issued into
+  // the set and slot block kb-1 just left; at its end everything of block kb+1 must have landed,
+  // the younger blocks stay in flight.
+  constexpr int NS = TK_GEMM32_STAGES;
+  v4i wset[NS][NP][2];
+#pragma unroll
+  for (int q = 0; q < NS; ++q)
+#pragma unroll
+    for (int y = 0; y < NP; ++y)
+#pragma unroll
+      for (int l = 0; l < 2; ++l) wset[q][y][l] = v4i{0, 0, 0, 0};
+  // wait until at most `blocks` of the youngest issued blocks are still in flight
+  auto wait_blocks = [&](int blocks) {
+    if (blocks <= 0) asm volatile("s_waitcnt vmcnt(0)");
+    else if (blocks == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SEGS + NB));
+    else if (blocks == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (SEGS + NB)));
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (SEGS + NB)));
+  };
+#pragma unroll
+  for (int q = 0; q < NS - 1; ++q)
+    if (q < nb) {
+      load_w(wset[q], q);
+      dma_block(q, q);
+    }
+  wait_blocks(min(NS - 2, nb - 1));  // block 0 has landed
+#pragma unroll
+  for (int q = 0; q < NS; ++q) tie_w(wset[q]);
+  __builtin_amdgcn_s_barrier();
+
+  const unsigned lds_lane = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t *)smem + (unsigned)(kappa * ROWS + (lane & 31)) * 16u;
+  auto block = [&](auto cur_c, int kb) {
+    constexpr int cur = decltype(cur_c)::value, nxt = (cur + NS - 1) % NS, n1 = (cur + 1) % NS;
+    if (kb + NS - 1 < nb) {
+      load_w(wset[nxt], kb + NS - 1);
+      dma_block(kb + NS - 1, nxt);
+    }
+    v4i a[2];
+#pragma unroll
+    for (int l = 0; l < 2; ++l)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        lds_read(a, lds_lane, cur * (A4 * 16) + (j * 4 + 2 * l) * (ROWS * 16));
+        lds_wait(a);
+#pragma unroll
+        for (int y = 0; y < NP; ++y) {
+          const v4i b = expand_codes((uint32_t)wset[cur][y][l][j]);
+#pragma unroll
+          for (int rt2 = 0; rt2 < 2; ++rt2)
+            acc[rt2][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[rt2], b, acc[rt2][y], 0, 0, 0);
+        }
+      }
+    // blocks issued after kb+1 and still allowed in flight: kb+2 .. min(kb+NS-1, nb-1)
+    wait_blocks(min(kb + NS - 1, nb - 1) - (kb + 1));
+    tie_w(wset[n1]);
+    __builtin_amdgcn_s_barrier();
+  };
+  int kb = 0;
+  for (; kb + NS <= nb; kb += NS) {  // one exit only: the accumulators keep their registers
+    block(std::integral_constant<int, 0>{}, kb);
+    block(std::integral_constant<int, 1>{}, kb + 1);
+    block(std::integral_constant<int, 2>{}, kb + 2);
+    if constexpr (NS > 3) block(std::integral_constant<int, 3>{}, kb + 3);
+  }
+  if (kb < nb) {
+    block(std::integral_constant<int, 0>{}, kb);
+    if (kb + 1 < nb) block(std::integral_constant<int, 1>{}, kb + 1);
+    if constexpr (NS > 3) {
+      if (kb + 2 < nb) block(std::integral_constant<int, 2>{}, kb + 2);
+    }
+  }
+
+  unsigned tid_e = threadIdx.x;
+  asm volatile("" : "+v"(tid_e));
+  tk_gemm32_epilogue<P, NT>(pr, hot, scales, acc, smem, (int)tid_e, bm, bn);
+}
+
+template <int P, int NT>
+__device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
+                                                   v16i (&acc)[2][NT * P / 2], uint8_t *smem, int tid, int bm, int bn) {
+  constexpr int ROWS = 64, A4 = 16 * ROWS, CST = TK_GEMM32_STAGES * A4 * 16, HP = NT / 2;
+  const int wave = tid >> 6, lane = tid & 63, r16 = lane & 15, h = (lane >> 4) & 1, kappa = lane >> 5;
+  const int R = hot.R, row0 = bm * ROWS, tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+  const int n_tiles = (hot.n + 15) >> 4;
+  const int *cst_rs = (const int *)(smem + CST);
+  const float *cst_as = (const float *)(smem + CST + 256);
+  const int *cst_exp = (const int *)(smem + CST + 512);
+  const int *cst_flag = (const int *)(smem + CST + 768);
+  unsigned my_flag = 0;
+  if (hot.flags && tid < ROWS) {
+    const bool in_range = hot.mode == TK_MODE_INT8 ? row0 + tid < R : (row0 >> 2) + tid < hot.M;
+    if (in_range) my_flag = cst_flag[tid] ? 1u : 0u;
+  }
+  // this lane's column in pair z of every plane: tile 2z + h, column r16
+  float sc[HP][P];
+#pragma unroll
+  for (int z = 0; z < HP; ++z) {
+    const int t = tile0 + 2 * z + h, n = t * 16 + r16;
+#pragma unroll
+    for (int p = 0; p < P; ++p) sc[z][p] = (t < n_tiles && n < hot.n) ? gload(scales[p] + n) : 0.0f;
+  }
+  const int wg_flag = __syncthreads_or((int)my_flag);
+  // constants of the 4 rows rl..rl+3 of the tile (rl a multiple of 4)
+  auto row_const = [&](int rl) {
+    RowConst rc;
+    const v4i rs4 = *(const v4i *)(cst_rs + rl);
+    const float4 as4 = *(const float4 *)(cst_as + rl);
+    rc.rs[0] = rs4.x; rc.rs[1] = rs4.y; rc.rs[2] = rs4.z; rc.rs[3] = rs4.w;
+    rc.as[0] = as4.x; rc.as[1] = as4.y; rc.as[2] = as4.z; rc.as[3] = as4.w;
+    rc.exp = cst_exp[rl >> 2];
+    rc.flag = 0;
+    if (wg_flag) {
+      if (hot.mode == TK_MODE_INT8) {
+        const v4i f4 = *(const v4i *)(cst_flag + rl);
+        rc.flag = (f4.x ? 1u : 0u) | (f4.y ? 2u : 0u) | (f4.z ? 4u : 0u) | (f4.w ? 8u : 0u);
+      } else {
+        rc.flag = cst_flag[rl >> 2] ? 1u : 0u;
+      }
+    }
+    return rc;
+  };
+  // the four accumulator registers 4q..4q+3 of row tile rt2, pair z, every plane
+  auto quad = [&](int rt2, int q, int z, v4i (&av)[P]) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      const v16i &c = acc[rt2][p * HP + z];
+      av[p] = v4i{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+    }
+  };
+
+  const int esz = hot.out_dtype == TK_BF16 ? 2 : 4;
+  const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0;
+  if (staged) {
+    constexpr int WG_COLS = TK_GEMM_WAVES * NT * 16;
+    const bool int8_mode = hot.mode == TK_MODE_INT8 || hot.out_dtype == TK_I32;
+    const int halves = esz == 4 ? 2 : 1;       // 4-byte outputs take the 64 rows in two halves
+    const int orows_half = int8_mode ? (64 / halves) : (16 / halves);
+    const int stride = WG_COLS * esz + 16;     // padded against bank conflicts
+    const int pieces_row = WG_COLS * esz / 16;
+    const int out_row0 = int8_mode ? row0 : (row0 >> 2);
+    const int out_rows = int8_mode ? hot.R : hot.M;
+    const int col0 = bn * WG_COLS;
+    const bool has_as = hot.act_scale != nullptr;
+    for (int hh = 0; hh < halves; ++hh) {
+      if (hh > 0) __syncthreads();
+#pragma unroll
+      for (int rt2 = 0; rt2 < 2; ++rt2) {
+        if (halves == 2 && rt2 != hh) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rl = rt2 * 32 + 8 * q + 4 * kappa;             // first of this lane's 4 rows, tile-local
+          const int sl = rl - (halves == 2 ? hh * 32 : 0);         // ... staging-local
+          const RowConst rc = row_const(rl);
+#pragma unroll
+          for (int z = 0; z < HP; ++z) {
+            const int cl = (wave * NT + 2 * z + h) * 16 + r16;
+            v4i av[P];
+            quad(rt2, q, z, av);
+            if (hot.out_dtype == TK_I32) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) *(int32_t *)(smem + (size_t)(sl + r) * stride + cl * 4) = av[0][r] - rc.rs[r];
+            } else if (hot.mode == TK_MODE_INT8) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const float f = int8_value<P>(av, r, sc[z], rc, has_as);
+                uint8_t *dst = smem + (size_t)(sl + r) * stride + cl * esz;
+                if (esz == 2) *(uint16_t *)dst = f32_to_bf16_rne(f); else *(float *)dst = f;
+              }
+            } else {
+              const float f = digits_value<P>(av, sc[z], rc);
+              uint8_t *dst = smem + (size_t)(sl >> 2) * stride + cl * esz;
+              if (esz == 2) *(uint16_t *)dst = f32_to_bf16_rne(f); else *(float *)dst = f;
+            }
+          }
+        }
+      }
+      __syncthreads();
+      const int per16 = 16 / esz;
+      for (int pc = tid; pc < orows_half * pieces_row; pc += TK_GEMM_THREADS) {
+        const int rl = pc / pieces_row, piece = pc - rl * pieces_row;
+        const int orow = out_row0 + hh * orows_half + rl;
+        const int c = col0 + piece * per16;
+        if (orow >= out_rows || c >= hot.n) continue;
+        if (wg_flag && hot.out_dtype != TK_I32 && gload(hot.flags + orow)) continue;  // written by exact_rows below
+        *(TK_GLOBAL v4u *)((uint8_t *)hot.out + ((size_t)orow * hot.n + c) * esz) = *(const v4u *)(smem + (size_t)rl * stride + piece * 16);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int rt2 = 0; rt2 < 2; ++rt2)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int rl = rt2 * 32 + 8 * q + 4 * kappa;
+        const RowConst rc = row_const(rl);
+#pragma unroll
+        for (int z = 0; z < HP; ++z) {
+          const int t = tile0 + 2 * z + h, n = t * 16 + r16;
+          if (t >= n_tiles || n >= hot.n) continue;
+          v4i av[P];
+          quad(rt2, q, z, av);
+          flow_epilogue<P>(hot, n, row0 + rl, av, sc[z], rc);
+        }
+      }
+  }
+  if (wg_flag) {
+    for (int z = 0; z < HP; ++z) {
+      const int t = tile0 + 2 * z + h, n = t * 16 + r16;
+      if (t >= pr.n_tiles || n >= pr.n) continue;
+      for (int rt2 = 0; rt2 < 2; ++rt2)
+        for (int q = 0; q < 4; ++q) {
+          const int rowbase = row0 + rt2 * 32 + 8 * q + 4 * kappa;
+          const unsigned fl = row_flags(pr, rowbase);
+          if (fl) exact_rows(pr, n, rowbase, fl);
+        }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // reference-order float kernel: one thread per (token, output)
 // ------------------------------------------------------------------------------------------
 
@@ -1634,8 +1994,28 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
 }
 
 // output tiles per workgroup of the GEMM for a plane count
-int tk_gemm_lds_bytes(void) { return 3 * 16 * 64 * 16 + 1024; }  // three A blocks + the row constants
-int tk_gemm_tiles_per_wg(int planes) { return TK_GEMM_WAVES * (planes == 1 ? 4 : (planes == 2 ? 2 : 1)); }
+int tk_gemm_lds_bytes(void) { return (TK_GEMM32_STAGES > 3 ? TK_GEMM32_STAGES : 3) * 16 * 64 * 16 + 1024; }  // the A blocks + the row constants
+int tk_gemm_tiles_per_wg(int planes) { return TK_GEMM_WAVES * (planes == 1 ? 4 : (planes <= 3 ? 2 : 1)); }
+
+template <typename K>
+static hipError_t gemm_launch_one(K kernel, hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
+                                  const TkLaunchCfg &cfg, unsigned wgs) {
+  if (cfg.lds_bytes > 64 * 1024) {
+    // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+    static thread_local const void *raised[16];
+    static thread_local int nraised = 0;
+    bool done = false;
+    for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
+    if (!done) {
+      // (not the full 160 KiB: the kernel also has a few static bytes)
+      hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+      if (e != hipSuccess) return e;
+      if (nraised < 16) raised[nraised++] = (const void *)kernel;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(wgs), dim3(TK_GEMM_THREADS), cfg.lds_bytes, s, sg, table, wg_prob);
+  return hipGetLastError();
+}
 
 // single != null: one problem, grid from its XCD split. table != null: a grouped launch of cfg.grid
 // workgroups (every member's share is a multiple of 8).
@@ -1650,14 +2030,18 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
   if (table) hipLaunchKernelGGL((tk_gemm_kernel<PP, NTT, true>), grid, block, cfg.lds_bytes, s, sg, table, wg_prob); \
   else hipLaunchKernelGGL((tk_gemm_kernel<PP, NTT, false>), grid, block, cfg.lds_bytes, s, sg, table, wg_prob);      \
   break;
+#define TK_GEMM32_CASE(PP, NTT)                                                                              \
+  if (table) return gemm_launch_one(tk_gemm32_kernel<PP, NTT, true>, s, sg, table, wg_prob, cfg, wgs);        \
+  return gemm_launch_one(tk_gemm32_kernel<PP, NTT, false>, s, sg, table, wg_prob, cfg, wgs);
   switch (cfg.planes) {
-    case 1: TK_GEMM_CASE(1, 4)
-    case 2: TK_GEMM_CASE(2, 2)
-    case 3: TK_GEMM_CASE(3, 1)
+    case 1: TK_GEMM32_CASE(1, 4)
+    case 2: TK_GEMM32_CASE(2, 2)
+    case 3: TK_GEMM32_CASE(3, 2)
     case 4: TK_GEMM_CASE(4, 1)
     default: return hipErrorInvalidValue;
   }
 #undef TK_GEMM_CASE
+#undef TK_GEMM32_CASE
   return hipGetLastError();
 }
 
