@@ -394,7 +394,7 @@ def main():
                    "copies": COPIES, "bytes_per_step": int(dec["bytes_per_launch_avg"] * len(SWEEP))},
         "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "tk_flow_kernel<2,*>", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
+                     "kernel": "tk_flow_kernel<2,*> (batch 1-4, 16), tk_flow32_kernel<2,1,*> (batch 8)", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
                      "algorithmic_bytes_per_launch": int(dec["bytes_per_launch_avg"])},
         "per_batch": dec["per_batch"],
         "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,

@@ -199,6 +199,11 @@ int tk_set_flow_run_tiles(tk_ctx *ctx, int tiles);
 /* Positions in the flow kernel's prefetch ring: 0 = chosen per launch (fewest padded positions for
  * the K block counts of the launch), or 2..5. A tuning knob: results do not depend on it. */
 int tk_set_flow_ring(tk_ctx *ctx, int positions);
+/* Matrix instruction of the flow kernel for 17..64 operand rows and one or two planes: 0 = chosen
+ * per launch (32x32x32 for 25..32 rows that take at most 64 KiB of LDS), 16 = always 16x16x64,
+ * 32 = 32x32x32 wherever its operand rows fit in LDS. A tuning and test knob: both forms give
+ * identical bits. */
+int tk_set_flow_mfma(tk_ctx *ctx, int rows);
 int tk_set_stream_min_groups(tk_ctx *ctx, int groups);
 int tk_get_stream_min_groups(const tk_ctx *ctx);
 

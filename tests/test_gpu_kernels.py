@@ -16,13 +16,16 @@ DECODE_SHAPES = [(1, 1, 1), (1, 7, 300), (5, 130, 257), (64, 3, 2560), (3, 33, 6
 GEMM_SHAPES = [(65, 8, 256), (100, 50, 700), (130, 257, 512), (128, 40, 2560), (200, 129, 300), (257, 16, 256)]
 
 
-@pytest.fixture(params=["ksplit", "stream", "flow"], autouse=True)
+@pytest.fixture(params=["ksplit", "stream", "flow", "flow32"], autouse=True)
 def decode_kernel(request, backend):
-    """Every case runs through all three decode kernels: K-split (default for narrow launches),
-    streaming and flow (forced here; the defaults for launches that fill the chip)."""
-    backend.set_decode_kernel({"ksplit": 1, "stream": 2, "flow": 3}[request.param])
+    """Every case runs through all decode kernels: K-split (default for narrow launches), streaming
+    and flow (forced here; the defaults for launches that fill the chip), the last with 17..64
+    operand rows on each of its two matrix instructions ("flow" 16x16x64, "flow32" 32x32x32)."""
+    backend.set_decode_kernel({"ksplit": 1, "stream": 2, "flow": 3, "flow32": 3}[request.param])
+    backend.set_flow_mfma(32 if request.param == "flow32" else 16)
     yield request.param
     backend.set_decode_kernel(0)
+    backend.set_flow_mfma(0)
 
 
 def _layer(backend, oracle, ws, scs, fmt=FMT_TQ2_0):
@@ -315,8 +318,9 @@ def test_gemm_epilogue_variants(backend, oracle, m, n, k, decode_kernel):
 @pytest.mark.parametrize("planes", [1, 2])
 def test_flow_runs_of_several_tiles(backend, oracle, nb, planes, decode_kernel):
     """A wave of the flow kernel walks runs of consecutive tiles as one stream behind a prefetch
-    ring; every K block count relative to the ring size, runs of 2 and 5 tiles, ragged last run."""
-    if decode_kernel != "flow":
+    ring; every K block count relative to the ring size, runs of 2 and 5 tiles, ragged last run,
+    one, two and four row tiles (the last two on either matrix instruction)."""
+    if decode_kernel not in ("flow", "flow32"):
         pytest.skip("flow kernel only")
     k = nb * 256 - 13
     n = 16 * 37 + 5
@@ -327,7 +331,7 @@ def test_flow_runs_of_several_tiles(backend, oracle, nb, planes, decode_kernel):
     try:
         for run_tiles in (2, 5):
             backend.set_flow_run_tiles(run_tiles)
-            for m in (1, 16):
+            for m in ((1, 16, 17, 64) if decode_kernel == "flow" else (17, 33, 64)):
                 print("case flow-runs", nb, planes, run_tiles, m, flush=True)
                 q = rng.integers(-128, 128, (m, k)).astype(np.int8)
                 dq, dout = backend.to_device(q, "i8"), backend.empty(m * n, "f32")

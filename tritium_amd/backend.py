@@ -393,6 +393,9 @@ class Mi355xBackend:
     def set_flow_ring(self, positions):
         _check(self._lib.tk_set_flow_ring(self._ctx, positions))
 
+    def set_flow_mfma(self, rows):
+        _check(self._lib.tk_set_flow_mfma(self._ctx, rows))
+
     def set_stream_min_groups(self, groups):
         _check(self._lib.tk_set_stream_min_groups(self._ctx, groups))
 

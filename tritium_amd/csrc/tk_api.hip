@@ -74,6 +74,7 @@ struct tk_ctx {
   int decode_force = 0;  // DECODE_AUTO
   int flow_run_tiles = 0;  // 0 = automatic
   int flow_ring = 0;       // 0 = automatic
+  int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
   int *d_invalid = nullptr;
 };
@@ -255,6 +256,15 @@ extern "C" int tk_set_flow_run_tiles(tk_ctx *ctx, int tiles) {
   return TK_OK;
 }
 
+extern "C" int tk_set_flow_mfma(tk_ctx *ctx, int rows) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_mfma: null context");
+  if (rows != 0 && rows != 16 && rows != 32)
+    return tk_fail(TK_ERR_INVALID_INPUT, "flow_mfma=%d - use 0 (automatic), 16 or 32", rows);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->flow_mfma = rows;
+  return TK_OK;
+}
+
 extern "C" int tk_set_flow_ring(tk_ctx *ctx, int positions) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_ring: null context");
   if (positions != 0 && (positions < 2 || positions > 5))
@@ -423,6 +433,35 @@ enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3, D
 
 static const size_t kLdsFlowMax = 160 * 1024;
 static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
+// widest row stride any kernel asks of the staged operand rows of an R-row problem
+static size_t kPrepRowsMax(size_t R) { return R + 16 > 64 ? R + 16 : 64; }
+
+// The 32x32x32 form of the flow kernel: 17..64 operand rows, one or two planes (more would not fit the
+// register file with a prefetch ring). Its operand rows have a fixed stride of 32 or 64 rows, in the
+// workspace and in LDS, and 1 KiB of LDS behind them holds the row constants.
+static const size_t kFlowWideExtraLds = 1024;
+static size_t flow_wide_rows(int rt) { return rt <= 2 ? 32 : 64; }
+static size_t flow_wide_lds(int rt, size_t nb) { return nb * 256 * flow_wide_rows(rt); }
+// Measured over 128-192 layer copies of N=8192 with K=1024/2048/2560 and one or two planes, float and
+// int8 contract: at 25..32 rows the wide form is 3-16% faster as long as its rows leave room for two
+// workgroups per CU (<= 64 KiB); with one workgroup per CU, or at 20-24 rows (which both forms pad
+// to 32), the 16x16x64 form is as fast or up to 4% faster. At 33..64 rows the picture is mixed (two
+// planes K=2048 int8: 9% faster; one plane: 4-18% slower), so those keep the 16x16x64 form unless
+// the wide one is asked for.
+static bool flow_wide(const tk_ctx *ctx, int planes, int rt, size_t nb, size_t rows) {
+  if (rt < 2 || planes > 2 || flow_wide_lds(rt, nb) + kFlowWideExtraLds > kLdsFlowMax) return false;
+  if (ctx->flow_mfma == 16) return false;
+  if (ctx->flow_mfma == 32) return true;
+  return rt == 2 && rows > 24 && flow_wide_lds(rt, nb) <= 64 * 1024;
+}
+static int flow_runs_per_wave(bool wide, int planes, int rt) {
+  return wide ? tk_flow32_runs_per_wave() : tk_flow_runs_per_wave(planes, rt);
+}
+static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds) {
+  cfg->wide_mfma = wide ? 1 : 0;
+  cfg->lds_bytes = flow_lds + (wide ? kFlowWideExtraLds : 0);
+  if (wide && cfg->ring > 4) cfg->ring = 4;
+}
 
 // Consecutive tiles per run of the flow kernel. A workgroup pays for staging its operand rows
 // (lds_bytes) once, so it should stream several times that in weights; beyond that, shorter runs
@@ -431,9 +470,9 @@ static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
 // (128 KiB of weights per workgroup), 32 rows at 4 (4x the staged bytes, four-wave workgroups), 64
 // rows at 8 (16x, eight-wave workgroups, one per CU).
 static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
-                          size_t nb) {
+                          size_t nb, bool wide) {
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
-  const size_t per_s = (size_t)waves * (size_t)tk_flow_runs_per_wave(planes, rt);
+  const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, planes, rt);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
   size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 ? 2 : 4);
   if (target < 128 * 1024) target = 128 * 1024;
@@ -547,6 +586,20 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   Plan pl;
   plan_shape(ctx, layer, n, k, m, mode, out_dtype, &pl);
   const size_t nb = pl.pr.nb, R = pl.pr.R;
+  int variant = DECODE_KSPLIT, run_tiles = 1;
+  unsigned flow_groups = 0;
+  bool wide = false;
+  size_t flow_lds = pl.flow_lds;
+  if (pl.skinny) {
+    wide = pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R);
+    if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
+    const int fw = flow_waves(flow_lds);
+    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide);
+    const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
+    flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
+    variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
+    if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
+  }
   TKCHK(ensure(ctx, ctx->ap, (size_t)pl.pr.rs * nb * 256));
   TKCHK(ensure(ctx, ctx->rowsum, R * 4));
   TKCHK(ensure(ctx, ctx->fscale, m * 4));
@@ -588,21 +641,13 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else {
     pr.act_scale = act_scale_in;
   }
-  int variant = DECODE_KSPLIT, run_tiles = 1;
-  unsigned flow_groups = 0;
-  if (pl.skinny) {
-    const int fw = flow_waves(pl.flow_lds);
-    run_tiles = flow_run_tiles(ctx, (unsigned)pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, pl.flow_lds, pr.nb);
-    const unsigned per_wg = (unsigned)fw * (unsigned)tk_flow_runs_per_wave(pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
-    flow_groups = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
-    variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
-  }
   if (pl.skinny && variant == DECODE_FLOW) {
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = flow_groups;
-    cfg.lds_bytes = pl.flow_lds;
-    cfg.waves = flow_waves(pl.flow_lds);
+    cfg.lds_bytes = flow_lds;
+    cfg.waves = flow_waves(flow_lds);
     cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt);
+    flow_cfg_form(&cfg, wide, flow_lds);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -856,7 +901,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       rows += (unsigned)m;
       prep_of[i] = (int)preps.size();
       preps.push_back(pp);
-      prep_off.push_back(take((R + 16) * nb * 256));  // room for the GEMM form's padded row stride
+      prep_off.push_back(take(kPrepRowsMax(R) * nb * 256));  // room for the padded row strides (prefill kernel, 32x32x32 flow)
       take(R * 4); take(m * 4); take(m * 4); take(m * 4); take(m * 4);
     }
     plans[i].pr.tile_begin = (int)tiles;
@@ -872,12 +917,16 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     if (plans[i].flow_lds > flds) flds = plans[i].flow_lds;
     flow_ok = flow_ok && plans[i].flow_ok;
   }
-  const int fw = flow_waves(flds);
-  size_t nb_max = 1;
-  for (size_t i = 0; i < count; ++i)
+  size_t nb_max = 1, rows_max = 1;
+  for (size_t i = 0; i < count; ++i) {
     if ((size_t)plans[i].pr.nb > nb_max) nb_max = plans[i].pr.nb;
-  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max);
-  const unsigned fper = (unsigned)fw * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)run_tiles;
+    if ((size_t)plans[i].pr.R > rows_max) rows_max = plans[i].pr.R;
+  }
+  const bool wide = flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
+  if (wide) flds = flow_wide_lds(rt, nb_max);
+  const int fw = flow_waves(flds);
+  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide);
+  const unsigned fper = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, planes, rt) * (unsigned)run_tiles;
   unsigned fgroups = 0;
   for (size_t i = 0; i < count; ++i) {
     sgroups += ((unsigned)plans[i].pr.n_tiles + tpw - 1) / tpw;
@@ -895,7 +944,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
   TkLaunchCfg flow_cfg{};
   if (variant == DECODE_GEMM) {
     // members whose rows fit go through the flow kernel in a launch of their own
-    size_t pflds = 0, pnb_max = 1;
+    size_t pflds = 0, pnb_max = 1, prows_max = 1;
     unsigned ptiles = 0;
     std::vector<int> nbs;
     std::vector<double> wts;
@@ -903,13 +952,16 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       if (!plans[i].flow_ok) continue;
       if (plans[i].flow_lds > pflds) pflds = plans[i].flow_lds;
       if ((size_t)plans[i].pr.nb > pnb_max) pnb_max = plans[i].pr.nb;
+      if ((size_t)plans[i].pr.R > prows_max) prows_max = plans[i].pr.R;
       ptiles += (unsigned)plans[i].pr.n_tiles;
       nbs.push_back(plans[i].pr.nb);
       wts.push_back((double)plans[i].pr.n_tiles * (double)plans[i].pr.nb);
     }
+    const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
+    if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds);
-    const int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max) : 1;
-    const unsigned pper = (unsigned)pfw * (unsigned)tk_flow_runs_per_wave(planes, rt) * (unsigned)prun;
+    const int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide) : 1;
+    const unsigned pper = (unsigned)pfw * (unsigned)flow_runs_per_wave(pwide, planes, rt) * (unsigned)prun;
     unsigned flow_total = 0;
     for (size_t i = 0; i < count; ++i) {
       if (plans[i].flow_ok) {
@@ -918,6 +970,10 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
         plans[i].pr.run_tiles = prun;
         for (unsigned j = 0; j < gi; ++j) flow_wg_prob.push_back((int)i);
         flow_total += gi;
+        if (pwide) {
+          plans[i].pr.rs = (int)flow_wide_rows(rt);
+          preps[prep_of[i]].rs = flow_wide_rows(rt);
+        }
         continue;
       }
       plan_gemm(&plans[i]);
@@ -934,6 +990,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
       flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt);
+      flow_cfg_form(&flow_cfg, pwide, pflds);
     }
   } else if (variant != DECODE_KSPLIT) {
     const unsigned per = variant == DECODE_FLOW ? fper : tpw;
@@ -942,6 +999,10 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       plans[i].pr.group_begin = (int)groups_total;
       plans[i].pr.run_tiles = run_tiles;
       if (variant == DECODE_STREAM) plans[i].pr.kc = plans[i].stream_kc;
+      if (variant == DECODE_FLOW && wide) {
+        plans[i].pr.rs = (int)flow_wide_rows(rt);
+        preps[prep_of[i]].rs = flow_wide_rows(rt);
+      }
       for (unsigned j = 0; j < gi; ++j) wg_prob.push_back((int)i);
       groups_total += gi;
     }
@@ -963,7 +1024,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     const size_t R = preps[j].R, nb = preps[j].nb, m = (size_t)preps[j].m;
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     uint8_t *base = (uint8_t *)g->ws + prep_off[j];
-    preps[j].ap = (int8_t *)base; base += al((R + 16) * nb * 256);
+    preps[j].ap = (int8_t *)base; base += al(kPrepRowsMax(R) * nb * 256);
     preps[j].rowsum = (int32_t *)base; base += al(R * 4);
     preps[j].act_scale = (float *)base; base += al(m * 4);
     preps[j].aux = (float *)base; base += al(m * 4);
@@ -1028,6 +1089,7 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     }
     g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt);
   }
+  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds);
   *out = g;
   return TK_OK;
 }

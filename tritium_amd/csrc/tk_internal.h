@@ -74,6 +74,7 @@ struct TkLaunchCfg {
   unsigned grid;
   int waves;    // flow kernel: waves per workgroup (4, or 8 when the operand rows need > 64 KiB of LDS)
   int ring;     // flow kernel: positions in the prefetch ring (2..5)
+  int wide_mfma; // flow kernel: 32x32x32 form (17..64 operand rows, row constants in LDS)
 };
 
 #ifdef __cplusplus
@@ -99,6 +100,7 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
 int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
 int tk_flow_ring(const int *nbs, const double *weights, int count, int rt);
+int tk_flow32_runs_per_wave(void);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

@@ -442,6 +442,16 @@ __device__ __forceinline__ TkHot make_hot(const TkProblem &pr) {
   return h;
 }
 
+// The problem of a launch without a table is the first kernel argument. Read through an opaque
+// pointer to the argument segment, its fields are fetched where they are used, as those of a table
+// entry are; read as a by-value argument, the compiler loads all of them up front and keeps them in
+// scalar registers for the whole kernel, which overflow into vector registers.
+__device__ __forceinline__ const TkProblem *single_problem() {
+  auto ka = __builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(ka));
+  return (const TkProblem *)ka;
+}
+
 struct RowConst {
   int rs[4];       // row sums of the 4 operand rows this lane finishes
   float as[4];     // INT8: per-token activation scale (1.0 when absent)
@@ -579,7 +589,7 @@ template <int P, int RT, int TW, int DR, bool TABLE>
 __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                       const int *__restrict__ wg_prob) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
+  const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : *single_problem();
   const int NW = (int)(blockDim.x >> 6);  // 4 or 8 waves
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int i = lane & 15, g = lane >> 4;
@@ -730,6 +740,231 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
           const unsigned fl = row_flags(pr, rowbase);
           if (fl) exact_rows(pr, n, rowbase, fl);
         }
+      }
+    }
+  }
+}
+
+// Row constants of the 4 operand rows starting at rowbase from a copy in LDS
+// (int rowsum[64] | float scale or int exponent [64] | uint flag[64]).
+__device__ __forceinline__ RowConst row_const_from_lds(const uint8_t *cst, int mode, int R, int M, int rowbase) {
+  const int *cst_rs = (const int *)cst;
+  const float *cst_as = (const float *)(cst + 256);
+  const int *cst_exp = (const int *)(cst + 256);
+  const uint32_t *cst_flag = (const uint32_t *)(cst + 512);
+  RowConst rc;
+  rc.exp = 0;
+  rc.flag = 0;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = rowbase + r;
+    rc.rs[r] = m < R ? cst_rs[m] : 0;
+    rc.as[r] = 1.0f;
+  }
+  if (mode == TK_MODE_INT8) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = rowbase + r;
+      if (m < R) {
+        rc.as[r] = cst_as[m];
+        if (cst_flag[m]) rc.flag |= 1u << r;
+      }
+    }
+  } else {
+    const int tok = rowbase >> 2;
+    if (tok < M) {
+      rc.exp = cst_exp[tok];
+      if (cst_flag[tok]) rc.flag = 1u;
+    }
+  }
+  return rc;
+}
+
+// ------------------------------------------------------------------------------------------
+// flow kernel for 17..64 operand rows on v_mfma_i32_32x32x32_i8 (4.0 POPS sustained where the
+// 16x16x64 form stops at 3.0: at these row counts the decode kernel is limited by the matrix pipe and
+// the vector work around it as much as by memory). Same stream and ring as tk_flow_kernel; what
+// differs is the lane map and the row stride of the operand rows, which is the compile-time
+// RS = 32 * RT2 (the prep kernels write that stride), so that every LDS read of a K block is one
+// base register plus an immediate. Lane L = 32*kappa + 16*h + r. A wave walks S PAIRS of adjacent
+// tiles; per position and plane it loads, from tile h of the pair, the 16-byte pieces g = kappa
+// (load 0) and g = 2+kappa (load 1, 512 bytes further) of row r: dword j of load l is the B operand
+// (32 weight rows x 32 k) of k step (l, j). The A operand of that step is piece (kb, j, 2*l + kappa)
+// of operand row 32*rt2 + (L & 31); it is read one step ahead of its use, the first step of a K
+// block during the last step of the block before (also across tiles: the operand rows of K block 0
+// are the same for every tile). Accumulator register i of lane L is row 32*rt2 + 8*(i/4) + 4*kappa
+// + i%4 of the column (h, r): four consecutive registers are four consecutive rows, as the
+// epilogues expect, and the two halves of a wave store 32 adjacent columns. Row constants live in
+// LDS behind the rows (16 row groups per lane are too many for registers): 1 KiB more LDS.
+// ------------------------------------------------------------------------------------------
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int P, int RT2, int DR, bool TABLE>
+__global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+                                                        const int *__restrict__ wg_prob) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : *single_problem();
+  constexpr int RS = 32 * RT2;           // row stride of the operand rows, in LDS and in pr.ap
+  constexpr unsigned POS = RS * 256u;    // bytes of operand rows per K block
+  static_assert((DR - 1) * POS + (14u * RS + 32u) * 16u < 65536u, "LDS offsets must fit the immediate");
+  const int NW = (int)(blockDim.x >> 6);  // 4 or 8 waves
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, h = (lane >> 4) & 1, kappa = lane >> 5;
+  const int nb = pr.nb, R = pr.R, S = pr.run_tiles, n_tiles = pr.n_tiles;
+  const TkHot hot = make_hot(pr);
+  const uint8_t *codes[P];
+  const float *scales[P];
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    codes[p] = pr.codes[p];
+    scales[p] = pr.scales[p];
+  }
+  constexpr int D = DR - 1;
+  const int nbpad = (nb + DR - 1) / DR * DR;
+  const int first = ((blockIdx.x - pr.group_begin) * NW + wave) * 2 * S;  // first tile of this wave
+  const unsigned plane_last = (unsigned)n_tiles * (unsigned)nb - 1u;      // last chunk of the plane
+  const unsigned skip = (unsigned)nb * 1024u;                             // the sibling tile of the pair
+  const unsigned lane_piece = (unsigned)(kappa * 16 + r16) * 16u;         // piece g = kappa of row r
+  unsigned roff = (unsigned)(first + h) * (unsigned)nb * 1024u + lane_piece - skip;
+  const unsigned run_last = (unsigned)(first + (S - 1) * 2 + h) * (unsigned)nb + (unsigned)nb - 1u;
+  const unsigned last_off = min(run_last, plane_last) * 1024u + lane_piece;
+
+  uint4 ring[DR][P][2];
+  auto request = [&](int slot, bool real, bool tile_start) {
+    roff += tile_start ? skip : 0u;
+    const unsigned off = min(roff, last_off);
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      ring[slot][p][0] = gload16(codes[p] + (size_t)off);
+      ring[slot][p][1] = gload16(codes[p] + (size_t)off + 512);
+    }
+    roff += real ? 1024u : 0u;
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) request(d, d < nb, d == 0);
+
+  // stage the operand rows of the problem in LDS (stride RS: the rows past R hold whatever the
+  // workspace held, and feed accumulators that are never stored), and the row constants behind them
+  uint8_t *cst = smem + (size_t)nb * POS;  // int rowsum[64] | float scale or int exponent [64] | uint flag[64]
+  {
+    const uint4 *ap4 = (const uint4 *)pr.ap;
+    uint4 *lds4w = (uint4 *)smem;
+    const int cnt = nb * 16 * RS;
+    for (int idx = threadIdx.x; idx < cnt; idx += (int)blockDim.x) lds4w[idx] = gload16(ap4 + idx);
+    if ((int)threadIdx.x < 64) {
+      const int m = (int)threadIdx.x;
+      int rsv = 0, ex = 0;
+      float asv = 1.0f;
+      unsigned fl = 0;
+      if (m < R) rsv = gload(hot.rowsum + m);
+      if (hot.mode == TK_MODE_INT8) {
+        if (m < R && hot.act_scale) asv = gload(hot.act_scale + m);
+        if (m < R && hot.flags) fl = gload(hot.flags + m);
+        ((float *)(cst + 256))[m] = asv;
+      } else {
+        if (m < hot.M) {
+          ex = gload(hot.exps + m);
+          if (hot.flags) fl = gload(hot.flags + m);
+        }
+        ((int *)(cst + 256))[m] = ex;
+      }
+      ((int *)cst)[m] = rsv;
+      ((uint32_t *)(cst + 512))[m] = fl;
+    }
+  }
+  __syncthreads();
+  // does any row of the problem take the exact fallback?
+  unsigned any_flag = 0;
+  if (hot.flags) {
+    const uint32_t *cf = (const uint32_t *)(cst + 512);
+    const int lim = hot.mode == TK_MODE_INT8 ? R : hot.M;
+    for (int m = 0; m < lim; ++m) any_flag |= cf[m];
+  }
+
+  // A operand of k step (l, j) = step 4*l + j of the K block whose rows start at byte `base`
+  const unsigned abase0 = (unsigned)(kappa * RS + (lane & 31)) * 16u;
+  auto lds_a = [&](unsigned base, int step, int rt2) -> v4i {
+    const int l = step >> 2, j = step & 3;
+    return *(const v4i *)(smem + base + (unsigned)(((j * 4 + 2 * l) * RS + rt2 * 32) * 16));
+  };
+  v4i a_cur[RT2];
+#pragma unroll
+  for (int rt2 = 0; rt2 < RT2; ++rt2) a_cur[rt2] = lds_a(abase0, 0, rt2);
+
+  for (int s = 0; s < S; ++s) {
+    const int t = first + 2 * s + h;  // this lane's tile of the pair
+    float sc[P];
+    {
+      const int n = min(t * 16 + r16, hot.n - 1);
+#pragma unroll
+      for (int p = 0; p < P; ++p) sc[p] = gload(scales[p] + n);
+    }
+    v16i acc[RT2][P];
+#pragma unroll
+    for (int rt2 = 0; rt2 < RT2; ++rt2)
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int c = 0; c < 16; ++c) acc[rt2][p][c] = 0;
+
+    int kbg = 0;
+    do {
+      const unsigned gbase = abase0 + (unsigned)kbg * POS;
+#pragma unroll
+      for (int d = 0; d < DR; ++d) {
+        const int kb = kbg + d;
+        {
+          int kb2 = kb + D;
+          if (kb2 >= nbpad) kb2 -= nbpad;
+          request((d + D) % DR, kb2 < nb, kb2 == 0);
+        }
+        if (kb < nb) {
+          const unsigned base = gbase + (unsigned)d * POS;
+          const unsigned nbase = kb + 1 < nb ? base + POS : abase0;  // K block 0 of the next tile
+#pragma unroll
+          for (int step = 0; step < 8; ++step) {
+            v4i a_nxt[RT2];
+#pragma unroll
+            for (int rt2 = 0; rt2 < RT2; ++rt2) a_nxt[rt2] = step < 7 ? lds_a(base, step + 1, rt2) : lds_a(nbase, 0, rt2);
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+              const uint4 w = ring[d][p][step >> 2];
+              const int j = step & 3;
+              const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
+              const v4i b = expand_codes(wj);
+#pragma unroll
+              for (int rt2 = 0; rt2 < RT2; ++rt2)
+                acc[rt2][p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_cur[rt2], b, acc[rt2][p], 0, 0, 0);
+            }
+#pragma unroll
+            for (int rt2 = 0; rt2 < RT2; ++rt2) a_cur[rt2] = a_nxt[rt2];
+          }
+        }
+      }
+      kbg += DR;
+    } while (kbg < nbpad);
+
+    const int n = t * 16 + r16;
+    if (t < n_tiles && n < hot.n) {
+#pragma unroll
+      for (int rt2 = 0; rt2 < RT2; ++rt2)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rl = rt2 * 32 + 8 * q + 4 * kappa;
+          const RowConst rc = row_const_from_lds(cst, hot.mode, R, hot.M, rl);
+          v4i av[P];
+#pragma unroll
+          for (int p = 0; p < P; ++p) av[p] = v4i{acc[rt2][p][4 * q], acc[rt2][p][4 * q + 1], acc[rt2][p][4 * q + 2], acc[rt2][p][4 * q + 3]};
+          flow_epilogue<P>(hot, n, rl, av, sc, rc);
+        }
+      if (any_flag) {
+        for (int rt2 = 0; rt2 < RT2; ++rt2)
+          for (int q = 0; q < 4; ++q) {
+            const int rowbase = rt2 * 32 + 8 * q + 4 * kappa;
+            const unsigned fl = row_flags(pr, rowbase);
+            if (fl) exact_rows(pr, n, rowbase, fl);
+          }
       }
     }
   }
@@ -1095,7 +1330,6 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, const TkHo
 // planes of one output meet in one lane; NT is even.
 // ------------------------------------------------------------------------------------------
 
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 template <int P, int NT>
 __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
@@ -1899,14 +2133,14 @@ static hipError_t flow_launch_one(K kernel, hipStream_t s, const TkProblem &sg, 
                                   const int *wg_prob, const TkLaunchCfg &cfg, int threads) {
   if (cfg.lds_bytes > 64 * 1024) {
     // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    static thread_local const void *raised[256];
+    static thread_local const void *raised[512];
     static thread_local int nraised = 0;
     bool done = false;
     for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
     if (!done) {
       hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
-      if (nraised < 256) raised[nraised++] = (const void *)kernel;
+      if (nraised < 512) raised[nraised++] = (const void *)kernel;
     }
   }
   hipLaunchKernelGGL(kernel, dim3(cfg.grid), dim3(threads), cfg.lds_bytes, s, sg, table, wg_prob);
@@ -1935,9 +2169,38 @@ static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkPro
   }
 }
 
+template <int P, int RT2>
+static hipError_t launch_flow32_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
+                                   const TkLaunchCfg &cfg) {
+  const int threads = cfg.waves * 64;
+  switch (cfg.ring) {
+    case 2:
+      if (table) return flow_launch_one(tk_flow32_kernel<P, RT2, 2, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow32_kernel<P, RT2, 2, false>, s, sg, table, wg_prob, cfg, threads);
+    case 3:
+      if (table) return flow_launch_one(tk_flow32_kernel<P, RT2, 3, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow32_kernel<P, RT2, 3, false>, s, sg, table, wg_prob, cfg, threads);
+    case 4:
+      if (table) return flow_launch_one(tk_flow32_kernel<P, RT2, 4, true>, s, sg, table, wg_prob, cfg, threads);
+      return flow_launch_one(tk_flow32_kernel<P, RT2, 4, false>, s, sg, table, wg_prob, cfg, threads);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <int P>
 static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                 const TkLaunchCfg &cfg) {
+  if (cfg.wide_mfma) {
+    if constexpr (P <= 2) {
+      switch (cfg.rt) {
+        case 2: return launch_flow32_pr<P, 1>(s, sg, table, wg_prob, cfg);
+        case 4: return launch_flow32_pr<P, 2>(s, sg, table, wg_prob, cfg);
+        default: return hipErrorInvalidValue;
+      }
+    } else {
+      return hipErrorInvalidValue;
+    }
+  }
   switch (cfg.rt) {
     case 1: return launch_flow_pr<P, 1>(s, sg, table, wg_prob, cfg);
     case 2: return launch_flow_pr<P, 2>(s, sg, table, wg_prob, cfg);
@@ -1948,6 +2211,8 @@ static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProb
 
 // lock-step runs per wave of the flow kernel for a (planes, rt) pair
 int tk_flow_runs_per_wave(int planes, int rt) { return (rt >= 4 && planes <= 2) ? 2 : 1; }
+// ... of the 32x32x32 form: always a pair of adjacent tiles
+int tk_flow32_runs_per_wave(void) { return 2; }
 
 // Ring size of the flow kernel (2..5 positions) for launches whose K block counts are nbs[0..count).
 // A deeper ring keeps more loads in flight per wave and costs registers, i.e. waves per SIMD.
