@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel (sweep average), from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration against a 1 GiB copy kernel):
 # profiles/decode_flow_c2_sweep_traffic.txt
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_147_111_792
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_145_160_540
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 
 K2, N2, PLANES2 = 2048, 8192, 2
