@@ -297,6 +297,7 @@ def bench_stack(T, be, rng, iters=100):
     for _ in range(layers_n):
         lins.append({name: be.linear([hostw[(n, k)][0]], [hostw[(n, k)][1]], n, k) for name, (n, k) in shapes.items()})
     code_bytes = layers_n * sum(n * ((k + 255) // 256) * 64 for n, k in shapes.values())
+    nw = [[be.to_device(rng.uniform(0.5, 1.5, h).astype(np.float32), "f32") for _ in range(2)] for _ in range(layers_n)]
     for m in (1, 32):
         hid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
         att = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
@@ -312,13 +313,25 @@ def bench_stack(T, be, rng, iters=100):
         res[f"batch{m}"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1),
                             "code_GB/s": round(code_bytes / ms / 1e6, 1)}
         g.destroy()
+        # the same step with the attention / FFN RMSNorms fused into the quantization of q,k,v and gate,up
+        norms = []
+        for li in range(layers_n):
+            norms += [(nw[li][0], 1e-5, False)] * 3 + [None] + [(nw[li][1], 1e-5, False)] * 2 + [None]
+        g = be.group(members, 1, "bf16", "bf16", norms=norms)
+        ms = time_calls(be, lambda i: g.launch(), iters)
+        res[f"batch{m}_rmsnorm_fused"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1)}
+        g.destroy()
         for x in outs + [hid, att, mid]:
             x.free()
     for L in lins:
         for l in L.values():
             l.free()
+    for pair in nw:
+        for w in pair:
+            w.free()
     res["workload"] = ("30 layers x (q,k,v,o,gate,up,down), hidden 2560, FFN 6912, 20/5 heads of 128, 1 plane, "
-                       "W1.58A8, bf16 in/out; 210 projections in one grouped launch on given inputs")
+                       "W1.58A8, bf16 in/out; 210 projections in one grouped launch on given inputs; "
+                       "*_rmsnorm_fused: q,k,v and gate,up read RMSNorm(input), computed inside the quantization launch")
     res["code_bytes_per_step"] = code_bytes
     return res
 

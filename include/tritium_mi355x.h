@@ -147,6 +147,28 @@ int tk_linear_float(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, i
 int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
                  size_t m, void *out, int out_dtype);
 
+/* RMSNorm in front of the per-token int8 quantization, as one launch: what the CUDA decode calls
+ * launch_rmsnorm_quant before the q/k/v and gate/up projections
+ * (crates/tritium-cuda/src/cuda/mod.rs:1029-1040). y[i] = (x[i] * inv) * s(w[i]),
+ * inv = 1 / sqrt(sum_squares / k + eps), s(w) = w or, zero_centered != 0, 1 + w
+ * (crates/tritium-nn/src/ops/rmsnorm.rs:43-96); the sum of squares folds in the reference's
+ * canonical order (256 slots, then a power-of-two tree, rmsnorm.rs:21-35), so the result has the
+ * bits of the host's rmsnorm followed by quantize_act_int8
+ * (crates/tritium-cuda/src/cuda/tests.rs:4675-4771). weight is a device pointer to k floats. */
+typedef struct tk_rmsnorm {
+  const float *weight;
+  float eps;
+  int zero_centered;
+} tk_rmsnorm;
+/* x [m,k] f32 or bf16 -> q [m,k] int8 row-major and act_scale [m]; rows whose normalized values
+ * hold NaN or Inf are reported as in tk_act_quant_i8. */
+int tk_rmsnorm_quant_i8(tk_ctx *ctx, const void *x, int x_dtype, const tk_rmsnorm *norm, size_t m, size_t k,
+                        int8_t *q, float *act_scale, uint32_t *nonfinite_rows);
+/* tk_linear_a8 on RMSNorm(x): norm, quantization and operand staging in one launch, then the
+ * contraction. */
+int tk_linear_rmsnorm_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *x, int x_dtype,
+                         const tk_rmsnorm *norm, size_t m, void *out, int out_dtype);
+
 /* Same contraction on activations that are already int8 (q [m,k]) with their per-token scales
  * (act_scale [m], may be null for 1.0): what the CUDA decode calls gemm_prequantized
  * (crates/tritium-cuda/src/cuda/mod.rs:1029-1064). out_dtype TK_I32 (one plane only) stores the
@@ -173,6 +195,12 @@ typedef struct tk_group_member {
 typedef enum tk_group_mode { TK_GROUP_FLOAT = 0, TK_GROUP_A8 = 1 } tk_group_mode;
 int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size_t count, int mode,
                     int act_dtype, int out_dtype, tk_group **out);
+/* A W1.58A8 group whose members read RMSNorm(act): norms[i] belongs to members[i]; an entry with a
+ * null weight leaves that member's activation as it is. Members that share activation and norm
+ * share one normalization + quantization (q/k/v after the attention norm, gate/up after the FFN
+ * norm: crates/tritium-cuda/src/cuda/mod.rs:1029-1064). */
+int tk_group_create_normed(tk_ctx *ctx, const tk_group_member *members, const tk_rmsnorm *norms, size_t count,
+                           int act_dtype, int out_dtype, tk_group **out);
 int tk_group_launch(tk_ctx *ctx, tk_group *group);
 /* The two launches of a group separately (activation prep, then the contraction), so a harness can
  * bracket the contraction kernel alone with events. tk_group_launch == parts(1, 1). */

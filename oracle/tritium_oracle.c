@@ -255,6 +255,50 @@ void to_quantize_act_int8(const float *act, size_t m, size_t k, float *q_out, fl
 }
 
 /* ------------------------------------------------------------------------- */
+/* RMSNorm — crates/tritium-nn/src/ops/rmsnorm.rs:21-96                        */
+/* ------------------------------------------------------------------------- */
+
+/* rmsnorm.rs:21-35 : 256 slots, slot t folds x[t], x[t+256], ... in ascending order (multiply, then
+ * add), then a power-of-two tree over the slots (off = 128 .. 1). */
+float to_sum_squares_canonical(const float *x, size_t n) {
+  float part[256];
+  for (int t = 0; t < 256; ++t) part[t] = 0.0f;
+  for (size_t i = 0; i < n; ++i) {
+    float sq = x[i] * x[i];
+    part[i % 256] = part[i % 256] + sq;
+  }
+  for (int off = 128; off > 0; off >>= 1)
+    for (int t = 0; t < off; ++t) part[t] = part[t] + part[t + off];
+  return part[0];
+}
+
+/* rmsnorm.rs:43-96 : out[i] = x[i] * inv * scale(w[i]) with inv = 1 / sqrt(sum/n + eps);
+ * scale(w) = w (rmsnorm) or 1 + w (rmsnorm_zero_centered). n == 0 writes nothing. */
+void to_rmsnorm(const float *x, const float *w, size_t n, float eps, int zero_centered, float *out) {
+  if (n == 0) return;
+  float mean_sq = to_sum_squares_canonical(x, n) / (float)n;
+  float inv = 1.0f / sqrtf(mean_sq + eps);
+  for (size_t i = 0; i < n; ++i) {
+    float sc = zero_centered ? 1.0f + w[i] : w[i];
+    float t = x[i] * inv;
+    out[i] = t * sc;
+  }
+}
+
+/* The fused decode step: RMSNorm of each row, then quantize_act_int8 of the result
+ * (host definition in crates/tritium-cuda/src/cuda/tests.rs:4692-4725; the launch it replaces:
+ * crates/tritium-cuda/src/cuda/mod.rs:1029-1040). */
+void to_rmsnorm_quant(const float *x, const float *w, size_t m, size_t k, float eps, int zero_centered,
+                      float *q_out, float *scale_out) {
+  float *y = (float *)malloc((k ? k : 1) * sizeof(float));
+  for (size_t r = 0; r < m; ++r) {
+    to_rmsnorm(x + r * k, w, k, eps, zero_centered, y);
+    to_quantize_act_int8(y, 1, k, q_out + r * k, scale_out + r);
+  }
+  free(y);
+}
+
+/* ------------------------------------------------------------------------- */
 /* CPU backend — crates/tritium-cpu/src/lib.rs:181-217,262-345                 */
 /* ------------------------------------------------------------------------- */
 

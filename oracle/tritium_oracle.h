@@ -75,6 +75,15 @@ int to_reference_mpgemm(const float *act, size_t act_len, const int8_t *trits, s
 /* ---- crates/tritium-spec/src/lib.rs:338-378 (== crates/tritium-nn/src/ops/act_quant.rs:94-157) ---- */
 void to_quantize_act_int8(const float *act, size_t m, size_t k, float *q_out, float *scale_out);
 
+/* ---- crates/tritium-nn/src/ops/rmsnorm.rs:21-35 : the canonical sum of squares ---- */
+float to_sum_squares_canonical(const float *x, size_t n);
+/* ---- crates/tritium-nn/src/ops/rmsnorm.rs:43-96 : rmsnorm / rmsnorm_zero_centered ---- */
+void to_rmsnorm(const float *x, const float *w, size_t n, float eps, int zero_centered, float *out);
+/* ---- crates/tritium-cuda/src/cuda/tests.rs:4692-4725 : host definition of the fused
+ *      rmsnorm -> int8 quantization (w is shared by the m rows of x [m,k]) ---- */
+void to_rmsnorm_quant(const float *x, const float *w, size_t m, size_t k, float eps, int zero_centered,
+                      float *q_out, float *scale_out);
+
 /* ---- crates/tritium-cpu/src/lib.rs:262-300 : upload_weights ----
  * Validates the packed length; for TQ2_0 reports the first row holding a reserved code in
  * *tq2_invalid_row (or -1). The bytes themselves are kept verbatim by the caller. */

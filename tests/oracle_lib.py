@@ -62,6 +62,12 @@ class Oracle:
         L.to_reference_mpgemm.argtypes = [f32p, sz, i8p, sz, f32p, sz, sz, sz, sz, f32p, sz]
         L.to_quantize_act_int8.argtypes = [f32p, sz, sz, f32p, f32p]
         L.to_quantize_act_int8.restype = None
+        L.to_sum_squares_canonical.argtypes = [f32p, sz]
+        L.to_sum_squares_canonical.restype = C.c_float
+        L.to_rmsnorm.argtypes = [f32p, f32p, sz, C.c_float, C.c_int, f32p]
+        L.to_rmsnorm.restype = None
+        L.to_rmsnorm_quant.argtypes = [f32p, f32p, sz, sz, C.c_float, C.c_int, f32p, f32p]
+        L.to_rmsnorm_quant.restype = None
         L.to_cpu_upload_check.argtypes = [u8p, sz, sz, sz, C.c_int, C.POINTER(C.c_long)]
         L.to_cpu_mpgemm.argtypes = [u8p, sz, C.c_int, f32p, sz, f32p, sz, sz, sz, sz, f32p, sz]
         L.to_cpu_mpgemm_with_act_quant.argtypes = L.to_cpu_mpgemm.argtypes
@@ -140,6 +146,27 @@ class Oracle:
         q = np.zeros(m * k, np.float32)
         s = np.zeros(m, np.float32)
         self.lib.to_quantize_act_int8(_p(a, f32p), m, k, _p(q, f32p), _p(s, f32p))
+        return q.reshape(m, k), s
+
+    def sum_squares_canonical(self, x):
+        a = np.ascontiguousarray(x, np.float32).reshape(-1)
+        return np.float32(self.lib.to_sum_squares_canonical(_p(a, f32p), a.size))
+
+    def rmsnorm(self, x, w, eps, zero_centered=False):
+        a = np.ascontiguousarray(x, np.float32).reshape(-1)
+        ww = np.ascontiguousarray(w, np.float32).reshape(-1)
+        assert a.size == ww.size
+        out = np.zeros(a.size, np.float32)
+        self.lib.to_rmsnorm(_p(a, f32p), _p(ww, f32p), a.size, eps, int(zero_centered), _p(out, f32p))
+        return out
+
+    def rmsnorm_quant(self, x, w, m, k, eps, zero_centered=False):
+        a = np.ascontiguousarray(x, np.float32).reshape(-1)
+        ww = np.ascontiguousarray(w, np.float32).reshape(-1)
+        assert a.size == m * k and ww.size == k
+        q = np.zeros(m * k, np.float32)
+        s = np.zeros(m, np.float32)
+        self.lib.to_rmsnorm_quant(_p(a, f32p), _p(ww, f32p), m, k, eps, int(zero_centered), _p(q, f32p), _p(s, f32p))
         return q.reshape(m, k), s
 
     def upload_check(self, packed, n, k, fmt):

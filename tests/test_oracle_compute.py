@@ -267,3 +267,89 @@ def test_bf16_helpers(oracle):
     want = x.to(torch.bfloat16).view(torch.int16).numpy().astype(np.uint16)
     got = np.array([oracle.f32_to_bf16(v) for v in x.tolist()], np.uint16)
     assert (got == want).all()
+
+
+# ---- RMSNorm (crates/tritium-nn/src/ops/rmsnorm.rs) ----
+
+def test_rmsnorm_unit_weights(oracle):
+    """The reference's own case (rmsnorm.rs:100-110): x = [3, 4], mean(x^2) = 12.5."""
+    out = oracle.rmsnorm([3.0, 4.0], [1.0, 1.0], 0.0)
+    inv = 1.0 / np.sqrt(np.float32(12.5))
+    assert abs(out[0] - 3.0 * inv) < 1e-6 and abs(out[1] - 4.0 * inv) < 1e-6
+
+
+def test_sum_squares_exact_on_small_integers(oracle):
+    """Integer inputs whose squares sum below 2^24: every order gives the exact sum, so this pins
+    the squaring and that every element of a ragged length is taken once."""
+    rng = np.random.default_rng(3)
+    for n in (1, 17, 255, 256, 257, 1000, 2559):
+        x = rng.integers(-9, 10, n).astype(np.float32)
+        assert oracle.sum_squares_canonical(x) == np.float32((x.astype(np.int64) ** 2).sum())
+
+
+def test_sum_squares_folds_a_slot_before_the_tree(oracle):
+    """x[1] and x[257] share slot 1: 1 + 1 = 2 survives next to 2^24 (2^24 + 2 is representable),
+    where a sequential fold loses both ones to ties-to-even (2^24 + 1 -> 2^24 twice)."""
+    x = np.zeros(258, np.float32)
+    x[0], x[1], x[257] = 4096.0, 1.0, 1.0
+    assert oracle.sum_squares_canonical(x) == np.float32(16777218.0)
+    seq = np.float32(0.0)
+    for v in x:
+        seq = np.float32(seq + v * v)
+    assert seq == np.float32(16777216.0)
+
+
+def test_sum_squares_tree_pairs_slots_128_apart(oracle):
+    """Slots 1 and 129 meet in the first tree step (off = 128) and reach slot 0 as 2; pairing
+    neighbours, or folding the slots in order, would add each 1 to 2^24 on its own and lose it."""
+    x = np.zeros(256, np.float32)
+    x[0], x[1], x[129] = 4096.0, 1.0, 1.0
+    assert oracle.sum_squares_canonical(x) == np.float32(16777218.0)
+    y = np.zeros(256, np.float32)
+    y[0], y[64], y[128] = 4096.0, 1.0, 1.0  # these meet 2^24 one at a time: both are lost
+    assert oracle.sum_squares_canonical(y) == np.float32(16777216.0)
+
+
+def test_rmsnorm_mean_eps_and_scale(oracle):
+    n = 300
+    # mean over n (not 256, not n-1): all 2.0 -> mean 4, inv 0.5 -> exactly 1.0
+    assert (oracle.rmsnorm(np.full(n, 2.0), np.ones(n), 0.0) == 1.0).all()
+    # eps sits inside the square root: mean 1, eps 3 -> 1/sqrt(4) = 0.5 (outside it would give 0.25)
+    w = np.arange(n, dtype=np.float32)
+    assert (oracle.rmsnorm(np.ones(n), w, 3.0) == np.float32(0.5) * w).all()
+    # a zero row stays zero (eps keeps inv finite)
+    assert (oracle.rmsnorm(np.zeros(n), w, 1e-5) == 0.0).all()
+    # zero-centered: 0 is the identity scale, 1 doubles (rmsnorm.rs:55-63)
+    assert (oracle.rmsnorm(np.full(n, 2.0), np.zeros(n), 0.0, zero_centered=True) == 1.0).all()
+    assert (oracle.rmsnorm(np.full(n, 2.0), np.ones(n), 0.0, zero_centered=True) == 2.0).all()
+    # n == 0 writes nothing
+    assert oracle.rmsnorm(np.zeros(0), np.zeros(0), 1e-5).size == 0
+
+
+def test_rmsnorm_multiplies_left_to_right(oracle):
+    """out = (x * inv) * w, each product rounded (rmsnorm.rs:91-93): on a row where x * (inv * w)
+    rounds differently the left-to-right value is the one returned."""
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(512).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 512).astype(np.float32)
+    eps = np.float32(1e-5)
+    inv = np.float32(1.0) / np.sqrt(np.float32(oracle.sum_squares_canonical(x) / np.float32(512) + eps))
+    left = (x * inv) * w
+    right = x * (inv * w)
+    assert (left != right).any()
+    assert (oracle.rmsnorm(x, w, eps).view(np.uint32) == left.view(np.uint32)).all()
+
+
+def test_rmsnorm_quant_composes_and_zero_row(oracle):
+    """Fused form = rmsnorm of each row, then quantize_act_int8 of it; an all-zero row gives zeros
+    and scale 0 (crates/tritium-cuda/src/cuda/tests.rs:4759-4771)."""
+    rng = np.random.default_rng(12)
+    m, k = 3, 300
+    x = rng.standard_normal((m, k)).astype(np.float32) * 3
+    x[1] = 0.0
+    w = rng.uniform(-2, 2, k).astype(np.float32)
+    q, s = oracle.rmsnorm_quant(x, w, m, k, 1e-5)
+    for r in range(m):
+        qq, ss = oracle.quantize_act_int8(oracle.rmsnorm(x[r], w, 1e-5), 1, k)
+        assert (q[r] == qq.reshape(-1)).all() and s[r] == ss[0]
+    assert (q[1] == 0).all() and s[1] == 0.0

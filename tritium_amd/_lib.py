@@ -31,6 +31,10 @@ class GroupMember(C.Structure):
     _fields_ = [("layer", LinearDesc), ("act", vp), ("m", sz), ("out", vp)]
 
 
+class RmsNorm(C.Structure):
+    _fields_ = [("weight", vp), ("eps", C.c_float), ("zero_centered", C.c_int)]
+
+
 # every symbol include/tritium_mi355x.h declares: (restype, argtypes)
 SIGNATURES = {
     "tk_init": (C.c_int, [C.c_int, C.POINTER(vp)]),
@@ -55,6 +59,10 @@ SIGNATURES = {
     "tk_act_quant_i8": (C.c_int, [vp, vp, C.c_int, sz, sz, vp, vp, vp]),
     "tk_linear_float": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
+    "tk_rmsnorm_quant_i8": (C.c_int, [vp, vp, C.c_int, C.POINTER(RmsNorm), sz, sz, vp, vp, vp]),
+    "tk_linear_rmsnorm_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, C.POINTER(RmsNorm), sz, vp, C.c_int]),
+    "tk_group_create_normed": (C.c_int, [vp, C.POINTER(GroupMember), C.POINTER(RmsNorm), sz, C.c_int, C.c_int,
+                                         C.POINTER(vp)]),
     "tk_linear_i8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, vp, sz, vp, C.c_int]),
     "tk_linear_float_seq": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_group_create": (C.c_int, [vp, C.POINTER(GroupMember), sz, C.c_int, C.c_int, C.c_int, C.POINTER(vp)]),

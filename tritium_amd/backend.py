@@ -364,8 +364,29 @@ class Mi355xBackend:
         _check(self._lib.tk_act_quant_i8(self._ctx, act.ptr, act.dtype, m, k, q.ptr, act_scale.ptr,
                                          nonfinite.ptr if nonfinite is not None else None))
 
-    def group(self, members, mode, act_dtype, out_dtype):
-        """members: list of (Linear, act DeviceArray, m, out DeviceArray)."""
+    @staticmethod
+    def _norm(weight, eps, zero_centered):
+        nm = L.RmsNorm()
+        nm.weight = weight.ptr if weight is not None else None
+        nm.eps = eps
+        nm.zero_centered = int(bool(zero_centered))
+        return nm
+
+    def rmsnorm_quant_i8(self, x, weight, eps, m, k, q, act_scale, nonfinite=None, zero_centered=False):
+        """RMSNorm of each row of x [m,k], then the per-token int8 quantization, in one launch."""
+        nm = self._norm(weight, eps, zero_centered)
+        _check(self._lib.tk_rmsnorm_quant_i8(self._ctx, x.ptr, x.dtype, C.byref(nm), m, k, q.ptr, act_scale.ptr,
+                                             nonfinite.ptr if nonfinite is not None else None))
+
+    def linear_rmsnorm_a8(self, layer, x, weight, eps, m, out, zero_centered=False):
+        """linear_a8 on RMSNorm(x): weight is a device array of k floats."""
+        nm = self._norm(weight, eps, zero_centered)
+        _check(self._lib.tk_linear_rmsnorm_a8(self._ctx, C.byref(layer.desc), x.ptr, x.dtype, C.byref(nm), m, out.ptr,
+                                              out.dtype))
+
+    def group(self, members, mode, act_dtype, out_dtype, norms=None):
+        """members: list of (Linear, act DeviceArray, m, out DeviceArray). norms (W1.58A8 groups
+        only): one entry per member, None or (weight DeviceArray, eps, zero_centered)."""
         arr = (L.GroupMember * len(members))()
         for i, (layer, act, m, out) in enumerate(members):
             arr[i].layer = layer.desc
@@ -373,9 +394,18 @@ class Mi355xBackend:
             arr[i].m = m
             arr[i].out = out.ptr
         h = C.c_void_p()
-        _check(self._lib.tk_group_create(self._ctx, arr, len(members), mode, DTYPES[act_dtype], DTYPES[out_dtype],
-                                         C.byref(h)))
-        return Group(self, h, members)
+        if norms is None:
+            _check(self._lib.tk_group_create(self._ctx, arr, len(members), mode, DTYPES[act_dtype],
+                                             DTYPES[out_dtype], C.byref(h)))
+            return Group(self, h, members)
+        if mode != 1 or len(norms) != len(members):
+            raise ValueError("norms need a W1.58A8 group and one entry per member")
+        narr = (L.RmsNorm * len(members))()
+        for i, nm in enumerate(norms):
+            narr[i] = self._norm(*nm) if nm is not None else self._norm(None, 0.0, False)
+        _check(self._lib.tk_group_create_normed(self._ctx, arr, narr, len(members), DTYPES[act_dtype],
+                                                DTYPES[out_dtype], C.byref(h)))
+        return Group(self, h, (members, norms))
 
     def set_gemm_min_m(self, v):
         _check(self._lib.tk_set_gemm_min_m(self._ctx, v))

@@ -75,7 +75,7 @@ struct tk_ctx {
   int flow_run_tiles = 0;  // 0 = automatic
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
-  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp;
+  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm;
   int *d_invalid = nullptr;
 };
 
@@ -571,8 +571,16 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
   }
 }
 
+static int check_norm(const tk_rmsnorm *norm) {
+  if (!norm || !norm->weight) return tk_fail(TK_ERR_INVALID_INPUT, "null RMSNorm weight");
+  if (!(norm->eps >= 0.0f) || !(norm->eps <= 3.402823466e38f))
+    return tk_fail(TK_ERR_INVALID_INPUT, "RMSNorm eps %g - use a finite value >= 0", (double)norm->eps);
+  return TK_OK;
+}
+
 static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int prep_kind, const void *act,
-                      int act_dtype, const float *act_scale_in, size_t m, void *out, int out_dtype) {
+                      int act_dtype, const float *act_scale_in, size_t m, void *out, int out_dtype,
+                      const tk_rmsnorm *norm = nullptr) {
   size_t n, k;
   TKCHK(validate_layer(ctx, layer, &n, &k));
   if (m == 0 || n == 0) return TK_OK;  // crates/tritium-rocm/src/rocm.rs:521-523
@@ -606,8 +614,15 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   TKCHK(ensure(ctx, ctx->aux, m * 4));
   TKCHK(ensure(ctx, ctx->exps, m * 4));
   TKCHK(ensure(ctx, ctx->flags, m * 4));
+  if (norm) TKCHK(ensure(ctx, ctx->ynorm, m * k * 4));
 
   TkPrep &pp = pl.prep;
+  if (norm) {
+    pp.norm_kind = norm->zero_centered ? 2 : 1;
+    pp.norm_eps = norm->eps;
+    pp.norm_w = norm->weight;
+    pp.ynorm = (float *)ctx->ynorm.p;
+  }
   pp.act = act;
   pp.ap = (int8_t *)ctx->ap.p;
   pp.rowsum = (int32_t *)ctx->rowsum.p;
@@ -631,8 +646,8 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     pr.act_scale = pp.act_scale;
     pr.aux = pp.aux;
     pr.flags = pp.flags;
-    pr.raw_act = act;
-    pr.raw_dtype = act_dtype;
+    pr.raw_act = norm ? (const void *)pp.ynorm : act;  // the exact fallback re-quantizes the normalized row
+    pr.raw_dtype = norm ? TK_F32 : act_dtype;
   } else if (prep_kind == TK_PREP_DIGITS) {
     pr.exps = pp.exps;
     pr.flags = pp.flags;
@@ -695,6 +710,17 @@ extern "C" int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void
   return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, act, act_dtype, nullptr, m, out, out_dtype);
 }
 
+extern "C" int tk_linear_rmsnorm_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *x, int x_dtype,
+                                    const tk_rmsnorm *norm, size_t m, void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(x_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  TKCHK(check_norm(norm));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, x, x_dtype, nullptr, m, out, out_dtype, norm);
+}
+
 extern "C" int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
                             size_t m, void *out, int out_dtype) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
@@ -727,12 +753,13 @@ extern "C" int tk_linear_float_seq(tk_ctx *ctx, const tk_linear_desc *layer, con
   return TK_OK;
 }
 
-extern "C" int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size_t m, size_t k, int8_t *q,
-                               float *act_scale, uint32_t *nonfinite_rows) {
+static int act_quant(tk_ctx *ctx, const void *act, int act_dtype, const tk_rmsnorm *norm, size_t m, size_t k,
+                     int8_t *q, float *act_scale, uint32_t *nonfinite_rows) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
   TKCHK(check_act_dtype(act_dtype));
+  if (norm) TKCHK(check_norm(norm));
   if (m == 0) return TK_OK;
-  if ((!act && k) || (!q && k) || !act_scale) return tk_fail(TK_ERR_INVALID_INPUT, "tk_act_quant_i8: null pointer");
+  if ((!act && k) || (!q && k) || !act_scale) return tk_fail(TK_ERR_INVALID_INPUT, "activation quantization: null pointer");
   if (m > (size_t)INT32_MAX || k > (size_t)INT32_MAX - 256)
     return tk_fail(TK_ERR_INVALID_INPUT, "shape m=%zu k=%zu exceeds the kernels' int index range", m, k);
   std::lock_guard<std::mutex> lk(ctx->mu);
@@ -748,8 +775,24 @@ extern "C" int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size
   pp.rs = m;
   pp.act_dtype = act_dtype;
   pp.m = (int)m;
+  if (norm) {
+    pp.norm_kind = norm->zero_centered ? 2 : 1;
+    pp.norm_eps = norm->eps;
+    pp.norm_w = norm->weight;
+  }
   HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_A8, &pp, nullptr, 0, (unsigned)m));
   return TK_OK;
+}
+
+extern "C" int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size_t m, size_t k, int8_t *q,
+                               float *act_scale, uint32_t *nonfinite_rows) {
+  return act_quant(ctx, act, act_dtype, nullptr, m, k, q, act_scale, nonfinite_rows);
+}
+
+extern "C" int tk_rmsnorm_quant_i8(tk_ctx *ctx, const void *x, int x_dtype, const tk_rmsnorm *norm, size_t m, size_t k,
+                                   int8_t *q, float *act_scale, uint32_t *nonfinite_rows) {
+  if (!norm) return tk_fail(TK_ERR_INVALID_INPUT, "null RMSNorm weight");
+  return act_quant(ctx, x, x_dtype, norm, m, k, q, act_scale, nonfinite_rows);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -845,11 +888,28 @@ struct tk_group {
   TkLaunchCfg flow_cfg{};
 };
 
+static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rmsnorm *norms, size_t count, int mode,
+                        int act_dtype, int out_dtype, tk_group **out);
+
 extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size_t count, int mode, int act_dtype,
                                int out_dtype, tk_group **out) {
+  return group_create(ctx, members, nullptr, count, mode, act_dtype, out_dtype, out);
+}
+
+extern "C" int tk_group_create_normed(tk_ctx *ctx, const tk_group_member *members, const tk_rmsnorm *norms,
+                                      size_t count, int act_dtype, int out_dtype, tk_group **out) {
+  if (!norms && count) return tk_fail(TK_ERR_INVALID_INPUT, "tk_group_create_normed: null norms");
+  return group_create(ctx, members, norms, count, TK_GROUP_A8, act_dtype, out_dtype, out);
+}
+
+static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rmsnorm *norms, size_t count, int mode,
+                        int act_dtype, int out_dtype, tk_group **out) {
   if (!ctx || !out || (!members && count)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_group_create: null pointer");
   *out = nullptr;
   if (mode != TK_GROUP_FLOAT && mode != TK_GROUP_A8) return tk_fail(TK_ERR_INVALID_INPUT, "group mode %d", mode);
+  if (norms)
+    for (size_t i = 0; i < count; ++i)
+      if (norms[i].weight) TKCHK(check_norm(&norms[i]));
   TKCHK(check_act_dtype(act_dtype));
   TKCHK(check_out_dtype(out_dtype, false));
   if (count == 0 || count > 65536) return tk_fail(TK_ERR_INVALID_INPUT, "group size %zu - use 1..65536", count);
@@ -882,11 +942,16 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     if (plans[i].cfg.rt > rt) rt = plans[i].cfg.rt;
     if (plans[i].cfg.lds_bytes > lds) lds = plans[i].cfg.lds_bytes;
     // members reading the same activation tensor share one prep (q/k/v, gate/up)
-    for (size_t j = 0; j < i; ++j)
-      if (members[j].act == members[i].act && members[j].m == m && plans[j].pr.k == plans[i].pr.k) {
+    const tk_rmsnorm *nm_i = norms && norms[i].weight ? &norms[i] : nullptr;
+    for (size_t j = 0; j < i; ++j) {
+      const tk_rmsnorm *nm_j = norms && norms[j].weight ? &norms[j] : nullptr;
+      const bool same_norm = (!nm_i && !nm_j) || (nm_i && nm_j && nm_i->weight == nm_j->weight && nm_i->eps == nm_j->eps &&
+                                                  !nm_i->zero_centered == !nm_j->zero_centered);
+      if (members[j].act == members[i].act && members[j].m == m && plans[j].pr.k == plans[i].pr.k && same_norm) {
         prep_of[i] = prep_of[j];
         break;
       }
+    }
     if (prep_of[i] < 0) {
       TkPrep pp = {};
       const size_t R = plans[i].pr.R, nb = plans[i].pr.nb;
@@ -899,10 +964,16 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
       pp.m = (int)m;
       pp.row_begin = (int)rows;
       rows += (unsigned)m;
+      if (nm_i) {
+        pp.norm_kind = nm_i->zero_centered ? 2 : 1;
+        pp.norm_eps = nm_i->eps;
+        pp.norm_w = nm_i->weight;
+      }
       prep_of[i] = (int)preps.size();
       preps.push_back(pp);
       prep_off.push_back(take(kPrepRowsMax(R) * nb * 256));  // room for the padded row strides (prefill kernel, 32x32x32 flow)
       take(R * 4); take(m * 4); take(m * 4); take(m * 4); take(m * 4);
+      if (nm_i) take(m * k * 4);
     }
     plans[i].pr.tile_begin = (int)tiles;
     tiles += plans[i].cfg.grid;
@@ -1029,7 +1100,8 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     preps[j].act_scale = (float *)base; base += al(m * 4);
     preps[j].aux = (float *)base; base += al(m * 4);
     preps[j].exps = (int32_t *)base; base += al(m * 4);
-    preps[j].flags = (uint32_t *)base;
+    preps[j].flags = (uint32_t *)base; base += al(m * 4);
+    if (preps[j].norm_kind) preps[j].ynorm = (float *)base;
   }
   std::vector<TkProblem> probs(count);
   for (size_t i = 0; i < count; ++i) {
@@ -1038,8 +1110,8 @@ extern "C" int tk_group_create(tk_ctx *ctx, const tk_group_member *members, size
     pr.ap = pp.ap;
     pr.rowsum = pp.rowsum;
     pr.flags = pp.flags;
-    pr.raw_act = members[i].act;
-    pr.raw_dtype = act_dtype;
+    pr.raw_act = pp.norm_kind ? (const void *)pp.ynorm : members[i].act;  // the exact fallback reads the normalized row
+    pr.raw_dtype = pp.norm_kind ? TK_F32 : act_dtype;
     pr.out = members[i].out;
     if (prep_kind == TK_PREP_A8) {
       pr.act_scale = pp.act_scale;

@@ -65,6 +65,13 @@ struct TkPrep {
   int act_dtype;
   int row_begin;        // first launch-wide token index of this tensor
   int m;
+  // A8 only: RMSNorm of each row in front of the quantization (norm_kind 0 = none, 1 = scale w,
+  // 2 = scale 1 + w). A normalized row that holds NaN or Inf is also written to ynorm [m,k] f32,
+  // which the exact fallback of such rows reads in place of the raw activation.
+  int norm_kind;
+  float norm_eps;
+  const float *norm_w;  // [k]
+  float *ynorm;
 };
 
 struct TkLaunchCfg {

@@ -1813,13 +1813,66 @@ __device__ __forceinline__ bool act_rows_vectorizable(const void *act, int dtype
 }
 
 // gamma = max |a| with the reference's `a > gamma` rule (NaN never wins), plus a non-finite flag.
+// RMSNorm in front of the quantization (crates/tritium-nn/src/ops/rmsnorm.rs:21-96). The sum of
+// squares folds in the reference's canonical order: slot t (= thread t of the 256) takes x[t],
+// x[t+256], ... in ascending order, multiply then add, and a power-of-two tree (off = 128 .. 1)
+// combines the slots; then inv = 1 / sqrt(sum / k + eps), every operation rounded once.
+struct RowNorm {
+  int kind;        // 0 none, 1 scale w, 2 scale 1 + w
+  float inv;
+  const float *w;
+};
+
+__device__ float row_inv_rms(const void *act, int dtype, size_t base, size_t k, float eps, float *part /* [256] */) {
+  static_assert(TK_WG == 256, "the canonical reduction has 256 slots");
+  float acc = 0.0f;
+  for (size_t i = threadIdx.x; i < k; i += 256) {
+    const float v = load_act(act, dtype, base + i);
+    acc = __fadd_rn(acc, __fmul_rn(v, v));
+  }
+  part[threadIdx.x] = acc;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if ((int)threadIdx.x < off) part[threadIdx.x] = __fadd_rn(part[threadIdx.x], part[threadIdx.x + off]);
+    __syncthreads();
+  }
+  const float mean_sq = __fdiv_rn(part[0], (float)k);
+  __syncthreads();
+  // sqrtf, not __fsqrt_rn: without OCML_BASIC_ROUNDED_OPERATIONS the latter is the approximate
+  // native square root; sqrtf and "/" are correctly rounded (hipcc's default for fp32)
+  return __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean_sq, eps)));
+}
+
+// y = (x * inv) * scale(w), left to right (rmsnorm.rs:91-93)
+__device__ __forceinline__ void apply_norm4(const RowNorm &nm, size_t e, size_t k, float (&v)[4]) {
+  if (!nm.kind) return;
+  float w[4];
+  if (e + 4 <= k && (((size_t)nm.w) & 15) == 0) {  // e is a multiple of 4
+    const v4u u = *(const TK_GLOBAL v4u *)(nm.w + e);
+    w[0] = __uint_as_float(u.x);
+    w[1] = __uint_as_float(u.y);
+    w[2] = __uint_as_float(u.z);
+    w[3] = __uint_as_float(u.w);
+  } else {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) w[b] = e + b < k ? gload(nm.w + e + b) : 0.0f;
+  }
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    if (e + b >= k) continue;
+    const float sc = nm.kind == 2 ? __fadd_rn(1.0f, w[b]) : w[b];
+    v[b] = __fmul_rn(__fmul_rn(v[b], nm.inv), sc);
+  }
+}
+
 __device__ void row_absmax(const void *act, int dtype, size_t base, size_t k, bool vec, float *sh, float &gamma,
-                           int &nonfinite, int *shi) {
+                           int &nonfinite, int *shi, const RowNorm &nm = RowNorm{0, 0.0f, nullptr}) {
   float g = 0.0f;
   int nf = 0;
   for (size_t e = (size_t)threadIdx.x * 4; e < k; e += TK_WG * 4) {
     float v[4];
     load_act4(act, dtype, base, e, k, vec, v);
+    apply_norm4(nm, e, k, v);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const float a = fabsf(v[b]);
@@ -1868,9 +1921,16 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
   const int dtype = pp.act_dtype;
   int8_t *ap = pp.ap, *qrm = pp.q_rowmajor;
   const bool vec = act_rows_vectorizable(act, dtype, k);
+  RowNorm nm = {pp.norm_kind, 0.0f, pp.norm_w};
+  float *ynorm = nullptr;
+  if (nm.kind) {
+    __shared__ float part[TK_WG];
+    nm.inv = row_inv_rms(act, dtype, base, k, pp.norm_eps, part);
+  }
   float gamma;
   int nonfinite;
-  row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi);
+  row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi, nm);
+  if (nm.kind && nonfinite) ynorm = pp.ynorm;  // only the exact fallback reads the normalized row
   const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
   const bool live = gamma != 0.0f && !nonfinite;
   int sum = 0;
@@ -1884,6 +1944,12 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
       const size_t e = e0 + (size_t)sl * 32;
       float v[4];
       load_act4(act, dtype, base, e, k, vec, v);
+      apply_norm4(nm, e, k, v);
+      if (ynorm) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          if (e + b < k) gstore(ynorm + base + e + b, v[b]);
+      }
       uint32_t packed = 0;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
