@@ -81,6 +81,16 @@ int tk_pack_rows(const int8_t *trits, size_t trits_len, size_t n, size_t k, int 
 int tk_unpack_rows(const uint8_t *packed, size_t packed_len, size_t n, size_t k, int format,
                    int8_t *trits, size_t trits_len);
 
+/* ---- I2_S ingest: convert_i2s_to_tq2_0 (crates/tritium-format/src/i2s_int8.rs:36-68) over
+ *      unpack_i2s_tensor (crates/tritium-format/src/i2s.rs:70-158). payload = n*k/4 quant bytes
+ *      (32-byte blocks of 128 elements of the flat [n,k] tensor, code = trit + 1, code 3 rejected)
+ *      + one little-endian f32 per-tensor scale (longer payloads, e.g. GGUF padding, are fine).
+ *      out receives n rows of TQ2_0 blocks with unit block scales, *scale the tensor's scale, which
+ *      the caller broadcasts as the per-channel scale. n*k must be a multiple of 128. ---- */
+size_t tk_i2s_payload_len(size_t n, size_t k); /* n*k/4 + 4; 0 when n*k is not a multiple of 128 */
+int tk_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k,
+                            uint8_t *out, size_t out_len, float *scale);
+
 /* ---- TernaryBackend::upload_weights (crates/tritium-spec/src/lib.rs:188-200;
  *      crates/tritium-cpu/src/lib.rs:262-300; crates/tritium-rocm/src/rocm.rs:446-475).
  * Copies; the returned handle owns device memory until tk_free_weights. `packed` is the byte
@@ -90,6 +100,10 @@ int tk_unpack_rows(const uint8_t *packed, size_t packed_len, size_t n, size_t k,
  * crates/tritium-cpu/src/lib.rs:19-21,202-205). ---- */
 int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k,
                       int format, tk_weights **out);
+/* tk_convert_i2s_to_tq2_0 followed by tk_upload_weights of the result (format TQ2_0): what a loader
+ * of a BitNet I2_S checkpoint calls per weight tensor. */
+int tk_upload_weights_i2s(tk_ctx *ctx, const uint8_t *payload, size_t payload_len, size_t n, size_t k,
+                          tk_weights **out, float *scale);
 void tk_free_weights(tk_weights *w);
 size_t tk_weights_len_bytes(const tk_weights *w); /* DeviceBuffer::len_bytes: the uploaded length */
 size_t tk_weights_n(const tk_weights *w);

@@ -219,6 +219,52 @@ int to_reference_mpgemm(const float *act, size_t act_len, const int8_t *w, size_
 }
 
 /* ------------------------------------------------------------------------- */
+/* I2_S — crates/tritium-format/src/i2s.rs, i2s_int8.rs:36-68                  */
+/* ------------------------------------------------------------------------- */
+
+/* i2s.rs:70-101 : byte gp supplies positions gp, 32+gp, 64+gp, 96+gp from bit pairs [7:6] .. [1:0];
+ * trit = code - 1; code 3 is an error. */
+int to_unpack_i2s_block(const uint8_t *block, size_t block_len, int8_t *trits, size_t trits_len) {
+  if (block_len != 32) return TO_ERR_SHAPE;   /* WrongBlockLen */
+  if (trits_len != 128) return TO_ERR_SHAPE;  /* WrongTritCount */
+  for (size_t gp = 0; gp < 32; ++gp)
+    for (int group = 0; group < 4; ++group) {
+      int shift = 6 - 2 * group;
+      unsigned code = (block[gp] >> shift) & 3u;
+      if (code == 3u) return TO_ERR_INVALID; /* InvalidI2sCode */
+      trits[group * 32 + gp] = (int8_t)((int)code - 1);
+    }
+  return TO_OK;
+}
+
+/* i2s.rs:116-158 : n_elements/4 quant bytes, then one little-endian f32 scale. */
+int to_unpack_i2s_tensor(const uint8_t *payload, size_t payload_len, size_t n_elements, int8_t *trits,
+                         size_t trits_len, float *scale) {
+  if (trits_len != n_elements || n_elements % 128 != 0) return TO_ERR_SHAPE;
+  size_t n_quant = n_elements / 4;
+  if (payload_len < n_quant + 4) return TO_ERR_SHAPE;
+  for (size_t b = 0; b < n_elements / 128; ++b) {
+    int rc = to_unpack_i2s_block(payload + b * 32, 32, trits + b * 128, 128);
+    if (rc) return rc;
+  }
+  uint32_t bits = (uint32_t)payload[n_quant] | ((uint32_t)payload[n_quant + 1] << 8) |
+                  ((uint32_t)payload[n_quant + 2] << 16) | ((uint32_t)payload[n_quant + 3] << 24);
+  memcpy(scale, &bits, 4);
+  return TO_OK;
+}
+
+/* i2s_int8.rs:47-68 : decode, then pack_tq2_0_row of every row with unit block scales. */
+int to_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k, uint8_t *out,
+                            size_t out_len, float *scale) {
+  size_t n_elements = n * k;
+  int8_t *trits = (int8_t *)malloc(n_elements ? n_elements : 1);
+  int rc = to_unpack_i2s_tensor(payload, payload_len, n_elements, trits, n_elements, scale);
+  if (!rc) rc = to_pack_matrix(trits, n, k, TO_FMT_TQ2_0, out, out_len);
+  free(trits);
+  return rc;
+}
+
+/* ------------------------------------------------------------------------- */
 /* act quant — crates/tritium-spec/src/lib.rs:351-378                          */
 /* ------------------------------------------------------------------------- */
 

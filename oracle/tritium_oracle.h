@@ -75,6 +75,15 @@ int to_reference_mpgemm(const float *act, size_t act_len, const int8_t *trits, s
 /* ---- crates/tritium-spec/src/lib.rs:338-378 (== crates/tritium-nn/src/ops/act_quant.rs:94-157) ---- */
 void to_quantize_act_int8(const float *act, size_t m, size_t k, float *q_out, float *scale_out);
 
+/* ---- crates/tritium-format/src/i2s.rs:70-101 : unpack_i2s_block (32 bytes -> 128 trits) ---- */
+int to_unpack_i2s_block(const uint8_t *block, size_t block_len, int8_t *trits, size_t trits_len);
+/* ---- crates/tritium-format/src/i2s.rs:116-158 : unpack_i2s_tensor (quants + trailing f32 scale) ---- */
+int to_unpack_i2s_tensor(const uint8_t *payload, size_t payload_len, size_t n_elements, int8_t *trits,
+                         size_t trits_len, float *scale);
+/* ---- crates/tritium-format/src/i2s_int8.rs:47-68 : convert_i2s_to_tq2_0 ---- */
+int to_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k, uint8_t *out,
+                            size_t out_len, float *scale);
+
 /* ---- crates/tritium-nn/src/ops/rmsnorm.rs:21-35 : the canonical sum of squares ---- */
 float to_sum_squares_canonical(const float *x, size_t n);
 /* ---- crates/tritium-nn/src/ops/rmsnorm.rs:43-96 : rmsnorm / rmsnorm_zero_centered ---- */

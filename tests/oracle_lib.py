@@ -62,6 +62,9 @@ class Oracle:
         L.to_reference_mpgemm.argtypes = [f32p, sz, i8p, sz, f32p, sz, sz, sz, sz, f32p, sz]
         L.to_quantize_act_int8.argtypes = [f32p, sz, sz, f32p, f32p]
         L.to_quantize_act_int8.restype = None
+        L.to_unpack_i2s_block.argtypes = [u8p, sz, i8p, sz]
+        L.to_unpack_i2s_tensor.argtypes = [u8p, sz, sz, i8p, sz, f32p]
+        L.to_convert_i2s_to_tq2_0.argtypes = [u8p, sz, sz, sz, u8p, sz, f32p]
         L.to_sum_squares_canonical.argtypes = [f32p, sz]
         L.to_sum_squares_canonical.restype = C.c_float
         L.to_rmsnorm.argtypes = [f32p, f32p, sz, C.c_float, C.c_int, f32p]
@@ -147,6 +150,26 @@ class Oracle:
         s = np.zeros(m, np.float32)
         self.lib.to_quantize_act_int8(_p(a, f32p), m, k, _p(q, f32p), _p(s, f32p))
         return q.reshape(m, k), s
+
+    def unpack_i2s_block(self, block, trits_len=128):
+        b = np.ascontiguousarray(block, np.uint8).reshape(-1)
+        t = np.zeros(trits_len, np.int8)
+        rc = self.lib.to_unpack_i2s_block(_p(b, u8p), b.size, _p(t, i8p), t.size)
+        return rc, t
+
+    def unpack_i2s_tensor(self, payload, n_elements, trits_len=None):
+        b = np.ascontiguousarray(payload, np.uint8).reshape(-1)
+        t = np.zeros(n_elements if trits_len is None else trits_len, np.int8)
+        s = np.zeros(1, np.float32)
+        rc = self.lib.to_unpack_i2s_tensor(_p(b, u8p), b.size, n_elements, _p(t, i8p), t.size, _p(s, f32p))
+        return rc, t, s[0]
+
+    def convert_i2s_to_tq2_0(self, payload, n, k):
+        b = np.ascontiguousarray(payload, np.uint8).reshape(-1)
+        out = np.zeros(n * self.row_bytes(k, FMT_TQ2_0), np.uint8)
+        s = np.zeros(1, np.float32)
+        rc = self.lib.to_convert_i2s_to_tq2_0(_p(b, u8p), b.size, n, k, _p(out, u8p), out.size, _p(s, f32p))
+        return rc, out, s[0]
 
     def sum_squares_canonical(self, x):
         a = np.ascontiguousarray(x, np.float32).reshape(-1)

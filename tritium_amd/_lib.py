@@ -58,6 +58,9 @@ SIGNATURES = {
     "tk_mpgemm_with_act_quant": (C.c_int, [vp, vp, sz, vp, vp, sz, sz, sz, sz, C.c_int, vp, sz]),
     "tk_act_quant_i8": (C.c_int, [vp, vp, C.c_int, sz, sz, vp, vp, vp]),
     "tk_linear_float": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
+    "tk_i2s_payload_len": (sz, [sz, sz]),
+    "tk_convert_i2s_to_tq2_0": (C.c_int, [vp, sz, sz, sz, vp, sz, C.POINTER(C.c_float)]),
+    "tk_upload_weights_i2s": (C.c_int, [vp, vp, sz, sz, sz, C.POINTER(vp), C.POINTER(C.c_float)]),
     "tk_linear_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_rmsnorm_quant_i8": (C.c_int, [vp, vp, C.c_int, C.POINTER(RmsNorm), sz, sz, vp, vp, vp]),
     "tk_linear_rmsnorm_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, C.POINTER(RmsNorm), sz, vp, C.c_int]),

@@ -285,7 +285,7 @@ class Mi355xBackend:
     def capabilities(self):
         return DeviceCaps(backend="mi355x", device_name=self.info.name.decode(),
                           features=["hip", self.info.arch.decode().split(":")[0], "tq2_0", "tq1_0", "mfma_i8",
-                                    "act_quant_i8", "additive_planes"],
+                                    "act_quant_i8", "additive_planes", "rmsnorm_quant_i8"],
                           total_memory_bytes=int(self.info.total_memory_bytes), supports_imma=True,
                           supports_fp8=False)
 
@@ -295,6 +295,15 @@ class Mi355xBackend:
         _check(self._lib.tk_upload_weights(self._ctx, b.ctypes.data, b.size, shape.n, shape.k, int(format),
                                            C.byref(h)))
         return Mi355xBuffer(self, h)
+
+    def upload_weights_i2s(self, payload, shape):
+        """I2_S tensor payload (quants + per-tensor f32 scale) -> (device buffer in TQ2_0 form, scale):
+        convert_i2s_to_tq2_0 (crates/tritium-format/src/i2s_int8.rs:36-68) followed by upload_weights."""
+        b = np.ascontiguousarray(payload, dtype=np.uint8).reshape(-1)
+        h, sc = C.c_void_p(), C.c_float(0.0)
+        _check(self._lib.tk_upload_weights_i2s(self._ctx, b.ctypes.data, b.size, shape.n, shape.k, C.byref(h),
+                                               C.byref(sc)))
+        return Mi355xBuffer(self, h), np.float32(sc.value)
 
     def _host_call(self, fn, p):
         if not isinstance(p.weights, Mi355xBuffer) or p.weights._backend is not self or not p.weights._h:
@@ -456,6 +465,16 @@ def pack_rows(trits, n, k, format=TernaryFormat.Tq2_0):
     out = np.empty(packed_len(n, k, format), np.uint8)
     _check(L.load().tk_pack_rows(t.ctypes.data, t.size, n, k, int(format), out.ctypes.data, out.size))
     return out
+
+
+def convert_i2s_to_tq2_0(payload, n, k):
+    """(TQ2_0 rows with unit block scales, per-tensor scale) of an I2_S tensor payload
+    (crates/tritium-format/src/i2s_int8.rs:36-68)."""
+    b = np.ascontiguousarray(payload, dtype=np.uint8).reshape(-1)
+    out = np.empty(packed_len(n, k, TernaryFormat.Tq2_0), np.uint8)
+    sc = C.c_float(0.0)
+    _check(L.load().tk_convert_i2s_to_tq2_0(b.ctypes.data, b.size, n, k, out.ctypes.data, out.size, C.byref(sc)))
+    return out, np.float32(sc.value)
 
 
 def unpack_rows(packed, n, k, format=TernaryFormat.Tq2_0):

@@ -359,6 +359,21 @@ extern "C" int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t pack
   return TK_OK;
 }
 
+extern "C" int tk_upload_weights_i2s(tk_ctx *ctx, const uint8_t *payload, size_t payload_len, size_t n, size_t k,
+                                     tk_weights **out, float *scale) {
+  if (!ctx || !out || !scale) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_weights_i2s: null pointer");
+  *out = nullptr;
+  const size_t len = tk_packed_len(n, k, TK_FORMAT_TQ2_0);
+  std::vector<uint8_t> packed;
+  try {
+    packed.resize(len);
+  } catch (const std::bad_alloc &) {
+    return tk_fail(TK_ERR_BACKEND, "tk_upload_weights_i2s: host allocation of %zu bytes failed", len);
+  }
+  TKCHK(tk_convert_i2s_to_tq2_0(payload, payload_len, n, k, packed.data(), len, scale));
+  return tk_upload_weights(ctx, packed.data(), len, n, k, TK_FORMAT_TQ2_0, out);
+}
+
 extern "C" void tk_free_weights(tk_weights *w) {
   if (!w) return;
   std::lock_guard<std::mutex> lk(w->ctx->mu);

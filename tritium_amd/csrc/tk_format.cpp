@@ -126,3 +126,51 @@ extern "C" int tk_unpack_rows(const uint8_t *packed, size_t packed_len, size_t n
     }
   return TK_OK;
 }
+
+// ------------------------------------------------------------------------------------------
+// I2_S (the BitNet GGUF tensor type 36) -> TQ2_0 rows, once at load:
+// convert_i2s_to_tq2_0 (crates/tritium-format/src/i2s_int8.rs:36-68) over unpack_i2s_tensor
+// (crates/tritium-format/src/i2s.rs:70-158). The payload is n*k/4 quant bytes followed by one
+// little-endian f32 per-tensor scale; the quants are 32-byte blocks of 128 elements in the flat
+// [n,k] row-major order, byte gp of a block holding the elements gp, 32+gp, 64+gp, 96+gp of the
+// block in its bit pairs [7:6], [5:4], [3:2], [1:0]; code = trit + 1, code 3 is reserved.
+// ------------------------------------------------------------------------------------------
+
+extern "C" size_t tk_i2s_payload_len(size_t n, size_t k) {
+  size_t elems;
+  if (__builtin_mul_overflow(n, k, &elems) || elems % 128 != 0) return 0;
+  return elems / 4 + 4;
+}
+
+extern "C" int tk_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k, uint8_t *out,
+                                       size_t out_len, float *scale) {
+  size_t elems;
+  if (__builtin_mul_overflow(n, k, &elems)) return tk_fail(TK_ERR_INVALID_INPUT, "I2_S element count overflows");
+  if (elems % 128 != 0)  // i2s.rs:122-127
+    return tk_fail(TK_ERR_INVALID_INPUT, "I2_S tensor of %zu elements is not a multiple of 128", elems);
+  const size_t quant_bytes = elems / 4, need = quant_bytes + 4;
+  if (payload_len < need) return tk_fail_mismatch(need, payload_len);  // i2s.rs:128-135
+  const size_t nb = (k + kBlock - 1) / kBlock, want_out = n * nb * 66;
+  if (out_len != want_out) return tk_fail_mismatch(want_out, out_len);
+  if ((!payload && payload_len) || (!out && out_len) || !scale)
+    return tk_fail(TK_ERR_INVALID_INPUT, "tk_convert_i2s_to_tq2_0: null pointer");
+  int8_t block[kBlock];
+  for (size_t row = 0; row < n; ++row)
+    for (size_t b = 0; b < nb; ++b) {
+      const size_t start = b * kBlock;
+      const size_t cnt = k - start < kBlock ? k - start : kBlock;
+      for (size_t e = 0; e < cnt; ++e) {
+        const size_t flat = row * k + start + e;          // position in the flat row-major tensor
+        const size_t within = flat & 127, gp = within & 31, group = within >> 5;
+        const unsigned code = (payload[(flat >> 7) * 32 + gp] >> (6 - 2 * group)) & 3u;
+        if (code == 3u) return tk_fail(TK_ERR_INVALID_INPUT, "I2_S code 0b11 at element %zu", flat);
+        block[e] = (int8_t)((int)code - 1);
+      }
+      std::memset(block + cnt, 0, kBlock - cnt);
+      pack_block_tq2(block, out + (row * nb + b) * 66);
+    }
+  uint32_t bits = (uint32_t)payload[quant_bytes] | ((uint32_t)payload[quant_bytes + 1] << 8) |
+                  ((uint32_t)payload[quant_bytes + 2] << 16) | ((uint32_t)payload[quant_bytes + 3] << 24);
+  std::memcpy(scale, &bits, 4);
+  return TK_OK;
+}
