@@ -5,6 +5,7 @@
 import os
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -26,9 +27,17 @@ def hipcc():
 
 
 def build_library(verbose=True):
-    """Compile every translation unit and link the shared library. Always rebuilds."""
+    """Compile every translation unit and link the shared library. Always rebuilds. The device
+    assembly of the kernel file is produced alongside and checked (check_isa) before linking."""
     objs = []
     procs = []
+    asm_file = tempfile.NamedTemporaryFile(suffix=".s", delete=False)
+    asm_file.close()
+    asm_cmd = [hipcc(), *FLAGS, "--offload-device-only", "-S", "-x", "hip", os.path.join(CSRC, "tk_kernels.hip"),
+               "-o", asm_file.name]
+    if verbose:
+        print(" ".join(asm_cmd), flush=True)
+    asm_proc = subprocess.Popen(asm_cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     for src in SOURCES:
         obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
         cmd = [hipcc(), *FLAGS, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
@@ -44,8 +53,20 @@ def build_library(verbose=True):
         if out.strip() and (verbose or p.returncode):
             print(out, flush=True)
         failed |= p.returncode != 0
-    if failed:
-        raise RuntimeError("hipcc failed")
+    asm_out, _ = asm_proc.communicate()
+    try:
+        if asm_proc.returncode:
+            print(asm_out, flush=True)
+            failed = True
+        if failed:
+            raise RuntimeError("hipcc failed")
+        from . import check_isa
+        with open(asm_file.name) as f:
+            bad = check_isa.check_text(f.read())
+        if bad:
+            raise RuntimeError("generated code reads registers of loads still in flight:\n" + check_isa.report(bad))
+    finally:
+        os.unlink(asm_file.name)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)

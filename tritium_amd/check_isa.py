@@ -1,0 +1,128 @@
+"""Build-time check of the prefill kernels' hand-issued loads.
+
+tk_gemm_kernel and tk_gemm32_kernel issue their weight loads as inline asm and wait for them with
+explicit `s_waitcnt vmcnt(N)` several hundred instructions later (the compiler's own wait insertion
+drains the whole counter when LDS-DMA and register loads are pending together). The compiler does
+not know that the destination registers of such an asm are still in flight: under register pressure
+it may split their live range and copy one (`v_mov_b32 v5, v66` ... `v_mov_b32 v66, v5`) before the
+wait, which reads a register the load has not written yet. Nothing in the source can forbid that,
+so the generated code is checked instead: between a vector-memory load and the wait that covers it,
+no other instruction may name one of its destination registers.
+
+    python -m tritium_amd.check_isa <file.s>      # exit status 1 and a report when a hazard is found
+"""
+import re
+import sys
+
+_VREG_RANGE = re.compile(r"\bv\[(\d+):(\d+)\]")
+_VREG_ONE = re.compile(r"\bv(\d+)\b")
+_VMCNT = re.compile(r"vmcnt\((\d+)\)")
+
+
+def _vregs(text):
+    regs = set()
+    for lo, hi in _VREG_RANGE.findall(text):
+        regs.update(range(int(lo), int(hi) + 1))
+    for r in _VREG_ONE.findall(_VREG_RANGE.sub(" ", text)):
+        regs.add(int(r))
+    return regs
+
+
+def check_function(name, lines):
+    """Scan of one function in layout order: returns a list of (line number, instruction, register)
+    hazards. Control flow is followed as far as forward branches go: a label entered only by jumps
+    starts from the loads that were in flight at the first jump to it, a label entered by falling
+    through keeps the state of the code above it; backward branches (loops) are not re-walked, which
+    is enough here because every iteration of the pipelined loops ends in the same wait."""
+    pending = []  # issue order: (destination registers, line) of every vector-memory operation
+    at_label = {}  # label -> loads in flight at the first forward jump to it
+    reachable = True
+    hazards = []
+    for no, raw in lines:
+        ins = raw.split(";")[0].strip()
+        if not ins or ins.startswith("."):
+            if ins.endswith(":"):  # a local label
+                label = ins[:-1]
+                if not reachable:
+                    pending = list(at_label.get(label, []))
+                reachable = True
+            continue
+        if ins.endswith(":"):
+            continue
+        if not reachable:
+            continue
+        op = ins.split()[0]
+        if op.startswith("s_cbranch") or op == "s_branch":
+            at_label.setdefault(ins.split()[-1], list(pending))
+            if op == "s_branch":
+                reachable = False
+            continue
+        if op == "s_endpgm":
+            reachable = False
+            continue
+        if op == "s_waitcnt":
+            m = _VMCNT.search(ins)
+            if m:
+                keep = int(m.group(1))
+                pending = pending[len(pending) - keep:] if keep else []
+            continue
+        in_flight = set().union(*(p[0] for p in pending)) if pending else set()
+        if op.startswith("global_load_lds"):  # LDS-DMA: counted by vmcnt, no destination register
+            used = _vregs(ins)
+            dest = set()
+        elif op.startswith(("global_load", "buffer_load", "flat_load", "scratch_load")):
+            operands = ins[len(op):].split(",")
+            dest = _vregs(operands[0])
+            used = _vregs(",".join(operands[1:]))
+        elif op.startswith(("global_store", "buffer_store", "flat_store", "scratch_store", "global_atomic")):
+            used = _vregs(ins)
+            dest = set()
+        else:
+            used = _vregs(ins)
+            dest = None
+        for r in sorted(used & in_flight):
+            hazards.append((no, ins, r))
+        if dest is not None:
+            for r in sorted(dest & in_flight):
+                hazards.append((no, ins, r))
+            pending.append((dest, no))
+    return hazards
+
+
+def check_text(text, only=("tk_gemm",)):
+    """Checks every function whose (mangled) name contains one of `only`. Returns {name: hazards}."""
+    found = {}
+    name, body = None, []
+    for no, line in enumerate(text.splitlines(), 1):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            name, body = m.group(1), []
+            continue
+        if name is None:
+            continue
+        if line.startswith(".Lfunc_end"):
+            if any(s in name for s in only):
+                hz = check_function(name, body)
+                if hz:
+                    found[name] = hz
+            name = None
+            continue
+        body.append((no, line))
+    return found
+
+
+def report(found):
+    out = []
+    for name, hz in found.items():
+        out.append(f"{name}: {len(hz)} use(s) of a register whose load is still in flight")
+        for no, ins, r in hz[:8]:
+            out.append(f"  line {no}: v{r} in `{ins}`")
+    return "\n".join(out)
+
+
+if __name__ == "__main__":
+    bad = check_text(open(sys.argv[1]).read())
+    if bad:
+        print(report(bad))
+        sys.exit(1)
+    print("no in-flight register is touched before its wait")

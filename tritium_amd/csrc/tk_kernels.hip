@@ -1427,7 +1427,10 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
 #pragma unroll
       for (int c = 0; c < 16; ++c) acc[rt2][y][c] = 0;
 
-  // operand loads as asm with explicit waits, as in the kernel above
+  // operand loads as asm with explicit waits, as in the kernel above. The compiler does not know
+  // that the destination registers of such a load are in flight until the wait: were it to split
+  // their live range (a copy out and back under register pressure) it would read stale data. The
+  // build checks the generated code for exactly that (tritium_amd/check_isa.py) and fails on it.
   auto lds_read = [&](v4i (&a)[2], unsigned addr, int off) {
 #pragma unroll
     for (int rt2 = 0; rt2 < 2; ++rt2)
