@@ -190,6 +190,29 @@ int tk_linear_rmsnorm_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *x
 int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
                  size_t m, void *out, int out_dtype);
 
+/* ---- block-scale additive planes (SALT): every plane is a TQ2_0 tensor whose per-256-block f16
+ *      scales count, W[n,k] = Σ_p s_p[n, k/256] · trit_p[n,k] (crates/tritium-format/src/salt.rs:1-19),
+ *      out[m,n] = Σ_k act[m,k] · W[n,k] on float activations. The host definition dequantizes the
+ *      row (planes in order) and folds one f32 accumulator over k
+ *      (salt.rs:720-738, crates/tritium-nn/src/layers/packed_salt.rs:585-628); the reference's GPU
+ *      kernel takes the planes plane-major and is held to 1e-4 of that
+ *      (crates/tritium-cuda/kernels/tq2_0_add.cu:640-719). ---- */
+/* tk_upload_weights of TQ2_0 rows that also keeps the block scales (device f32, 64 B per KiB of codes) */
+int tk_upload_weights_scaled(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k,
+                             tk_weights **out);
+typedef struct tk_salt_desc {
+  const tk_weights *planes[TK_MAX_PLANES]; /* each from tk_upload_weights_scaled, same [n,k] */
+  int n_planes;
+} tk_salt_desc;
+/* act [m,k] f32 or bf16, out [m,n] f32 or bf16. Up to 16 tokens whose four digit rows fit in LDS
+ * run on the matrix cores, block by block (within 1e-4 of the host definition, normally ~1e-6);
+ * other shapes, and tokens holding NaN or Inf, take the host's order exactly (slow). */
+int tk_linear_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
+                   void *out, int out_dtype);
+/* The host's order for every output: bit-identical to dequantize-then-fold. */
+int tk_linear_salt_seq(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
+                       void *out, int out_dtype);
+
 /* Reference-order float contraction: one thread per output, a single f32 accumulator walked in k
  * order (crates/tritium-core/src/reference.rs:25-54) — bit-identical to the CPU backend for any
  * float input, NaN/Inf included. Slow; kept as the exact fallback and as a cross-check. */

@@ -301,6 +301,80 @@ void to_quantize_act_int8(const float *act, size_t m, size_t k, float *q_out, fl
 }
 
 /* ------------------------------------------------------------------------- */
+/* SALT block-scale planes — crates/tritium-format/src/salt.rs:720-738,        */
+/* crates/tritium-nn/src/layers/packed_salt.rs:585-628                         */
+/* ------------------------------------------------------------------------- */
+
+/* IEEE binary16 -> binary32, exact (half::f16::to_f32). */
+float to_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu, bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else { /* subnormal: normalise */
+      int e = -1;
+      do { man <<= 1; ++e; } while (!(man & 0x400u));
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7F800000u | (man << 13);
+  } else {
+    bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+/* salt.rs:720-738 dequant_salt_row: W[i] = sum over planes, in plane order from 0.0, of
+ * f32(block scale) * f32(trit); each plane is one TQ2_0 row of num_blocks(k) blocks. */
+int to_salt_dequant_row(const uint8_t *const *planes, size_t t_planes, size_t k, float *out) {
+  size_t nb = to_num_blocks(k);
+  int8_t *trits = (int8_t *)malloc(k ? k : 1);
+  uint16_t *scales = (uint16_t *)malloc((nb ? nb : 1) * sizeof(uint16_t));
+  int rc = TO_OK;
+  for (size_t i = 0; i < k; ++i) out[i] = 0.0f;
+  for (size_t p = 0; p < t_planes && !rc; ++p) {
+    rc = to_unpack_row(planes[p], nb * TO_TQ2_0_BLOCK_BYTES, TO_FMT_TQ2_0, trits, k, scales, nb);
+    if (rc) break;
+    for (size_t i = 0; i < k; ++i) {
+      float term = to_f16_to_f32(scales[i / TO_QK_K]) * (float)trits[i];
+      out[i] = out[i] + term;
+    }
+  }
+  free(trits);
+  free(scales);
+  return rc;
+}
+
+/* packed_salt.rs:585-628 : out[m,n] = one f32 accumulator over k in order of act[m,k] * W[n,k],
+ * W the dequantized row. planes[p] is plane p of all n rows, row-major (the plane-major layout of
+ * crates/tritium-cuda/kernels/tq2_0_add.cu:659-672). */
+int to_salt_mpgemm(const uint8_t *const *planes, size_t t_planes, size_t n, size_t k, const float *act,
+                   size_t m, float *out) {
+  size_t rb = to_num_blocks(k) * TO_TQ2_0_BLOCK_BYTES;
+  float *w = (float *)malloc((k ? k : 1) * sizeof(float));
+  const uint8_t **row = (const uint8_t **)malloc((t_planes ? t_planes : 1) * sizeof(*row));
+  int rc = TO_OK;
+  for (size_t ni = 0; ni < n && !rc; ++ni) {
+    for (size_t p = 0; p < t_planes; ++p) row[p] = planes[p] + ni * rb;
+    rc = to_salt_dequant_row(row, t_planes, k, w);
+    if (rc) break;
+    for (size_t mi = 0; mi < m; ++mi) {
+      float acc = 0.0f;
+      for (size_t ki = 0; ki < k; ++ki) {
+        float prod = act[mi * k + ki] * w[ki];
+        acc = acc + prod;
+      }
+      out[mi * n + ni] = acc;
+    }
+  }
+  free(w);
+  free(row);
+  return rc;
+}
+
+/* ------------------------------------------------------------------------- */
 /* RMSNorm — crates/tritium-nn/src/ops/rmsnorm.rs:21-96                        */
 /* ------------------------------------------------------------------------- */
 

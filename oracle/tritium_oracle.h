@@ -84,6 +84,15 @@ int to_unpack_i2s_tensor(const uint8_t *payload, size_t payload_len, size_t n_el
 int to_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k, uint8_t *out,
                             size_t out_len, float *scale);
 
+/* ---- half::f16::to_f32 (exact) ---- */
+float to_f16_to_f32(uint16_t h);
+/* ---- crates/tritium-format/src/salt.rs:720-738 : dequant_salt_row over T planes of one row ---- */
+int to_salt_dequant_row(const uint8_t *const *planes, size_t t_planes, size_t k, float *out);
+/* ---- crates/tritium-nn/src/layers/packed_salt.rs:585-628 : forward over dequantized rows;
+ *      planes[p] = plane p of all n rows (crates/tritium-cuda/kernels/tq2_0_add.cu:659-672) ---- */
+int to_salt_mpgemm(const uint8_t *const *planes, size_t t_planes, size_t n, size_t k, const float *act,
+                   size_t m, float *out);
+
 /* ---- crates/tritium-nn/src/ops/rmsnorm.rs:21-35 : the canonical sum of squares ---- */
 float to_sum_squares_canonical(const float *x, size_t n);
 /* ---- crates/tritium-nn/src/ops/rmsnorm.rs:43-96 : rmsnorm / rmsnorm_zero_centered ---- */

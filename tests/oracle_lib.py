@@ -65,6 +65,10 @@ class Oracle:
         L.to_unpack_i2s_block.argtypes = [u8p, sz, i8p, sz]
         L.to_unpack_i2s_tensor.argtypes = [u8p, sz, sz, i8p, sz, f32p]
         L.to_convert_i2s_to_tq2_0.argtypes = [u8p, sz, sz, sz, u8p, sz, f32p]
+        L.to_f16_to_f32.argtypes = [C.c_uint16]
+        L.to_f16_to_f32.restype = C.c_float
+        L.to_salt_dequant_row.argtypes = [C.POINTER(C.c_void_p), sz, sz, f32p]
+        L.to_salt_mpgemm.argtypes = [C.POINTER(C.c_void_p), sz, sz, sz, f32p, sz, f32p]
         L.to_sum_squares_canonical.argtypes = [f32p, sz]
         L.to_sum_squares_canonical.restype = C.c_float
         L.to_rmsnorm.argtypes = [f32p, f32p, sz, C.c_float, C.c_int, f32p]
@@ -170,6 +174,35 @@ class Oracle:
         s = np.zeros(1, np.float32)
         rc = self.lib.to_convert_i2s_to_tq2_0(_p(b, u8p), b.size, n, k, _p(out, u8p), out.size, _p(s, f32p))
         return rc, out, s[0]
+
+    def f16_to_f32(self, h):
+        return np.float32(self.lib.to_f16_to_f32(int(h)))
+
+    def salt_dequant_row(self, plane_rows, k):
+        """plane_rows: list of T packed TQ2_0 rows (one per plane) of one output channel."""
+        bs = [np.ascontiguousarray(b, np.uint8) for b in plane_rows]
+        pa = (C.c_void_p * len(bs))(*[b.ctypes.data for b in bs])
+        out = np.zeros(k, np.float32)
+        rc = self.lib.to_salt_dequant_row(pa, len(bs), k, _p(out, f32p))
+        return rc, out
+
+    def salt_mpgemm(self, planes, n, k, act, m):
+        """planes: list of T arrays, each the n packed TQ2_0 rows (with block scales) of one plane."""
+        bs = [np.ascontiguousarray(b, np.uint8) for b in planes]
+        pa = (C.c_void_p * len(bs))(*[b.ctypes.data for b in bs])
+        a = np.ascontiguousarray(act, np.float32).reshape(-1)
+        assert a.size == m * k
+        out = np.zeros(m * n, np.float32)
+        rc = self.lib.to_salt_mpgemm(pa, len(bs), n, k, _p(a, f32p), m, _p(out, f32p))
+        return rc, out.reshape(m, n)
+
+    def pack_matrix_scaled(self, trits, block_scales_f16, n, k, fmt=FMT_TQ2_0):
+        """Rows packed with the given f16 block scales (uint16 bit patterns [n, nb])."""
+        t = np.ascontiguousarray(trits, np.int8).reshape(n, k)
+        sc = np.ascontiguousarray(block_scales_f16, np.uint16).reshape(n, -1)
+        rows = [self.pack_row(t[r], fmt, sc[r]) for r in range(n)]
+        assert all(rc == 0 for rc, _ in rows)
+        return np.concatenate([b for _, b in rows])
 
     def sum_squares_canonical(self, x):
         a = np.ascontiguousarray(x, np.float32).reshape(-1)

@@ -1,0 +1,114 @@
+"""Block-scale additive planes (SALT) through the device-resident C ABI.
+
+The host definition (dequantize the row, planes in order; then one f32 accumulator over k:
+crates/tritium-format/src/salt.rs:720-738, crates/tritium-nn/src/layers/packed_salt.rs:585-628) is the
+oracle. The reference-order kernel must reproduce it bit for bit; the matrix-core form is held to the
+bound the reference sets for its own GPU kernel, 1e-4 (crates/tritium-cuda/kernels/tq2_0_add.cu:651-655)."""
+import numpy as np
+import pytest
+
+import tritium_amd as T
+from helpers import accepts, bf16_bits_to_f32, f32_to_bf16_bits, rel_err, same_bits, ternary
+from test_oracle_salt import f16_bits
+
+pytestmark = pytest.mark.gpu
+
+SALT_REL = 1e-4  # tq2_0_add.cu:651-655
+
+
+def make_planes(backend, oracle, rng, n, k, t_planes):
+    nb = (k + 255) // 256
+    packed, bufs = [], []
+    for p in range(t_planes):
+        trits = ternary(rng, n, k, (0.4, 0.7, 0.85, 0.85)[p])
+        sc = f16_bits(rng.uniform(0.02, 1.0, (n, nb)) * (0.5 ** p))
+        packed.append(oracle.pack_matrix_scaled(trits, sc, n, k))
+        bufs.append(backend.upload_weights_scaled(packed[-1], T.GemmShape(0, n, k)))
+    return packed, bufs
+
+
+@pytest.mark.parametrize("m,n,k,t_planes", [(1, 48, 256, 1), (3, 33, 700, 2), (5, 130, 1000, 3), (17, 20, 300, 4)])
+def test_reference_order_kernel_is_bit_exact(backend, oracle, m, n, k, t_planes):
+    print("case salt-seq", m, n, k, t_planes, flush=True)
+    rng = np.random.default_rng(m * 13 + n + k)
+    packed, bufs = make_planes(backend, oracle, rng, n, k, t_planes)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    rc, want = oracle.salt_mpgemm(packed, n, k, act, m)
+    dact, dout = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    backend.linear_salt(bufs, dact, m, dout, seq=True)
+    assert rc == 0 and same_bits(dout.to_host(), want)
+    for a in [dact, dout] + bufs:
+        a.free()
+
+
+@pytest.mark.parametrize("t_planes", [1, 2, 3, 4])
+@pytest.mark.parametrize("m,n,k", [(1, 48, 256), (2, 130, 700), (4, 64, 2048), (5, 33, 1000), (8, 257, 2560), (16, 96, 2048)])
+def test_matrix_core_form_within_the_reference_bound(backend, oracle, m, n, k, t_planes):
+    print("case salt-flow", m, n, k, t_planes, flush=True)
+    rng = np.random.default_rng(m * 17 + n + k + t_planes)
+    packed, bufs = make_planes(backend, oracle, rng, n, k, t_planes)
+    bits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32) * 2)
+    act = bf16_bits_to_f32(bits).reshape(m, k)
+    rc, want = oracle.salt_mpgemm(packed, n, k, act, m)
+    for dtype, dev in (("bf16", bits), ("f32", act)):
+        dact, dout = backend.to_device(dev, dtype), backend.empty(m * n, "f32")
+        backend.linear_salt(bufs, dact, m, dout)
+        got = dout.to_host().reshape(m, n)
+        assert rc == 0 and accepts(got, want, rel=SALT_REL, floor=1.0).all()
+        assert rel_err(got, want) < 2e-5  # what it actually achieves: the f32 fold's own rounding
+        dact.free()
+        dout.free()
+    for b in bufs:
+        b.free()
+
+
+def test_tokens_with_nan_or_inf_take_the_host_order(backend, oracle):
+    rng = np.random.default_rng(40)
+    m, n, k = 4, 40, 600
+    packed, bufs = make_planes(backend, oracle, rng, n, k, 2)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[1, 7] = np.nan
+    act[2, 300] = np.inf
+    rc, want = oracle.salt_mpgemm(packed, n, k, act, m)
+    dact, dout = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    backend.linear_salt(bufs, dact, m, dout)
+    got = dout.to_host().reshape(m, n)
+    assert same_bits(got[1], want[1]) and same_bits(got[2], want[2])
+    assert accepts(got[[0, 3]], want[[0, 3]], rel=SALT_REL, floor=1.0).all()
+    for a in [dact, dout] + bufs:
+        a.free()
+
+
+def test_rows_beyond_the_matrix_core_form_fall_back(backend, oracle):
+    """17 tokens are 68 digit rows: the launch takes the reference-order kernel and is bit-exact."""
+    rng = np.random.default_rng(41)
+    m, n, k = 17, 24, 512
+    packed, bufs = make_planes(backend, oracle, rng, n, k, 2)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    rc, want = oracle.salt_mpgemm(packed, n, k, act, m)
+    dact, dout = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    backend.linear_salt(bufs, dact, m, dout)
+    assert same_bits(dout.to_host(), want)
+    for a in [dact, dout] + bufs:
+        a.free()
+
+
+def test_scaled_upload_still_serves_the_plain_contract(backend, oracle):
+    """mpgemm ignores block scales (crates/tritium-cpu/src/lib.rs:302-345), also on a buffer that kept them;
+    and a buffer without them is refused by the block-scale entry point."""
+    rng = np.random.default_rng(42)
+    m, n, k = 2, 20, 512
+    packed, bufs = make_planes(backend, oracle, rng, n, k, 1)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    sc = rng.uniform(0.01, 0.1, n).astype(np.float32)
+    out = np.zeros((m, n), np.float32)
+    backend.mpgemm(T.MpGemm(act, bufs[0], sc, T.GemmShape(m, n, k), T.TernaryFormat.Tq2_0, out))
+    from oracle_lib import FMT_TQ2_0
+    rc, want = oracle.cpu_mpgemm(packed[0], FMT_TQ2_0, act, sc, m, n, k)
+    assert rc == 0 and same_bits(out, want)
+    plain = backend.upload_weights(packed[0], T.GemmShape(0, n, k), T.TernaryFormat.Tq2_0)
+    dact, dout = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    with pytest.raises(T.InvalidInput):
+        backend.linear_salt([plain], dact, m, dout)
+    for a in [dact, dout, plain] + bufs:
+        a.free()

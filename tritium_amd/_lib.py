@@ -31,6 +31,10 @@ class GroupMember(C.Structure):
     _fields_ = [("layer", LinearDesc), ("act", vp), ("m", sz), ("out", vp)]
 
 
+class SaltDesc(C.Structure):
+    _fields_ = [("planes", vp * TK_MAX_PLANES), ("n_planes", C.c_int)]
+
+
 class RmsNorm(C.Structure):
     _fields_ = [("weight", vp), ("eps", C.c_float), ("zero_centered", C.c_int)]
 
@@ -61,6 +65,9 @@ SIGNATURES = {
     "tk_i2s_payload_len": (sz, [sz, sz]),
     "tk_convert_i2s_to_tq2_0": (C.c_int, [vp, sz, sz, sz, vp, sz, C.POINTER(C.c_float)]),
     "tk_upload_weights_i2s": (C.c_int, [vp, vp, sz, sz, sz, C.POINTER(vp), C.POINTER(C.c_float)]),
+    "tk_upload_weights_scaled": (C.c_int, [vp, vp, sz, sz, sz, C.POINTER(vp)]),
+    "tk_linear_salt": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
+    "tk_linear_salt_seq": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_rmsnorm_quant_i8": (C.c_int, [vp, vp, C.c_int, C.POINTER(RmsNorm), sz, sz, vp, vp, vp]),
     "tk_linear_rmsnorm_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, C.POINTER(RmsNorm), sz, vp, C.c_int]),

@@ -305,6 +305,23 @@ class Mi355xBackend:
                                                C.byref(sc)))
         return Mi355xBuffer(self, h), np.float32(sc.value)
 
+    def upload_weights_scaled(self, packed, shape):
+        """TQ2_0 rows whose f16 block scales are kept on the device (block-scale planes)."""
+        b = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+        h = C.c_void_p()
+        _check(self._lib.tk_upload_weights_scaled(self._ctx, b.ctypes.data, b.size, shape.n, shape.k, C.byref(h)))
+        return Mi355xBuffer(self, h)
+
+    def linear_salt(self, planes, act, m, out, seq=False):
+        """Block-scale additive planes on float activations: planes = buffers from
+        upload_weights_scaled; seq=True takes the host's summation order for every output."""
+        d = L.SaltDesc()
+        for i, w in enumerate(planes):
+            d.planes[i] = w._h
+        d.n_planes = len(planes)
+        fn = self._lib.tk_linear_salt_seq if seq else self._lib.tk_linear_salt
+        _check(fn(self._ctx, C.byref(d), act.ptr, act.dtype, m, out.ptr, out.dtype))
+
     def _host_call(self, fn, p):
         if not isinstance(p.weights, Mi355xBuffer) or p.weights._backend is not self or not p.weights._h:
             raise InvalidInput("buffer is not a Mi355xBuffer of this backend")

@@ -75,13 +75,14 @@ struct tk_ctx {
   int flow_run_tiles = 0;  // 0 = automatic
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
-  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm;
+  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum;
   int *d_invalid = nullptr;
 };
 
 struct tk_weights {
   tk_ctx *ctx;
   uint8_t *codes;
+  float *block_scales;  // [(tile, K block), 16 rows] f32, only for uploads that keep the block scales
   size_t n, k, nb, n_tiles, len_bytes;
   int format;
   long invalid_row;
@@ -294,8 +295,21 @@ extern "C" size_t tk_get_exact_max_macs(const tk_ctx *ctx) { return ctx ? ctx->e
 // weights
 // ------------------------------------------------------------------------------------------
 
+static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k, int format,
+                          bool keep_block_scales, tk_weights **out);
+
 extern "C" int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k,
                                  int format, tk_weights **out) {
+  return upload_weights(ctx, packed, packed_len, n, k, format, false, out);
+}
+
+extern "C" int tk_upload_weights_scaled(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k,
+                                        tk_weights **out) {
+  return upload_weights(ctx, packed, packed_len, n, k, TK_FORMAT_TQ2_0, true, out);
+}
+
+static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, size_t n, size_t k, int format,
+                          bool keep_block_scales, tk_weights **out) {
   if (!ctx || !out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_weights: null pointer");
   *out = nullptr;
   const size_t bb = fmt_block_bytes(format);
@@ -317,11 +331,13 @@ extern "C" int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t pack
   HIPCHK(hipSetDevice(ctx->device));
   const size_t n_tiles = (n + 15) / 16;
   const size_t code_bytes = n_tiles * nb * TK_CHUNK_BYTES;
-  void *codes = nullptr, *raw = nullptr;
+  void *codes = nullptr, *raw = nullptr, *bscales = nullptr;
   TKCHK(dev_malloc(code_bytes, &codes));
   int rc = dev_malloc(packed_len, &raw);
+  if (!rc && keep_block_scales) rc = dev_malloc(n_tiles * nb * 16 * sizeof(float), &bscales);
   if (rc) {
     (void)hipFree(codes);
+    if (raw) (void)hipFree(raw);
     return rc;
   }
   int invalid = INT32_MAX;
@@ -330,7 +346,8 @@ extern "C" int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t pack
   if (e == hipSuccess) e = hipMemcpyAsync(ctx->d_invalid, &invalid, sizeof invalid, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) {
     if (format == TK_FORMAT_TQ2_0)
-      e = tk_launch_relayout_tq2(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb, ctx->d_invalid);
+      e = tk_launch_relayout_tq2(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb, ctx->d_invalid,
+                                 (float *)bscales);
     else
       e = tk_launch_relayout_tq1(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb);
   }
@@ -339,15 +356,18 @@ extern "C" int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t pack
   (void)hipFree(raw);
   if (e != hipSuccess) {
     (void)hipFree(codes);
+    if (bscales) (void)hipFree(bscales);
     return tk_fail(TK_ERR_BACKEND, "upload_weights: %s", hipGetErrorString(e));
   }
   tk_weights *w = new (std::nothrow) tk_weights();
   if (!w) {
     (void)hipFree(codes);
+    if (bscales) (void)hipFree(bscales);
     return tk_fail(TK_ERR_BACKEND, "tk_upload_weights: host allocation failed");
   }
   w->ctx = ctx;
   w->codes = (uint8_t *)codes;
+  w->block_scales = (float *)bscales;
   w->n = n;
   w->k = k;
   w->nb = nb;
@@ -380,6 +400,7 @@ extern "C" void tk_free_weights(tk_weights *w) {
   (void)hipSetDevice(w->ctx->device);
   (void)hipStreamSynchronize(w->ctx->stream);
   (void)hipFree(w->codes);
+  if (w->block_scales) (void)hipFree(w->block_scales);
   delete w;
 }
 extern "C" size_t tk_weights_len_bytes(const tk_weights *w) { return w ? w->len_bytes : 0; }
@@ -734,6 +755,118 @@ extern "C" int tk_linear_rmsnorm_a8(tk_ctx *ctx, const tk_linear_desc *layer, co
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
   return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, x, x_dtype, nullptr, m, out, out_dtype, norm);
+}
+
+// Block-scale additive planes on float activations. seq != 0 forces the reference-order kernel.
+static int run_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m, void *out,
+                    int out_dtype, bool seq) {
+  if (!layer) return tk_fail(TK_ERR_INVALID_INPUT, "null layer descriptor");
+  if (layer->n_planes < 1 || layer->n_planes > TK_MAX_PLANES)
+    return tk_fail(TK_ERR_INVALID_INPUT, "n_planes=%d - use 1..%d", layer->n_planes, TK_MAX_PLANES);
+  for (int p = 0; p < layer->n_planes; ++p) {
+    const tk_weights *w = layer->planes[p];
+    if (!w) return tk_fail(TK_ERR_INVALID_INPUT, "plane %d: null weights handle", p);
+    if (w->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "plane %d: buffer belongs to another context", p);
+    if (!w->block_scales)
+      return tk_fail(TK_ERR_INVALID_INPUT, "plane %d was uploaded without its block scales (tk_upload_weights_scaled)", p);
+    if (p && (w->n != layer->planes[0]->n || w->k != layer->planes[0]->k))
+      return tk_fail(TK_ERR_INVALID_INPUT, "plane %d is [%zu,%zu] but plane 0 is [%zu,%zu]", p, w->n, w->k,
+                     layer->planes[0]->n, layer->planes[0]->k);
+    if (w->invalid_row >= 0)
+      return tk_fail(TK_ERR_BACKEND, "unpack row %ld: decoded value 2 outside ternary range", w->invalid_row);
+  }
+  const size_t n = layer->planes[0]->n, k = layer->planes[0]->k, nb = num_blocks(k);
+  if (m == 0 || n == 0) return TK_OK;
+  if (!act || !out) return tk_fail(TK_ERR_INVALID_INPUT, "null activation or output pointer");
+  size_t total;
+  if (__builtin_mul_overflow(m, n, &total) || total > (size_t)INT32_MAX || m * 4 > (size_t)INT32_MAX)
+    return tk_fail(TK_ERR_INVALID_INPUT, "shape m=%zu n=%zu k=%zu exceeds the kernels' int index range", m, n, k);
+
+  TkProblem pr;
+  memset(&pr, 0, sizeof pr);
+  for (int p = 0; p < layer->n_planes; ++p) {
+    pr.codes[p] = layer->planes[p]->codes;
+    pr.bscale[p] = layer->planes[p]->block_scales;
+  }
+  const size_t R = 4 * m;
+  pr.n = (int)n;
+  pr.k = (int)k;
+  pr.nb = (int)nb;
+  pr.R = (int)R;
+  pr.rs = (int)R;
+  pr.M = (int)m;
+  pr.mode = TK_MODE_DIGITS;
+  pr.out_dtype = out_dtype;
+  pr.planes = layer->n_planes;
+  pr.n_tiles = (int)((n + 15) / 16);
+  pr.raw_act = act;
+  pr.raw_dtype = act_dtype;
+  pr.out = out;
+  const size_t lds = nb * 256 * R + nb * R * 4;  // operand rows + their per-block sums
+  if (seq || R > 64 || lds > kLdsFlowMax) {
+    HIPCHK(tk_launch_salt_seq(ctx->stream, &pr));
+    return TK_OK;
+  }
+  TKCHK(ensure(ctx, ctx->ap, R * nb * 256));
+  TKCHK(ensure(ctx, ctx->rowsum, R * 4));
+  TKCHK(ensure(ctx, ctx->exps, m * 4));
+  TKCHK(ensure(ctx, ctx->flags, m * 4));
+  TKCHK(ensure(ctx, ctx->blocksum, nb * R * 4));
+  TkPrep pp = {};
+  pp.act = act;
+  pp.ap = (int8_t *)ctx->ap.p;
+  pp.rowsum = (int32_t *)ctx->rowsum.p;
+  pp.exps = (int32_t *)ctx->exps.p;
+  pp.flags = (uint32_t *)ctx->flags.p;
+  pp.blocksum = (int32_t *)ctx->blocksum.p;
+  pp.k = k;
+  pp.nb = nb;
+  pp.R = R;
+  pp.rs = R;
+  pp.act_dtype = act_dtype;
+  pp.m = (int)m;
+  HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_DIGITS, &pp, nullptr, 0, (unsigned)m));
+  pr.ap = pp.ap;
+  pr.rowsum = pp.rowsum;
+  pr.exps = pp.exps;
+  pr.flags = pp.flags;
+  pr.blocksum = pp.blocksum;
+  TkLaunchCfg cfg = {};
+  cfg.planes = layer->n_planes;
+  cfg.rt = R <= 16 ? 1 : (R <= 32 ? 2 : 4);
+  cfg.lds_bytes = lds;
+  cfg.waves = flow_waves(lds);
+  // tiles per run: as the plain flow kernel (2 / 4 / 8 for one / two / four row tiles), fewer when
+  // the launch would not give every CU its workgroups
+  int s_tiles = cfg.rt == 1 ? 2 : (cfg.rt == 2 ? 4 : 8);
+  const unsigned per_cu = cfg.waves >= 8 ? 1u : 2u;
+  while (s_tiles > 1 && (unsigned)pr.n_tiles / ((unsigned)cfg.waves * (unsigned)s_tiles) < per_cu * (unsigned)ctx->info.compute_units)
+    --s_tiles;
+  pr.run_tiles = s_tiles;
+  const unsigned per_wg = (unsigned)cfg.waves * (unsigned)s_tiles;
+  cfg.grid = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
+  HIPCHK(tk_launch_salt_flow(ctx->stream, &pr, cfg));
+  return TK_OK;
+}
+
+extern "C" int tk_linear_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
+                              void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_salt(ctx, layer, act, act_dtype, m, out, out_dtype, false);
+}
+
+extern "C" int tk_linear_salt_seq(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
+                                  void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_salt(ctx, layer, act, act_dtype, m, out, out_dtype, true);
 }
 
 extern "C" int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,

@@ -35,6 +35,10 @@ struct TkProblem {
   const int32_t *exps;       // DIGITS: [M] binary exponent of the fixed-point grid
   const uint32_t *flags;     // [M] non-zero -> row takes the exact sequential fallback (or null)
   const void *raw_act;       // original activations [M,K] for the fallback (or null)
+  // block-scale planes only: per plane the f32 block scales [(tile, K block), 16 rows], and the sums
+  // of every operand row over each K block [nb][R]
+  const float *bscale[TK_MAX_PLANES];
+  const int32_t *blocksum;
   void *out;                 // [M,N]
   int n, k, nb, R, M;
   int rs;                    // row stride of `ap` in rows (>= R; the GEMM pads it, see tk_api.hip)
@@ -68,6 +72,7 @@ struct TkPrep {
   // A8 only: RMSNorm of each row in front of the quantization (norm_kind 0 = none, 1 = scale w,
   // 2 = scale 1 + w). A normalized row that holds NaN or Inf is also written to ynorm [m,k] f32,
   // which the exact fallback of such rows reads in place of the raw activation.
+  int32_t *blocksum;    // DIGITS, optional: [nb][R] sums of each operand row over one K block
   int norm_kind;
   float norm_eps;
   const float *norm_w;  // [k]
@@ -89,7 +94,7 @@ extern "C++" {
 #endif
 // kernel launchers (tk_kernels.hip). Return hipError_t from the launch.
 hipError_t tk_launch_relayout_tq2(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb,
-                                  int *invalid_row);
+                                  int *invalid_row, float *block_scales);
 hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb);
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
                                   int8_t *trits);
@@ -108,6 +113,10 @@ int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
 int tk_flow_ring(const int *nbs, const double *weights, int count, int rt);
 int tk_flow32_runs_per_wave(void);
+// block-scale planes (float activations): flow form for <= 64 operand rows resident in LDS, and the
+// reference-order kernel for everything else
+hipError_t tk_launch_salt_flow(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg);
+hipError_t tk_launch_salt_seq(hipStream_t s, const TkProblem *single);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);

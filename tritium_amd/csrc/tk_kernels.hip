@@ -781,6 +781,187 @@ __device__ __forceinline__ RowConst row_const_from_lds(const uint8_t *cst, int m
 }
 
 // ------------------------------------------------------------------------------------------
+// Block-scale additive planes (SALT, crates/tritium-format/src/salt.rs:1-19): every plane is a
+// TQ2_0 row whose per-256-block f16 scale counts, W[n,k] = sum_p s_p[n, k/256] * trit_p[n,k], and
+// out[m,n] = sum_k act[m,k] * W[n,k] on float activations. Host definition: dequantize the row (planes
+// added in order, f32), then one f32 accumulator over k (crates/tritium-nn/src/layers/packed_salt.rs:
+// 585-628); the reference's own GPU kernel is held to 1e-4 of that
+// (crates/tritium-cuda/kernels/tq2_0_add.cu:640-719).
+// ------------------------------------------------------------------------------------------
+
+// The host's order, exactly: used for launches the flow form does not take and for tokens holding
+// NaN or Inf.
+__device__ __noinline__ float salt_exact_dot(const TkProblem &pr, int n, int tok) {
+  const int nb = pr.nb, kdim = pr.k, planes = pr.planes;
+  const size_t tile_base = (size_t)(n >> 4) * nb;
+  float acc = 0.0f;
+  for (int kb = 0; kb < nb; ++kb) {
+    float sc[TK_MAX_PLANES];
+    for (int p = 0; p < planes; ++p) sc[p] = pr.bscale[p][(tile_base + kb) * 16 + (n & 15)];
+    const int kend = min(kdim, (kb + 1) * 256);
+    for (int k = kb * 256; k < kend; ++k) {
+      float w = 0.0f;
+      for (int p = 0; p < planes; ++p) w = __fadd_rn(w, __fmul_rn(sc[p], (float)(code_at(pr.codes[p], nb, n, k) - 1)));
+      acc = __fadd_rn(acc, __fmul_rn(load_act(pr.raw_act, pr.raw_dtype, (size_t)tok * kdim + k), w));
+    }
+  }
+  return acc;
+}
+
+__global__ __launch_bounds__(TK_WG) void tk_salt_seq_kernel(TkProblem pr) {
+  size_t idx = (size_t)blockIdx.x * TK_WG + threadIdx.x;
+  size_t total = (size_t)pr.M * pr.n;
+  if (idx >= total) return;
+  store_out(pr.out, pr.out_dtype, idx, salt_exact_dot(pr, (int)(idx % pr.n), (int)(idx / pr.n)));
+}
+
+// Flow form: the stream, ring and LDS-resident operand rows of tk_flow_kernel (one run per wave, three
+// ring positions), float activations as four digit rows per token. What differs is that a K block
+// is finished on its own: after its four MFMA steps the lane turns the block's integer sums into
+// the token's value (minus the block's operand-row sums, which stand in for code = trit + 1),
+// multiplies by the block scale of its output column and adds that to a float accumulator; the
+// integer accumulators start again from zero. Per block: exact up to 1.5 ulp; the f32 sum over
+// blocks and planes is what the 1e-4 bound covers.
+template <int P, int RT>
+__global__ __launch_bounds__(512) void tk_salt_flow_kernel(const TkProblem single) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const TkProblem &pr = *single_problem();
+  constexpr int DR = 3, D = DR - 1;
+  const int NW = (int)(blockDim.x >> 6);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int i = lane & 15, g = lane >> 4;
+  const int nb = pr.nb, R = pr.R, S = pr.run_tiles, n_tiles = pr.n_tiles, M = pr.M, ncols = pr.n;
+  const int out_dtype = pr.out_dtype;
+  void *const out = pr.out;
+  const uint8_t *codes[P];
+  const float *bscale[P];
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    codes[p] = pr.codes[p];
+    bscale[p] = pr.bscale[p];
+  }
+  const int nbpad = (nb + DR - 1) / DR * DR;
+  const int first = (blockIdx.x * NW + wave) * S;
+  const unsigned plane_last = (unsigned)n_tiles * (unsigned)nb - 1u;
+  unsigned roff = (unsigned)first * (unsigned)nb * 1024u + (unsigned)lane * 16u;
+  const unsigned run_last = (unsigned)(first + S - 1) * (unsigned)nb + (unsigned)nb - 1u;
+  const unsigned last_off = min(run_last, plane_last) * 1024u + (unsigned)lane * 16u;
+
+  uint4 ring[DR][P];
+  float ring_s[DR][P];
+  auto request = [&](int slot, bool real) {
+    const unsigned off = min(roff, last_off);
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      ring[slot][p] = gload16(codes[p] + (size_t)off);
+      ring_s[slot][p] = gload(bscale[p] + (size_t)(off >> 10) * 16 + i);  // chunk index * 16 + column
+    }
+    roff += real ? 1024u : 0u;
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d) request(d, d < nb);
+
+  // operand rows, then the per-block row sums behind them
+  int *lds_bs = (int *)(smem + (size_t)nb * 256 * R);
+  {
+    const uint4 *ap4 = (const uint4 *)pr.ap;
+    uint4 *lds4w = (uint4 *)smem;
+    const int cnt = nb * 16 * R;
+    for (int idx = threadIdx.x; idx < cnt; idx += (int)blockDim.x) lds4w[idx] = gload16(ap4 + idx);
+    for (int idx = threadIdx.x; idx < nb * R; idx += (int)blockDim.x) lds_bs[idx] = gload(pr.blocksum + idx);
+  }
+  int exps[RT];
+  unsigned flag[RT];
+  unsigned any_flag = 0;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int tok = rt * 4 + g;
+    exps[rt] = tok < M ? gload(pr.exps + tok) : 0;
+    flag[rt] = tok < M && pr.flags ? gload(pr.flags + tok) : 0u;
+    any_flag |= flag[rt];
+  }
+  __syncthreads();
+  const uint4 *lds4 = (const uint4 *)smem;
+  int arow[RT], srow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    arow[rt] = min(rt * 16 + i, R - 1);
+    srow[rt] = min(rt * 16 + 4 * g, R - 4);  // R is a multiple of 4 (four digit rows per token)
+  }
+
+  for (int s = 0; s < S; ++s) {
+    v4i acc[RT][P];
+    float facc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      facc[rt] = 0.0f;
+#pragma unroll
+      for (int p = 0; p < P; ++p) acc[rt][p] = v4i{0, 0, 0, 0};
+    }
+    int kbg = 0;
+    do {
+#pragma unroll
+      for (int d = 0; d < DR; ++d) {
+        const int kb = kbg + d;
+        {
+          int kb2 = kb + D;
+          if (kb2 >= nbpad) kb2 -= nbpad;
+          request((d + D) % DR, kb2 < nb);
+        }
+        if (kb < nb) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            v4i a[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+              const uint4 q = lds4[((kb * 4 + j) * 4 + g) * R + arow[rt]];
+              a[rt] = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+            }
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+              const uint4 w = ring[d][p];
+              const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
+              const v4i b = expand_codes(wj);
+#pragma unroll
+              for (int rt = 0; rt < RT; ++rt)
+                acc[rt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[rt][p], 0, 0, 0);
+            }
+          }
+          // finish the block: value of the token's dot product over these 256 k, times the block scale
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            const v4i rs = *(const v4i *)(lds_bs + kb * R + srow[rt]);
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+              const float v = digits_to_float(acc[rt][p][3] - rs[3], acc[rt][p][2] - rs[2], acc[rt][p][1] - rs[1],
+                                              acc[rt][p][0] - rs[0], exps[rt]);
+              facc[rt] = __fadd_rn(facc[rt], __fmul_rn(v, ring_s[d][p]));
+              acc[rt][p] = v4i{0, 0, 0, 0};
+            }
+          }
+        }
+      }
+      kbg += DR;
+    } while (kbg < nbpad);
+
+    const int t = first + s, n = t * 16 + i;
+    if (t < n_tiles && n < ncols) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int tok = rt * 4 + g;
+        if (tok < M && !flag[rt]) store_out(out, out_dtype, (size_t)tok * ncols + n, facc[rt]);
+      }
+      if (any_flag) {
+        for (int rt = 0; rt < RT; ++rt) {
+          const int tok = rt * 4 + g;
+          if (tok < M && flag[rt]) store_out(out, out_dtype, (size_t)tok * ncols + n, salt_exact_dot(pr, n, tok));
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // flow kernel for 17..64 operand rows on v_mfma_i32_32x32x32_i8 (4.0 POPS sustained where the
 // 16x16x64 form stops at 3.0: at these row counts the decode kernel is limited by the matrix pipe and
 // the vector work around it as much as by memory). Same stream and ring as tk_flow_kernel; what
@@ -1697,8 +1878,16 @@ __global__ __launch_bounds__(TK_WG) void tk_seq_kernel(TkProblem pr) {
 // ------------------------------------------------------------------------------------------
 
 // TQ2_0 (66-byte blocks, only 2-byte aligned) -> T16. One thread per 16-byte piece.
+// IEEE binary16 bits -> float, exact
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+  const uint32_t sign = (h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+  if (exp == 0) return __uint_as_float(sign) + (sign ? -1.0f : 1.0f) * (float)man * 5.9604644775390625e-8f;  // man * 2^-24
+  if (exp == 31) return __uint_as_float(sign | 0x7F800000u | (man << 13));
+  return __uint_as_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
 __global__ void tk_relayout_tq2_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ codes, size_t n,
-                                       size_t nb, size_t pieces, int *invalid_row) {
+                                       size_t nb, size_t pieces, int *invalid_row, float *__restrict__ block_scales) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= pieces) return;
   size_t l = idx & 63, chunk = idx >> 6;
@@ -1720,6 +1909,16 @@ __global__ void tk_relayout_tq2_kernel(const uint8_t *__restrict__ raw, uint8_t 
     if (bad) atomicMin(invalid_row, (int)row);
   }
   ((uint4 *)codes)[idx] = make_uint4(w[0], w[1], w[2], w[3]);
+  // the block's f16 scale (crates/tritium-format/src/lib.rs:359-371), kept for the block-scale planes:
+  // entry (chunk, row of the tile) as f32, 0 for the padding rows of the last tile
+  if (block_scales && g == 0) {
+    float sc = 0.0f;
+    if (row < n) {
+      const uint8_t *blk = raw + (row * nb + kb) * 66;
+      sc = f16_bits_to_f32((uint32_t)blk[64] | ((uint32_t)blk[65] << 8));
+    }
+    block_scales[chunk * 16 + (l & 15)] = sc;
+  }
 }
 
 // TQ1_0 (54-byte base-3 blocks, crates/tritium-format/src/tq1.rs:85-121) -> T16 2-bit codes.
@@ -2037,6 +2236,26 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
     }
 #pragma unroll
     for (int dg = 0; dg < 4; ++dg) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, tok * 4 + dg)) = piece[dg];
+    if (pp.blocksum) {
+      // sums of each digit row over this K block alone (the 16 pieces of a block sit in 16
+      // consecutive lanes): entry [kb][row], row stride = the operand row count
+      int bs[4];
+#pragma unroll
+      for (int dg = 0; dg < 4; ++dg) {
+        int v = 0;
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+          const uint32_t u = piece[dg][sl];
+          v += (int)(int8_t)(u & 0xFF) + (int)(int8_t)((u >> 8) & 0xFF) + (int)(int8_t)((u >> 16) & 0xFF) + (int)(int8_t)(u >> 24);
+        }
+        for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        bs[dg] = v;
+      }
+      if (q16 == 0) {
+#pragma unroll
+        for (int dg = 0; dg < 4; ++dg) pp.blocksum[kb * pp.R + tok * 4 + dg] = bs[dg];
+      }
+    }
   }
 #pragma unroll
   for (int dg = 0; dg < 4; ++dg) {
@@ -2097,11 +2316,11 @@ __global__ void tk_copy_kernel_dev(uint4 *__restrict__ dst, const uint4 *__restr
 static inline unsigned grid_for(size_t total, unsigned block) { return (unsigned)((total + block - 1) / block); }
 
 hipError_t tk_launch_relayout_tq2(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb,
-                                  int *invalid_row) {
+                                  int *invalid_row, float *block_scales) {
   size_t pieces = ((n + 15) / 16) * nb * 64;
   if (!pieces) return hipSuccess;
   hipLaunchKernelGGL(tk_relayout_tq2_kernel, dim3(grid_for(pieces, 256)), dim3(256), 0, s, raw, codes, n, nb, pieces,
-                     invalid_row);
+                     invalid_row, block_scales);
   return hipGetLastError();
 }
 
@@ -2376,6 +2595,43 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
   }
 #undef TK_GEMM_CASE
 #undef TK_GEMM32_CASE
+  return hipGetLastError();
+}
+
+template <int P>
+static hipError_t launch_salt_p(hipStream_t s, const TkProblem &sg, const TkLaunchCfg &cfg) {
+  TkLaunchCfg c = cfg;
+  auto go = [&](auto kernel) {
+    if (c.lds_bytes > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kernel, dim3(c.grid), dim3(c.waves * 64), c.lds_bytes, s, sg);
+    return hipGetLastError();
+  };
+  switch (cfg.rt) {
+    case 1: return go(tk_salt_flow_kernel<P, 1>);
+    case 2: return go(tk_salt_flow_kernel<P, 2>);
+    case 4: return go(tk_salt_flow_kernel<P, 4>);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t tk_launch_salt_flow(hipStream_t s, const TkProblem *single, const TkLaunchCfg &cfg) {
+  if (!cfg.grid) return hipSuccess;
+  switch (cfg.planes) {
+    case 1: return launch_salt_p<1>(s, *single, cfg);
+    case 2: return launch_salt_p<2>(s, *single, cfg);
+    case 3: return launch_salt_p<3>(s, *single, cfg);
+    case 4: return launch_salt_p<4>(s, *single, cfg);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t tk_launch_salt_seq(hipStream_t s, const TkProblem *single) {
+  size_t total = (size_t)single->M * single->n;
+  if (!total) return hipSuccess;
+  hipLaunchKernelGGL(tk_salt_seq_kernel, dim3(grid_for(total, TK_WG)), dim3(TK_WG), 0, s, *single);
   return hipGetLastError();
 }
 
