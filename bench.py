@@ -281,6 +281,42 @@ def bench_config5(T, be, rng):
     return res
 
 
+def bench_salt(T, be, rng, iters=30):
+    """Block-scale additive planes (SALT): the headline shape K=2048 x 2 planes with per-256-block f16
+    scales, one tall layer of N = 262,144 output channels per launch (2 x 134 MB of codes; two
+    layers alternate, so the 0.54 GB working set exceeds the last-level cache), bf16 activations, f32
+    out. Algorithmic bytes count the block scales at their f16 size."""
+    k, n_unit, reps, planes = K2, N2, 32, 2
+    n = n_unit * reps
+    nb = (k + 255) // 256
+    layers = []
+    for _ in range(2):
+        bufs = []
+        for p0 in (0.4, 0.7):
+            trits = ternary(rng, n_unit, k, p0)
+            packed = T.pack_rows(trits, n_unit, k).reshape(n_unit, nb, 66).copy()
+            sc = rng.uniform(0.02, 1.0, (n_unit, nb)).astype(np.float16).view(np.uint16)
+            packed[:, :, 64] = (sc & 0xFF).astype(np.uint8)
+            packed[:, :, 65] = (sc >> 8).astype(np.uint8)
+            bufs.append(be.upload_weights_scaled(np.tile(packed.reshape(-1), reps), T.GemmShape(0, n, k)))
+        layers.append(bufs)
+    res = {"workload": f"2 block-scale planes, K={k}, N={n} per launch (two layers alternate), bf16 activations, f32 out, "
+                       "digit split + contraction"}
+    for m in (1, 4, 16):
+        act = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32)), "bf16")
+        out = be.empty(m * n, "f32")
+        ms = time_calls(be, lambda i: be.linear_salt(layers[i % 2], act, m, out), iters)
+        by = planes * n * nb * (64 + 2) + m * k * 2 + m * n * 4
+        res[f"batch{m}"] = {"ms_per_call": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+                            "frac_of_hbm_peak": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        act.free()
+        out.free()
+    for bufs in layers:
+        for b in bufs:
+            b.free()
+    return res
+
+
 def bench_stack(T, be, rng, iters=100):
     """configs[3]: the 7 ternary projections of 30 decoder layers (hidden 2560, FFN 6912, 20 query
     heads and 5 KV heads of 128), W1.58A8, one launch for the whole stack with given inputs.
@@ -373,7 +409,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,salt",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -427,7 +463,8 @@ def main():
                 "config1": ("config1_f32_batch1", lambda: bench_config1(T, be, rng)),
                 "prefill": ("prefill_gemm", lambda: bench_prefill(T, be, rng, 2048, 2560, 6912)),
                 "stack": ("projection_stack", lambda: bench_stack(T, be, rng)),
-                "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng))}
+                "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng)),
+                "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng))}
         out["extra"] = {}
         for leg in [x for x in args.extra_legs.split(",") if x]:
             if leg not in legs:

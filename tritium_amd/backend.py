@@ -285,7 +285,7 @@ class Mi355xBackend:
     def capabilities(self):
         return DeviceCaps(backend="mi355x", device_name=self.info.name.decode(),
                           features=["hip", self.info.arch.decode().split(":")[0], "tq2_0", "tq1_0", "mfma_i8",
-                                    "act_quant_i8", "additive_planes", "rmsnorm_quant_i8"],
+                                    "act_quant_i8", "additive_planes", "rmsnorm_quant_i8", "salt_block_scales"],
                           total_memory_bytes=int(self.info.total_memory_bytes), supports_imma=True,
                           supports_fp8=False)
 

@@ -163,7 +163,7 @@ class Mi355xBackend : public TernaryBackend {
     DeviceCaps c;
     c.backend = "mi355x";
     c.device_name = info.name;
-    c.features = {"hip", "gfx950", "tq2_0", "tq1_0", "mfma_i8", "act_quant_i8", "additive_planes", "rmsnorm_quant_i8"};
+    c.features = {"hip", "gfx950", "tq2_0", "tq1_0", "mfma_i8", "act_quant_i8", "additive_planes", "rmsnorm_quant_i8", "salt_block_scales"};
     c.total_memory_bytes = info.total_memory_bytes;
     c.supports_imma = true;
     return c;
