@@ -815,18 +815,18 @@ __global__ __launch_bounds__(TK_WG) void tk_salt_seq_kernel(TkProblem pr) {
   store_out(pr.out, pr.out_dtype, idx, salt_exact_dot(pr, (int)(idx % pr.n), (int)(idx / pr.n)));
 }
 
-// Flow form: the stream, ring and LDS-resident operand rows of tk_flow_kernel (one run per wave, three
-// ring positions), float activations as four digit rows per token. What differs is that a K block
+// Flow form: the stream, ring and LDS-resident operand rows of tk_flow_kernel (one run per wave),
+// float activations as four digit rows per token. What differs is that a K block
 // is finished on its own: after its four MFMA steps the lane turns the block's integer sums into
 // the token's value (minus the block's operand-row sums, which stand in for code = trit + 1),
 // multiplies by the block scale of its output column and adds that to a float accumulator; the
 // integer accumulators start again from zero. Per block: exact up to 1.5 ulp; the f32 sum over
 // blocks and planes is what the 1e-4 bound covers.
-template <int P, int RT>
+template <int P, int RT, int DR>
 __global__ __launch_bounds__(512) void tk_salt_flow_kernel(const TkProblem single) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = *single_problem();
-  constexpr int DR = 3, D = DR - 1;
+  constexpr int D = DR - 1;
   const int NW = (int)(blockDim.x >> 6);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int i = lane & 15, g = lane >> 4;
@@ -893,11 +893,7 @@ __global__ __launch_bounds__(512) void tk_salt_flow_kernel(const TkProblem singl
     v4i acc[RT][P];
     float facc[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      facc[rt] = 0.0f;
-#pragma unroll
-      for (int p = 0; p < P; ++p) acc[rt][p] = v4i{0, 0, 0, 0};
-    }
+    for (int rt = 0; rt < RT; ++rt) facc[rt] = 0.0f;
     int kbg = 0;
     do {
 #pragma unroll
@@ -923,20 +919,20 @@ __global__ __launch_bounds__(512) void tk_salt_flow_kernel(const TkProblem singl
               const uint32_t wj = j == 0 ? w.x : (j == 1 ? w.y : (j == 2 ? w.z : w.w));
               const v4i b = expand_codes(wj);
 #pragma unroll
-              for (int rt = 0; rt < RT; ++rt)
-                acc[rt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[rt][p], 0, 0, 0);
+              for (int rt = 0; rt < RT; ++rt)  // the first step of a block starts from zero
+                acc[rt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, j == 0 ? v4i{0, 0, 0, 0} : acc[rt][p], 0, 0, 0);
             }
           }
-          // finish the block: value of the token's dot product over these 256 k, times the block scale
+          // finish the block: the token's dot product over these 256 k in units of its grid (the
+          // power of two is applied once, after the last block), times the block scale
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) {
             const v4i rs = *(const v4i *)(lds_bs + kb * R + srow[rt]);
 #pragma unroll
             for (int p = 0; p < P; ++p) {
               const float v = digits_to_float(acc[rt][p][3] - rs[3], acc[rt][p][2] - rs[2], acc[rt][p][1] - rs[1],
-                                              acc[rt][p][0] - rs[0], exps[rt]);
+                                              acc[rt][p][0] - rs[0], 0);
               facc[rt] = __fadd_rn(facc[rt], __fmul_rn(v, ring_s[d][p]));
-              acc[rt][p] = v4i{0, 0, 0, 0};
             }
           }
         }
@@ -949,7 +945,7 @@ __global__ __launch_bounds__(512) void tk_salt_flow_kernel(const TkProblem singl
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         const int tok = rt * 4 + g;
-        if (tok < M && !flag[rt]) store_out(out, out_dtype, (size_t)tok * ncols + n, facc[rt]);
+        if (tok < M && !flag[rt]) store_out(out, out_dtype, (size_t)tok * ncols + n, ldexpf(facc[rt], exps[rt]));
       }
       if (any_flag) {
         for (int rt = 0; rt < RT; ++rt) {
@@ -2610,9 +2606,11 @@ static hipError_t launch_salt_p(hipStream_t s, const TkProblem &sg, const TkLaun
     return hipGetLastError();
   };
   switch (cfg.rt) {
-    case 1: return go(tk_salt_flow_kernel<P, 1>);
-    case 2: return go(tk_salt_flow_kernel<P, 2>);
-    case 4: return go(tk_salt_flow_kernel<P, 4>);
+    // three ring positions for every row-tile count: the depths the plain flow kernel likes
+    // (5 / 4 / 2) measured 2-7% slower here
+    case 1: return go(tk_salt_flow_kernel<P, 1, 3>);
+    case 2: return go(tk_salt_flow_kernel<P, 2, 3>);
+    case 4: return go(tk_salt_flow_kernel<P, 4, 3>);
     default: return hipErrorInvalidValue;
   }
 }
