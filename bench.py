@@ -416,8 +416,8 @@ def main():
                     help="also launch a plain 1 GiB device copy kernel 3 times (scale for hardware traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (the path shards over output channels without any "
-                 "exchange, see DESIGN.md); --gpus N with N > 1 is not supported.")
+        sys.exit("bench.py: this build runs on ONE GPU (the path would shard over output channels, each GPU "
+                 "holding a slice of every plane, without any exchange); --gpus N with N > 1 is not supported.")
     import tritium_amd as T
     be = T.Mi355xBackend(0)
     info = be.info
