@@ -2106,6 +2106,43 @@ __device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const T
   return table[lo];
 }
 
+// The 16 elements of operand piece (kb, q16) of a row: four groups of four, 32 elements apart.
+__device__ __forceinline__ void load_piece(const void *act, int dtype, size_t base, size_t e0, size_t k, bool vec,
+                                           float (&v)[16]) {
+#pragma unroll
+  for (int sl = 0; sl < 4; ++sl) {
+    float t[4];
+    load_act4(act, dtype, base, e0 + (size_t)sl * 32, k, vec, t);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) v[sl * 4 + b] = t[b];
+  }
+}
+
+// Rows of up to TK_PREP_HELD * 256 pieces (K <= 16384) are read from memory once: every thread keeps
+// its pieces in registers between the pass that finds the row maximum and the pass that quantizes.
+#define TK_PREP_HELD 4
+__device__ __forceinline__ void row_absmax_held(const void *act, int dtype, size_t base, size_t k, size_t npieces,
+                                                bool vec, float (&held)[TK_PREP_HELD][16], float *sh, float &gamma,
+                                                int &nonfinite, int *shi) {
+  float g = 0.0f;
+  int nf = 0;
+#pragma unroll
+  for (int it = 0; it < TK_PREP_HELD; ++it) {
+    const size_t pc = (size_t)threadIdx.x + (size_t)it * TK_WG;
+    if (pc < npieces) {
+      load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, held[it]);
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const float a = fabsf(held[it][x]);  // elements past k were loaded as 0
+        if (a > g) g = a;
+        nf |= !(a <= 3.402823466e38f);
+      }
+    }
+  }
+  gamma = block_max(g, sh);
+  nonfinite = block_sum(nf, shi) != 0;
+}
+
 // Per-token int8 absmax quant (crates/tritium-spec/src/lib.rs:351-378) straight into operand order.
 __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                            int nprep) {
@@ -2125,14 +2162,21 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
     __shared__ float part[TK_WG];
     nm.inv = row_inv_rms(act, dtype, base, k, pp.norm_eps, part);
   }
+  const size_t npieces = nb * 16;
+  const bool resident = !nm.kind && npieces <= (size_t)TK_PREP_HELD * TK_WG;
+  float held[TK_PREP_HELD][16];
   float gamma;
   int nonfinite;
-  row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi, nm);
+  if (resident)
+    row_absmax_held(act, dtype, base, k, npieces, vec, held, shf, gamma, nonfinite, shi);
+  else
+    row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi, nm);
   if (nm.kind && nonfinite) ynorm = pp.ynorm;  // only the exact fallback reads the normalized row
   const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
   const bool live = gamma != 0.0f && !nonfinite;
   int sum = 0;
-  for (size_t pc = threadIdx.x; pc < nb * 16; pc += TK_WG) {
+  // quantize the 16 values of piece pc and store them in operand order (and row-major, if asked)
+  auto emit = [&](size_t pc, const float (&v)[16]) {
     const size_t kb = pc >> 4;
     const int q16 = (int)(pc & 15);
     const size_t e0 = piece_elem0(kb, q16);
@@ -2140,20 +2184,17 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
 #pragma unroll
     for (int sl = 0; sl < 4; ++sl) {
       const size_t e = e0 + (size_t)sl * 32;
-      float v[4];
-      load_act4(act, dtype, base, e, k, vec, v);
-      apply_norm4(nm, e, k, v);
       if (ynorm) {
 #pragma unroll
         for (int b = 0; b < 4; ++b)
-          if (e + b < k) gstore(ynorm + base + e + b, v[b]);
+          if (e + b < k) gstore(ynorm + base + e + b, v[sl * 4 + b]);
       }
       uint32_t packed = 0;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         int q = 0;
         if (live && e + b < k) {
-          float r = rintf(__fmul_rn(v[b], s));  // one multiply, ties to even
+          float r = rintf(__fmul_rn(v[sl * 4 + b], s));  // one multiply, ties to even
           r = r < -128.0f ? -128.0f : (r > 127.0f ? 127.0f : r);
           q = (int)r;
         }
@@ -2171,6 +2212,27 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
       }
     }
     if (ap) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, row)) = piece;
+  };
+  if (resident) {
+#pragma unroll
+    for (int it = 0; it < TK_PREP_HELD; ++it) {
+      const size_t pc = (size_t)threadIdx.x + (size_t)it * TK_WG;
+      if (pc < npieces) emit(pc, held[it]);
+    }
+  } else {
+    for (size_t pc = threadIdx.x; pc < npieces; pc += TK_WG) {
+      float v[16];
+      const size_t e0 = piece_elem0(pc >> 4, (int)(pc & 15));
+      load_piece(act, dtype, base, e0, k, vec, v);
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        float t[4] = {v[sl * 4], v[sl * 4 + 1], v[sl * 4 + 2], v[sl * 4 + 3]};
+        apply_norm4(nm, e0 + (size_t)sl * 32, k, t);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) v[sl * 4 + b] = t[b];
+      }
+      emit(pc, v);
+    }
   }
   sum = block_sum(sum, shi);
   if (threadIdx.x == 0) {
@@ -2196,15 +2258,22 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
   const int dtype = pp.act_dtype;
   int8_t *ap = pp.ap;
   const bool vec = act_rows_vectorizable(act, dtype, k);
+  const size_t npieces = nb * 16;
+  const bool resident = npieces <= (size_t)TK_PREP_HELD * TK_WG;
+  float held[TK_PREP_HELD][16];
   float gamma;
   int nonfinite;
-  row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi);
+  if (resident)
+    row_absmax_held(act, dtype, base, k, npieces, vec, held, shf, gamma, nonfinite, shi);
+  else
+    row_absmax(act, dtype, base, k, vec, shf, gamma, nonfinite, shi);
   int E = 0;
   if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
   const int shift = 30 - E;
   const bool live = gamma != 0.0f && !nonfinite;
   int sums[4] = {0, 0, 0, 0};
-  for (size_t pc = threadIdx.x; pc < nb * 16; pc += TK_WG) {
+  // split the 16 values of piece pc into their four digit rows and store those in operand order
+  auto emit = [&](size_t pc, const float (&v)[16]) {
     const size_t kb = pc >> 4;
     const int q16 = (int)(pc & 15);
     const size_t e0 = piece_elem0(kb, q16);
@@ -2212,13 +2281,11 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
 #pragma unroll
     for (int sl = 0; sl < 4; ++sl) {
       const size_t e = e0 + (size_t)sl * 32;
-      float v[4];
-      load_act4(act, dtype, base, e, k, vec, v);
       uint32_t packed[4] = {0, 0, 0, 0};
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         int q = 0;
-        if (live && e + b < k) q = __float2int_rn(ldexpf(v[b], shift));  // |q| <= 2^30
+        if (live && e + b < k) q = __float2int_rn(ldexpf(v[sl * 4 + b], shift));  // |q| <= 2^30
 #pragma unroll
         for (int dg = 0; dg < 4; ++dg) {
           int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
@@ -2238,19 +2305,32 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
       int bs[4];
 #pragma unroll
       for (int dg = 0; dg < 4; ++dg) {
-        int v = 0;
+        int t = 0;
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
           const uint32_t u = piece[dg][sl];
-          v += (int)(int8_t)(u & 0xFF) + (int)(int8_t)((u >> 8) & 0xFF) + (int)(int8_t)((u >> 16) & 0xFF) + (int)(int8_t)(u >> 24);
+          t += (int)(int8_t)(u & 0xFF) + (int)(int8_t)((u >> 8) & 0xFF) + (int)(int8_t)((u >> 16) & 0xFF) + (int)(int8_t)(u >> 24);
         }
-        for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o);
-        bs[dg] = v;
+        for (int o = 8; o > 0; o >>= 1) t += __shfl_xor(t, o);
+        bs[dg] = t;
       }
       if (q16 == 0) {
 #pragma unroll
         for (int dg = 0; dg < 4; ++dg) pp.blocksum[kb * pp.R + tok * 4 + dg] = bs[dg];
       }
+    }
+  };
+  if (resident) {
+#pragma unroll
+    for (int it = 0; it < TK_PREP_HELD; ++it) {
+      const size_t pc = (size_t)threadIdx.x + (size_t)it * TK_WG;
+      if (pc < npieces) emit(pc, held[it]);
+    }
+  } else {
+    for (size_t pc = threadIdx.x; pc < npieces; pc += TK_WG) {
+      float v[16];
+      load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, v);
+      emit(pc, v);
     }
   }
 #pragma unroll
