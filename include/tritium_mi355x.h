@@ -204,9 +204,10 @@ typedef struct tk_salt_desc {
   const tk_weights *planes[TK_MAX_PLANES]; /* each from tk_upload_weights_scaled, same [n,k] */
   int n_planes;
 } tk_salt_desc;
-/* act [m,k] f32 or bf16, out [m,n] f32 or bf16. Up to 16 tokens whose four digit rows fit in LDS
- * run on the matrix cores, block by block (within 1e-4 of the host definition, normally ~1e-6);
- * other shapes, and tokens holding NaN or Inf, take the host's order exactly (slow). */
+/* act [m,k] f32 or bf16, out [m,n] f32 or bf16. Tokens run on the matrix cores, block by block,
+ * 16 at a time (within 1e-4 of the host definition, normally ~1e-6; more than 16 tokens stream the
+ * planes once per 16); rows too long for LDS (K beyond ~9,800) and tokens holding NaN or Inf take
+ * the host's order exactly (slow). */
 int tk_linear_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
                    void *out, int out_dtype);
 /* The host's order for every output: bit-identical to dequantize-then-fold. */

@@ -802,6 +802,17 @@ static int run_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int
   pr.raw_act = act;
   pr.raw_dtype = act_dtype;
   pr.out = out;
+  // More than 16 tokens: slices of 16 go through the matrix-core form one after the other (each
+  // streams the planes again; a block-scale form of the prefill kernel does not exist yet).
+  if (!seq && m > 16 && nb * 256 * 64 + nb * 64 * 4 <= kLdsFlowMax) {
+    const size_t asz = act_dtype == TK_BF16 ? 2 : 4, osz = out_dtype == TK_BF16 ? 2 : 4;
+    for (size_t m0 = 0; m0 < m; m0 += 16) {
+      const size_t mc = m - m0 < 16 ? m - m0 : 16;
+      TKCHK(run_salt(ctx, layer, (const uint8_t *)act + m0 * k * asz, act_dtype, mc, (uint8_t *)out + m0 * n * osz,
+                     out_dtype, false));
+    }
+    return TK_OK;
+  }
   const size_t lds = nb * 256 * R + nb * R * 4;  // operand rows + their per-block sums
   if (seq || R > 64 || lds > kLdsFlowMax) {
     HIPCHK(tk_launch_salt_seq(ctx->stream, &pr));
