@@ -102,3 +102,53 @@ def test_exact_max_macs_knob(backend):
     backend.set_exact_max_macs(0)
     assert backend.exact_max_macs() == 0
     backend.set_exact_max_macs(1 << 20)
+
+
+def test_one_backend_shared_by_threads(backend, oracle):
+    """TernaryBackend is Send + Sync: one object serves concurrent callers
+    (crates/tritium-spec/src/lib.rs:166; crates/tritium-rocm/src/rocm.rs:207-211). Four threads issue
+    fused calls of different shapes at the same time; every result has the oracle's bits, and an
+    error raised in one thread does not leak into another's last-error text."""
+    import threading
+
+    from helpers import same_bits, scales, ternary
+    from oracle_lib import FMT_TQ2_0
+
+    rng = np.random.default_rng(77)
+    jobs = []
+    for m, n, k in ((1, 48, 512), (3, 33, 700), (5, 130, 300), (2, 64, 1280)):
+        w, sc = ternary(rng, n, k), scales(rng, n)
+        packed = oracle.pack_matrix(w, n, k, FMT_TQ2_0)
+        buf = backend.upload_weights(packed, T.GemmShape(0, n, k), T.TernaryFormat.Tq2_0)
+        act = rng.standard_normal((m, k)).astype(np.float32)
+        rc, want = oracle.cpu_mpgemm_with_act_quant(packed, FMT_TQ2_0, act, sc, m, n, k)
+        assert rc == 0
+        jobs.append((buf, act, sc, (m, n, k), want))
+    failures = []
+
+    def worker(job, idx):
+        buf, act, sc, (m, n, k), want = job
+        try:
+            for it in range(25):
+                out = np.zeros((m, n), np.float32)
+                backend.mpgemm_with_act_quant(T.MpGemm(act, buf, sc, T.GemmShape(m, n, k), T.TernaryFormat.Tq2_0, out))
+                if not same_bits(out, want):
+                    failures.append((idx, it, "bits"))
+                if idx == 0 and it % 5 == 0:  # a failing call in one thread, while the others compute
+                    try:
+                        backend.mpgemm(T.MpGemm(act[:, :-1], buf, sc, T.GemmShape(m, n, k), T.TernaryFormat.Tq2_0, out))
+                        failures.append((idx, it, "no error"))
+                    except T.ShapeMismatch as e:
+                        if (e.expected, e.got) != (m * k, m * (k - 1)):
+                            failures.append((idx, it, "mismatch fields"))
+        except Exception as e:  # noqa: BLE001 - reported below
+            failures.append((idx, "exception", repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(job, i)) for i, job in enumerate(jobs)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures[:5]
+    for job in jobs:
+        job[0].free()
