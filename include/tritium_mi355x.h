@@ -207,7 +207,8 @@ typedef struct tk_salt_desc {
 /* act [m,k] f32 or bf16, out [m,n] f32 or bf16. Tokens run on the matrix cores, block by block,
  * 16 at a time (within 1e-4 of the host definition, normally ~1e-6; more than 16 tokens stream the
  * planes once per 16); rows too long for LDS (K beyond ~9,800) and tokens holding NaN or Inf take
- * the host's order exactly (slow). */
+ * the host's order exactly (slow). A block scale that is itself infinite or NaN makes its outputs
+ * non-finite here and NaN on the host (which multiplies it with the zero trits too). */
 int tk_linear_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
                    void *out, int out_dtype);
 /* The host's order for every output: bit-identical to dequantize-then-fold. */

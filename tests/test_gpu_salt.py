@@ -135,3 +135,36 @@ def test_scaled_upload_still_serves_the_plain_contract(backend, oracle):
         backend.linear_salt([plain], dact, m, dout)
     for a in [dact, dout, plain] + bufs:
         a.free()
+
+
+def test_every_f16_block_scale_reaches_the_kernels_exactly(backend, oracle):
+    """One row per f16 bit pattern, one non-zero trit against an activation of 1: the output is the
+    block scale itself, so the device's f16 -> f32 conversion is checked over all 65,536 patterns
+    (subnormals, zeros, infinities, NaNs) through both kernels."""
+    n, k = 65536, 256
+    trits = np.zeros((n, k), np.int8)
+    trits[:, 0] = 1
+    bits = np.arange(n, dtype=np.uint16).reshape(n, 1)
+    packed = oracle.pack_matrix_scaled(trits, bits, n, k)
+    buf = backend.upload_weights_scaled(packed, T.GemmShape(0, n, k))
+    act = np.zeros((1, k), np.float32)
+    act[0, 0] = 1.0
+    rc, want = oracle.salt_mpgemm([packed], n, k, act, 1)
+    want = want.reshape(-1)
+    scale = bits.reshape(-1).view(np.float16).astype(np.float32)
+    finite = np.isfinite(scale)
+    scale[0x8000] = 0.0  # 0.0 + (-0.0) * 1 is +0.0: the one pattern whose row is not the scale's own bits
+    assert rc == 0 and (want[finite].view(np.uint32) == scale[finite].view(np.uint32)).all()
+    assert np.isnan(want[~finite]).all()  # an infinite scale times a zero trit is NaN, on the host too
+    dact, dout = backend.to_device(act, "f32"), backend.empty(n, "f32")
+    backend.linear_salt([buf], dact, 1, dout, seq=True)
+    got = dout.to_host()
+    assert np.isnan(got[~finite]).all() and (got[finite].view(np.uint32) == want[finite].view(np.uint32)).all()
+    # the matrix-core form multiplies the block's integer sum by the scale once: the same values for
+    # every finite scale (an infinite or NaN scale gives Inf or NaN there, the host NaN)
+    backend.linear_salt([buf], dact, 1, dout)
+    got = dout.to_host()
+    assert (got[finite].view(np.uint32) == want[finite].view(np.uint32)).all()
+    assert (~np.isfinite(got[~finite])).all()
+    for a in (dact, dout, buf):
+        a.free()
