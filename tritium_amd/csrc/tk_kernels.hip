@@ -2514,7 +2514,7 @@ static hipError_t flow_launch_one(K kernel, hipStream_t s, const TkProblem &sg, 
 template <int P, int RT>
 static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                  const TkLaunchCfg &cfg) {
-  constexpr int TW = (RT >= 4 && P <= 2) ? 2 : 1;
+  constexpr int TW = ((RT >= 4 && P <= 2) || (RT == 2 && P == 1)) ? 2 : 1;
   const int threads = cfg.waves * 64;
   switch (cfg.ring) {
     case 2:
@@ -2573,8 +2573,10 @@ static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProb
   }
 }
 
-// lock-step runs per wave of the flow kernel for a (planes, rt) pair
-int tk_flow_runs_per_wave(int planes, int rt) { return (rt >= 4 && planes <= 2) ? 2 : 1; }
+// lock-step runs per wave of the flow kernel for a (planes, rt) pair: two where registers allow and a
+// single run would keep too few bytes in flight (four row tiles of one or two planes; two row
+// tiles of one plane: K=2048 N=8192, 32 int8 rows, one plane went from 263 to 228 us)
+int tk_flow_runs_per_wave(int planes, int rt) { return ((rt >= 4 && planes <= 2) || (rt == 2 && planes == 1)) ? 2 : 1; }
 // ... of the 32x32x32 form: always a pair of adjacent tiles
 int tk_flow32_runs_per_wave(void) { return 2; }
 
