@@ -504,14 +504,16 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds) {
 // win (more, shorter-lived workgroups keep more loads in flight and balance the tail). Measured on
 // K=2048 N=8192 x 2 planes over 128 layer copies: 4-16 operand rows peak at 2 tiles per run
 // (128 KiB of weights per workgroup), 32 rows at 4 (4x the staged bytes, four-wave workgroups), 64
-// rows at 8 (16x, eight-wave workgroups, one per CU).
+// rows at 8 (16x, eight-wave workgroups, one per CU). Re-measured with the ring at 4 positions: 4-8
+// operand rows (8-16 KiB staged) are 5-8% faster with runs of ONE tile (64 KiB per workgroup), 16
+// rows stay at 2.
 static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
                           size_t nb, bool wide) {
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, planes, rt);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
   size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 ? 2 : 4);
-  if (target < 128 * 1024) target = 128 * 1024;
+  if (target < 64 * 1024) target = 64 * 1024;
   size_t s = 1;
   while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
   // keep every CU supplied: two four-wave workgroups each, or one eight-wave workgroup (those fill
@@ -519,6 +521,25 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   const unsigned per_cu = waves >= 8 ? 1u : 2u;
   while (s > 1 && total_tiles / (per_s * s) < per_cu * (unsigned)ctx->info.compute_units) --s;
   return (int)s;
+}
+
+// Members of a grouped launch get whole workgroups: a member of n tiles occupies ceil(n / per) * per
+// tile slots, per = tiles per workgroup. With members of very different sizes (q/k/v/o/gate/up: 160,
+// 40, 40, 160, 432, 432 tiles) long runs leave most slots of the small members empty: shorten the
+// runs until at most a tenth of the slots is padding (30 layers x 6 projections at 32 tokens:
+// 199 -> 174 us per step).
+static int trim_run_tiles(const tk_ctx *ctx, int s, size_t per_s, const std::vector<unsigned> &member_tiles) {
+  if (ctx->flow_run_tiles > 0) return s;
+  unsigned total = 0;
+  for (unsigned n : member_tiles) total += n;
+  while (s > 1) {
+    const unsigned per = (unsigned)per_s * (unsigned)s;
+    unsigned slots = 0;
+    for (unsigned n : member_tiles) slots += (n + per - 1) / per * per;
+    if ((double)(slots - total) <= 0.10 * (double)slots) break;
+    --s;
+  }
+  return s;
 }
 
 static const size_t kLdsStreamBudget = 64 * 1024;
@@ -697,7 +718,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
     cfg.waves = flow_waves(flow_lds);
-    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt);
+    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R);
     flow_cfg_form(&cfg, wide, flow_lds);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
@@ -1155,7 +1176,12 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   const bool wide = flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
   if (wide) flds = flow_wide_lds(rt, nb_max);
   const int fw = flow_waves(flds);
-  const int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide);
+  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide);
+  {
+    std::vector<unsigned> member_tiles(count);
+    for (size_t i = 0; i < count; ++i) member_tiles[i] = (unsigned)plans[i].pr.n_tiles;
+    run_tiles = trim_run_tiles(ctx, run_tiles, (size_t)fw * (size_t)flow_runs_per_wave(wide, planes, rt), member_tiles);
+  }
   const unsigned fper = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, planes, rt) * (unsigned)run_tiles;
   unsigned fgroups = 0;
   for (size_t i = 0; i < count; ++i) {
@@ -1190,7 +1216,13 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds);
-    const int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide) : 1;
+    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide) : 1;
+    {
+      std::vector<unsigned> member_tiles;
+      for (size_t i = 0; i < count; ++i)
+        if (plans[i].flow_ok) member_tiles.push_back((unsigned)plans[i].pr.n_tiles);
+      prun = trim_run_tiles(ctx, prun, (size_t)pfw * (size_t)flow_runs_per_wave(pwide, planes, rt), member_tiles);
+    }
     const unsigned pper = (unsigned)pfw * (unsigned)flow_runs_per_wave(pwide, planes, rt) * (unsigned)prun;
     unsigned flow_total = 0;
     for (size_t i = 0; i < count; ++i) {
@@ -1219,7 +1251,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.lds_bytes = pflds;
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
-      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt);
+      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max);
       flow_cfg_form(&flow_cfg, pwide, pflds);
     }
   } else if (variant != DECODE_KSPLIT) {
@@ -1318,7 +1350,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       nbs[i] = plans[i].pr.nb;
       wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
     }
-    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt);
+    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max);
   }
   if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds);
   *out = g;

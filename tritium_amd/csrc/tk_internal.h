@@ -111,7 +111,7 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
                           const TkLaunchCfg &cfg);
 int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
-int tk_flow_ring(const int *nbs, const double *weights, int count, int rt);
+int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows);
 int tk_flow32_runs_per_wave(void);
 // block-scale planes (float activations): flow form for <= 64 operand rows resident in LDS, and the
 // reference-order kernel for everything else

@@ -2582,13 +2582,18 @@ int tk_flow32_runs_per_wave(void) { return 2; }
 
 // Ring size of the flow kernel (2..5 positions) for launches whose K block counts are nbs[0..count).
 // A deeper ring keeps more loads in flight per wave and costs registers, i.e. waves per SIMD.
-// Measured on K=2048 N=8192 x 2 planes: one row tile likes 5 positions, two row tiles 4, four row
-// tiles (250 registers, eight waves per CU whatever the ring) 2. A ring that does not divide a K
-// block count pads that problem's tiles with idle positions; a candidate is taken in the order of
-// preference unless it pads more than a quarter of the positions (weighted by each problem's chunk
-// count), and if all do, the one that pads least.
-int tk_flow_ring(const int *nbs, const double *weights, int count, int rt) {
-  const int pref1[4] = {5, 4, 3, 2}, pref2[4] = {4, 5, 3, 2}, pref4[4] = {2, 3, 4, 5};
+// Measured on K=2048 N=8192 x 2 planes: one and two row tiles like 4 positions (with runs of a
+// single tile, 4 beat 5 by 5% at 4-8 operand rows), four row tiles (250 registers, eight waves per CU
+// whatever the ring) 2. A ring that does not divide a K block count pads that problem's tiles with
+// idle positions; a candidate is taken in the order of preference unless it pads more than a tenth
+// (one row tile: K=2560 runs 2% faster on 5 positions than on 4 padded to 12) or a quarter (more
+// row tiles) of the positions, weighted by each problem's chunk count; if all do, the one that
+// pads least.
+int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows) {
+  // one row tile: 4 positions with runs of one tile (up to 8 rows), 5 with runs of two (9..16 rows)
+  const int pref1a[4] = {4, 5, 3, 2}, pref1b[4] = {5, 4, 3, 2}, pref2[4] = {4, 5, 3, 2}, pref4[4] = {2, 3, 4, 5};
+  const int *pref1 = rows <= 8 ? pref1a : pref1b;
+  const double limit = rt == 1 ? 0.10 : 0.25;
   const int *cand = rt == 1 ? pref1 : (rt == 2 ? pref2 : pref4);
   int best = cand[0];
   double best_waste = -1.0;
@@ -2601,7 +2606,7 @@ int tk_flow_ring(const int *nbs, const double *weights, int count, int rt) {
       total += w;
     }
     waste = total > 0.0 ? waste / total : 0.0;
-    if (waste <= 0.25) return cand[c];
+    if (waste <= limit) return cand[c];
     if (best_waste < 0.0 || waste < best_waste) {
       best_waste = waste;
       best = cand[c];
