@@ -871,6 +871,7 @@ static int run_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int
   // tiles per run: as the plain flow kernel (2 / 4 / 8 for one / two / four row tiles), fewer when
   // the launch would not give every CU its workgroups
   int s_tiles = cfg.rt == 1 ? 2 : (cfg.rt == 2 ? 4 : 8);
+  if (ctx->flow_run_tiles > 0) s_tiles = ctx->flow_run_tiles;
   const unsigned per_cu = cfg.waves >= 8 ? 1u : 2u;
   while (s_tiles > 1 && (unsigned)pr.n_tiles / ((unsigned)cfg.waves * (unsigned)s_tiles) < per_cu * (unsigned)ctx->info.compute_units)
     --s_tiles;
