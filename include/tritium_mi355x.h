@@ -252,10 +252,6 @@ void tk_group_destroy(tk_group *group);
 int tk_set_gemm_min_m(tk_ctx *ctx, int min_m);
 int tk_get_gemm_min_m(const tk_ctx *ctx);
 
-/* The decode path has two kernels with identical results: one splits K over the waves of a
- * workgroup (fine grain, for a single narrow layer) and one streams whole output tiles per wave
- * (for launches that fill the chip). The streaming form is taken when a launch needs at least
- * this many workgroups; default = the device's CU count. */
 /* Force one decode kernel for every later launch: 0 automatic, 1 K-split, 2 streaming (K passes
  * through LDS), 3 flow (all of K resident in LDS; falls back to 2 when it does not fit). All give
  * identical bits; the knob exists for tests and tuning. */
@@ -271,6 +267,10 @@ int tk_set_flow_ring(tk_ctx *ctx, int positions);
  * 32 = 32x32x32 wherever its operand rows fit in LDS. A tuning and test knob: both forms give
  * identical bits. */
 int tk_set_flow_mfma(tk_ctx *ctx, int rows);
+/* The K-split decode kernel has the finer grain (a single narrow layer), the streaming and flow
+ * kernels walk whole output tiles per wave (launches that fill the chip): the latter are taken when
+ * a launch needs at least this many workgroups; default = the device's CU count. No counterpart
+ * in the reference; results do not depend on it. */
 int tk_set_stream_min_groups(tk_ctx *ctx, int groups);
 int tk_get_stream_min_groups(const tk_ctx *ctx);
 
@@ -282,7 +282,9 @@ int tk_get_stream_min_groups(const tk_ctx *ctx);
 int tk_set_exact_max_macs(tk_ctx *ctx, size_t macs);
 size_t tk_get_exact_max_macs(const tk_ctx *ctx);
 
-/* ---- plumbing: device memory, stream, events (what the harness and a backend crate need) ---- */
+/* ---- plumbing: device memory, stream, events (what the harness and a backend crate need; the
+ *      reference's device backends own the same privately: crates/tritium-rocm/src/rocm.rs:84-174
+ *      device buffers, :207-242 stream and synchronous calls) ---- */
 int tk_malloc(tk_ctx *ctx, size_t bytes, void **dptr);
 int tk_free(tk_ctx *ctx, void *dptr);
 int tk_memcpy_h2d(tk_ctx *ctx, void *dst, const void *src, size_t bytes);
