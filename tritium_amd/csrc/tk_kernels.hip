@@ -1965,14 +1965,37 @@ __global__ void tk_decode_trits_kernel(const uint8_t *__restrict__ codes, size_t
 // activation prep: one workgroup per token
 // ------------------------------------------------------------------------------------------
 
-__device__ float block_max(float v, float *sh) {
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+// Row maximum and "any lane saw NaN/Inf" in one pass through LDS (one barrier pair instead of two).
+__device__ void block_max_any(float &v, int &flag, float *sh, int *shi) {
+  for (int o = 32; o > 0; o >>= 1) {
+    v = fmaxf(v, __shfl_xor(v, o));
+    flag |= __shfl_xor(flag, o);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sh[threadIdx.x >> 6] = v;
+    shi[threadIdx.x >> 6] = flag;
+  }
   __syncthreads();
-  float r = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  v = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  flag = shi[0] | shi[1] | shi[2] | shi[3];
   __syncthreads();
-  return r;
 }
+
+// Four block sums at once (the four digit rows of a token); sh4 holds 16 ints.
+__device__ void block_sum4(int (&v)[4], int *sh4) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+    for (int o = 32; o > 0; o >>= 1) v[d] += __shfl_xor(v[d], o);
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) sh4[(threadIdx.x >> 6) * 4 + d] = v[d];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int d = 0; d < 4; ++d) v[d] = sh4[d] + sh4[4 + d] + sh4[8 + d] + sh4[12 + d];
+  __syncthreads();
+}
+
 __device__ int block_sum(int v, int *sh) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
   if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
@@ -2078,8 +2101,9 @@ __device__ void row_absmax(const void *act, int dtype, size_t base, size_t k, bo
       nf |= !(a <= 3.402823466e38f);  // NaN or Inf
     }
   }
-  gamma = block_max(g, sh);
-  nonfinite = block_sum(nf, shi) != 0;
+  block_max_any(g, nf, sh, shi);
+  gamma = g;
+  nonfinite = nf != 0;
 }
 
 // A thread of the prep kernels builds whole 16-byte pieces of the operand layout. Piece q of K block
@@ -2139,8 +2163,9 @@ __device__ __forceinline__ void row_absmax_held(const void *act, int dtype, size
       }
     }
   }
-  gamma = block_max(g, sh);
-  nonfinite = block_sum(nf, shi) != 0;
+  block_max_any(g, nf, sh, shi);
+  gamma = g;
+  nonfinite = nf != 0;
 }
 
 // Per-token int8 absmax quant (crates/tritium-spec/src/lib.rs:351-378) straight into operand order.
@@ -2249,7 +2274,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
 __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                                int nprep) {
   __shared__ float shf[4];
-  __shared__ int shi[4];
+  __shared__ int shi[16];
   int rowi;
   const TkPrep &pp = find_prep(single, table, nprep, rowi);
   const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
@@ -2333,10 +2358,10 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
       emit(pc, v);
     }
   }
-#pragma unroll
-  for (int dg = 0; dg < 4; ++dg) {
-    int sm = block_sum(sums[dg], shi);
-    if (threadIdx.x == 0) pp.rowsum[tok * 4 + dg] = sm;
+  block_sum4(sums, shi);
+  if (threadIdx.x < 4) {
+    const int t = threadIdx.x;
+    pp.rowsum[tok * 4 + t] = t == 0 ? sums[0] : t == 1 ? sums[1] : t == 2 ? sums[2] : sums[3];
   }
   if (threadIdx.x == 0) {
     pp.exps[tok] = -shift;
