@@ -694,7 +694,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   pp.rs = (size_t)pl.pr.rs;
   pp.act_dtype = act_dtype;
   pp.m = (int)m;
-  HIPCHK(tk_launch_prep(ctx->stream, prep_kind, &pp, nullptr, 0, (unsigned)m));
+  HIPCHK(tk_launch_prep(ctx->stream, prep_kind, &pp, nullptr, 0, 0, (unsigned)m));
 
   TkProblem &pr = pl.pr;
   pr.ap = pp.ap;
@@ -858,7 +858,7 @@ static int run_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int
   pp.rs = R;
   pp.act_dtype = act_dtype;
   pp.m = (int)m;
-  HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_DIGITS, &pp, nullptr, 0, (unsigned)m));
+  HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_DIGITS, &pp, nullptr, 0, 0, (unsigned)m));
   pr.ap = pp.ap;
   pr.rowsum = pp.rowsum;
   pr.exps = pp.exps;
@@ -962,7 +962,7 @@ static int act_quant(tk_ctx *ctx, const void *act, int act_dtype, const tk_rmsno
     pp.norm_eps = norm->eps;
     pp.norm_w = norm->weight;
   }
-  HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_A8, &pp, nullptr, 0, (unsigned)m));
+  HIPCHK(tk_launch_prep(ctx->stream, TK_PREP_A8, &pp, nullptr, 0, 0, (unsigned)m));
   return TK_OK;
 }
 
@@ -1059,6 +1059,7 @@ struct tk_group {
   void *ws = nullptr;        // one allocation holding every member's operand rows and side arrays
   void *tables = nullptr;    // TkProblem[count], TkPrep[nprep], then int wg_prob[] (streaming form)
   int nprobs = 0, nprep = 0, prep_kind = 0;
+  int prep_uniform_m = 0;    // > 0: prep entry j starts at token j * prep_uniform_m
   unsigned prep_rows = 0;
   int variant = 1;
   size_t wg_prob_off = 0;
@@ -1337,6 +1338,9 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   g->wg_prob_off = wg_prob_off;
   g->nprobs = (int)count;
   g->nprep = (int)preps.size();
+  g->prep_uniform_m = preps.empty() ? 0 : preps[0].m;
+  for (size_t j = 0; j < preps.size(); ++j)
+    if (preps[j].m != preps[0].m || preps[j].row_begin != (int)j * preps[0].m) g->prep_uniform_m = 0;
   g->prep_kind = prep_kind;
   g->prep_rows = rows;
   g->cfg.planes = planes;
@@ -1365,7 +1369,7 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   HIPCHK(hipSetDevice(ctx->device));
   const TkProblem *probs = (const TkProblem *)g->tables;
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
-  if (do_prep) HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_rows));
+  if (do_prep) HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
   if (do_main && g->has_flow_part)
     HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),

@@ -98,7 +98,8 @@ hipError_t tk_launch_relayout_tq2(hipStream_t s, const uint8_t *raw, uint8_t *co
 hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb);
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
                                   int8_t *trits);
-hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep,
+// uniform_m > 0 says that entry j of the table starts at token j * uniform_m (all tensors equally long).
+hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
                           unsigned rows);
 hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
                             const TkLaunchCfg &cfg);

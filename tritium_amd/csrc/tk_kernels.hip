@@ -2119,8 +2119,16 @@ __device__ __forceinline__ size_t piece_offset(size_t kb, int q, size_t R, size_
   return (((kb * 4 + j) * 4 + g) * R + row) * 16;
 }
 
-__device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const TkPrep *table, int nprep, int &row) {
+// uniform_m > 0: every tensor of the table has that many tokens, so the entry follows from the
+// workgroup index without the chain of dependent loads the search costs.
+__device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const TkPrep *table, int nprep, int uniform_m,
+                                                   int &row) {
   if (!table) { row = blockIdx.x; return single; }
+  if (uniform_m > 0) {
+    const int t = (int)blockIdx.x / uniform_m;
+    row = (int)blockIdx.x - t * uniform_m;
+    return table[t];
+  }
   int lo = 0, hi = nprep - 1;
   while (lo < hi) {
     int mid = (lo + hi + 1) >> 1;
@@ -2170,11 +2178,11 @@ __device__ __forceinline__ void row_absmax_held(const void *act, int dtype, size
 
 // Per-token int8 absmax quant (crates/tritium-spec/src/lib.rs:351-378) straight into operand order.
 __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const TkPrep *__restrict__ table,
-                                                           int nprep) {
+                                                           int nprep, int uniform_m) {
   __shared__ float shf[4];
   __shared__ int shi[4];
   int rowi;
-  const TkPrep &pp = find_prep(single, table, nprep, rowi);
+  const TkPrep &pp = find_prep(single, table, nprep, uniform_m, rowi);
   const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = row * k;
   const void *act = pp.act;
@@ -2272,11 +2280,11 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
 // Scaling a float by a power of two is exact, so the rounding to an integer happens once, in
 // single precision.
 __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, const TkPrep *__restrict__ table,
-                                                               int nprep) {
+                                                               int nprep, int uniform_m) {
   __shared__ float shf[4];
   __shared__ int shi[16];
   int rowi;
-  const TkPrep &pp = find_prep(single, table, nprep, rowi);
+  const TkPrep &pp = find_prep(single, table, nprep, uniform_m, rowi);
   const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = tok * k;
   const void *act = pp.act;
@@ -2371,10 +2379,10 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
 
 // Already-quantized int8 rows -> operand order + row sums.
 __global__ __launch_bounds__(TK_WG) void tk_prep_i8_kernel(TkPrep single, const TkPrep *__restrict__ table,
-                                                           int nprep) {
+                                                           int nprep, int uniform_m) {
   __shared__ int shi[4];
   int rowi;
-  const TkPrep &pp = find_prep(single, table, nprep, rowi);
+  const TkPrep &pp = find_prep(single, table, nprep, uniform_m, rowi);
   const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const int8_t *q = (const int8_t *)pp.act;
   int8_t *ap = pp.ap;
@@ -2438,15 +2446,15 @@ hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n,
   return hipGetLastError();
 }
 
-hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep,
+hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
                           unsigned rows) {
   if (!rows) return hipSuccess;
   TkPrep dummy = {};
   const TkPrep &sg = single ? *single : dummy;
   switch (kind) {
-    case TK_PREP_A8: hipLaunchKernelGGL(tk_prep_a8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep); break;
-    case TK_PREP_DIGITS: hipLaunchKernelGGL(tk_prep_digits_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep); break;
-    case TK_PREP_I8: hipLaunchKernelGGL(tk_prep_i8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep); break;
+    case TK_PREP_A8: hipLaunchKernelGGL(tk_prep_a8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m); break;
+    case TK_PREP_DIGITS: hipLaunchKernelGGL(tk_prep_digits_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m); break;
+    case TK_PREP_I8: hipLaunchKernelGGL(tk_prep_i8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
