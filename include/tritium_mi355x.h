@@ -130,6 +130,27 @@ int tk_mpgemm_with_act_quant(tk_ctx *ctx, const float *act, size_t act_len,
                              const tk_weights *weights, const float *scales, size_t scales_len,
                              size_t m, size_t n, size_t k, int format, float *out, size_t out_len);
 
+/* ---- TernaryBackend::mpgemm_projected_vjp (crates/tritium-spec/src/lib.rs:93-117 the operands,
+ *      :217-232 the method; oracle: crates/tritium-cpu/src/lib.rs:347-395 ->
+ *      crates/tritium-cpu/src/kernel.rs:199-317; device precedent
+ *      crates/tritium-cuda/src/cuda/backend.rs:8683-8760). Host slices in and out, synchronous.
+ *        grad_act[m,k] = sum_n grad_output[m,n] * (trit[n,k] * scales[n])
+ *        grad_w[n,k]   = sum_m grad_output[m,n] * act[m,k]     (w.r.t. P[n,k] = scales[n]*trit[n,k])
+ *        grad_bias[n]  = sum_m grad_output[m,n]                (grad_bias == NULL: Option::None)
+ *      every sum in index order with unfused f32 operations, i.e. the bits of the CPU backend's
+ *      scalar path (the reference's own bar between backends is 1e-4 relative,
+ *      crates/tritium-cuda/src/cuda/tests.rs:733). All outputs are fully overwritten on success and
+ *      untouched on error. TQ2_0 and TQ1_0 buffers are both taken, as by the CPU backend.
+ * Errors, in the CPU backend's order: buffer n/k/format differ from the call's -> TK_ERR_INVALID_INPUT;
+ * a plane holding the reserved code -> TK_ERR_BACKEND ("unpack row R: decoded value 2 outside ternary
+ * range"); act, scales, grad_output, grad_act, grad_w, grad_bias length -> TK_ERR_SHAPE_MISMATCH.
+ * m == 0 or n == 0: outputs zero-filled; k == 0: grad_bias still summed. */
+int tk_mpgemm_projected_vjp(tk_ctx *ctx, const float *act, size_t act_len, const tk_weights *weights,
+                            const float *scales, size_t scales_len, const float *grad_output,
+                            size_t grad_output_len, size_t m, size_t n, size_t k, int format,
+                            float *grad_act, size_t grad_act_len, float *grad_w, size_t grad_w_len,
+                            float *grad_bias, size_t grad_bias_len);
+
 /* ---- device-resident extension, reached through TernaryBackend::as_concrete
  *      (crates/tritium-spec/src/lib.rs:320-332); precedent: the CUDA backend's device-resident
  *      decode (crates/tritium-cuda/src/cuda/mod.rs:1029-1064,2998-3041). All pointers below are
@@ -214,6 +235,15 @@ int tk_linear_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int 
 /* The host's order for every output: bit-identical to dequantize-then-fold. */
 int tk_linear_salt_seq(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
                        void *out, int out_dtype);
+
+/* mpgemm_projected_vjp on device-resident operands (same arithmetic and bits as
+ * tk_mpgemm_projected_vjp; precedent for device-resident gradients:
+ * crates/tritium-cuda/src/cuda/backend.rs:8755-8830, which stages exactly these buffers). scales [n],
+ * act [m,k], grad_output [m,n], grad_act [m,k], grad_w [n,k], grad_bias [n] or NULL, all f32 on
+ * ctx's device; enqueued on ctx's stream, not synchronised. */
+int tk_projected_vjp(tk_ctx *ctx, const tk_weights *weights, const float *scales, const float *act,
+                     const float *grad_output, size_t m, float *grad_act, float *grad_w,
+                     float *grad_bias);
 
 /* Reference-order float contraction: one thread per output, a single f32 accumulator walked in k
  * order (crates/tritium-core/src/reference.rs:25-54) — bit-identical to the CPU backend for any

@@ -495,6 +495,54 @@ int to_cpu_mpgemm_with_act_quant(const uint8_t *packed, size_t packed_len, int f
   return rc;
 }
 
+/* TernaryBackend::mpgemm_projected_vjp as the CPU backend runs it without SIMD
+ * (crates/tritium-cpu/src/lib.rs:347-395 -> crates/tritium-cpu/src/kernel.rs:82-189 and 199-317):
+ *   grad_act[m,k]  = sum over n, in order, of  upstream * (trit * scales[n])      (kernel.rs:150-163, 281-293)
+ *   grad_w[n,k]    = sum over m, in order, of  upstream * act[m,k]                (kernel.rs:165-177, 295-307)
+ *   grad_bias[n]   = sum over m, in order, of  upstream                           (kernel.rs:181-189)
+ * with upstream = grad_output[m,n], every product and sum rounded to f32 on its own. Length checks
+ * come in the reference's order and nothing is written when one fails; a TQ2_0 plane holding the
+ * reserved code is refused before any output is touched (lib.rs:365-370). grad_bias may be NULL. */
+int to_cpu_projected_vjp(const uint8_t *packed, size_t packed_len, int format, const float *act,
+                         size_t act_len, const float *scales, size_t scales_len,
+                         const float *grad_output, size_t grad_output_len, size_t m, size_t n,
+                         size_t k, float *grad_act, size_t grad_act_len, float *grad_w,
+                         size_t grad_w_len, float *grad_bias, size_t grad_bias_len) {
+  int8_t *trits = NULL;
+  int rc = unpack_weights(packed, packed_len, format, n, k, &trits);
+  if (rc) return rc;
+  rc = TO_OK;
+  if (act_len != m * k || scales_len != n || grad_output_len != m * n || grad_act_len != m * k ||
+      grad_w_len != n * k || (grad_bias && grad_bias_len != n))
+    rc = TO_ERR_SHAPE; /* kernel.rs:102-120 */
+  if (!rc) {
+    for (size_t i = 0; i < m * k; ++i) grad_act[i] = 0.0f; /* kernel.rs:122-123 */
+    for (size_t i = 0; i < n * k; ++i) grad_w[i] = 0.0f;
+    for (size_t mi = 0; mi < m; ++mi)
+      for (size_t ni = 0; ni < n; ++ni) {
+        const float upstream = grad_output[mi * n + ni];
+        for (size_t ki = 0; ki < k; ++ki) {
+          const float projected = (float)trits[ni * k + ki] * scales[ni];
+          grad_act[mi * k + ki] = grad_act[mi * k + ki] + upstream * projected;
+        }
+      }
+    for (size_t ni = 0; ni < n; ++ni)
+      for (size_t mi = 0; mi < m; ++mi) {
+        const float upstream = grad_output[mi * n + ni];
+        for (size_t ki = 0; ki < k; ++ki)
+          grad_w[ni * k + ki] = grad_w[ni * k + ki] + upstream * act[mi * k + ki];
+      }
+    if (grad_bias)
+      for (size_t ni = 0; ni < n; ++ni) {
+        float acc = 0.0f;
+        for (size_t mi = 0; mi < m; ++mi) acc = acc + grad_output[mi * n + ni];
+        grad_bias[ni] = acc;
+      }
+  }
+  free(trits);
+  return rc;
+}
+
 int to_int8_accumulators(const uint8_t *packed, size_t packed_len, int format, const int8_t *q,
                          size_t m, size_t n, size_t k, int32_t *acc) {
   int8_t *trits = NULL;

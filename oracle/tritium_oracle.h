@@ -125,6 +125,15 @@ int to_cpu_mpgemm_with_act_quant(const uint8_t *packed, size_t packed_len, int f
 
 /* Exact int32 accumulators Σ_k q[m,k]·trit[n,k] for int8 activations (the value the reference's
  * f32 fold holds before its two multiplies: crates/tritium-cpu/src/kernel.rs:588-599,824-828). */
+/* mpgemm_projected_vjp, scalar path of the CPU backend (crates/tritium-cpu/src/kernel.rs:82-189):
+ * pinned by the reference's known-answer case (crates/tritium-cpu/src/lib.rs:500-533) and against a
+ * float64 evaluation of the three sums. grad_bias may be NULL. */
+int to_cpu_projected_vjp(const uint8_t *packed, size_t packed_len, int format, const float *act,
+                         size_t act_len, const float *scales, size_t scales_len,
+                         const float *grad_output, size_t grad_output_len, size_t m, size_t n,
+                         size_t k, float *grad_act, size_t grad_act_len, float *grad_w,
+                         size_t grad_w_len, float *grad_bias, size_t grad_bias_len);
+
 int to_int8_accumulators(const uint8_t *packed, size_t packed_len, int format, const int8_t *q,
                          size_t m, size_t n, size_t k, int32_t *acc);
 

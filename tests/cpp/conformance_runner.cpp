@@ -42,7 +42,29 @@ int main(int argc, char **argv) {
   }
   CHECK(be->device_id() == "mi355x:0", "device_id %s", be->device_id().c_str());
   CHECK(be->capabilities().backend == "mi355x" && be->capabilities().supports_imma, "capabilities");
-  CHECK(be->mpgemm_projected_vjp().has_value(), "vjp must be refused");
+  {
+    // the reference's known-answer case of the packed VJP (crates/tritium-cpu/src/lib.rs:500-533)
+    const int8_t w[6] = {1, 0, -1, -1, 1, 1};
+    const size_t len = 2 * to_row_bytes(3, TO_FMT_TQ2_0);
+    std::vector<uint8_t> packed(len);
+    to_pack_matrix(w, 2, 3, TO_FMT_TQ2_0, packed.data(), len);
+    std::unique_ptr<DeviceBuffer> buf;
+    GemmShape shape{2, 2, 3};
+    Status e = be->upload_weights(packed.data(), len, shape, TernaryFormat::Tq2_0, &buf);
+    CHECK(!e, "vjp upload");
+    const float act[6] = {1.0f, 2.0f, 3.0f, -1.0f, 4.0f, 0.5f}, sc[2] = {2.0f, 0.5f}, gy[4] = {3.0f, -2.0f, 4.0f, 1.0f};
+    float ga[6], gw[6], gb[2];
+    MpGemmProjectedVjp p{act, 6, buf.get(), sc, 2, gy, 4, shape, TernaryFormat::Tq2_0, ga, 6, gw, 6, gb, 2};
+    e = be->mpgemm_projected_vjp(p);
+    CHECK(!e, "vjp: %s", e ? e->message.c_str() : "");
+    const float want_a[6] = {7.0f, -1.0f, -7.0f, 7.5f, 0.5f, -7.5f}, want_w[6] = {-1.0f, 22.0f, 11.0f, -3.0f, 0.0f, -5.5f},
+                want_b[2] = {7.0f, -1.0f};
+    CHECK(same_bits(ga, want_a, 6) && same_bits(gw, want_w, 6) && same_bits(gb, want_b, 2), "vjp known answer");
+    MpGemmProjectedVjp bad = p;
+    bad.grad_act_len = 0;
+    e = be->mpgemm_projected_vjp(bad);
+    CHECK(e && e->kind == BackendError::ShapeMismatch && e->expected == 6 && e->got == 0, "vjp shape error");
+  }
   CHECK(be->as_concrete() != nullptr, "as_concrete");
 
   to_vector_set *set = to_generate_vectors(0xC0FFEE, 64);

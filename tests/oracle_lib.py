@@ -82,6 +82,8 @@ class Oracle:
         pp = C.POINTER(C.c_void_p)
         L.to_cpu_mpgemm_planes.argtypes = [pp, C.POINTER(sz), C.c_int, pp, sz, f32p, sz, sz, sz, f32p]
         L.to_cpu_linear_a8_planes.argtypes = L.to_cpu_mpgemm_planes.argtypes
+        L.to_cpu_projected_vjp.argtypes = [u8p, sz, C.c_int, f32p, sz, f32p, sz, f32p, sz, sz, sz, sz, f32p, sz, f32p, sz,
+                                           f32p, sz]
         L.to_cpu_mpgemm_fast.argtypes = [u8p, sz, C.c_int, f32p, f32p, sz, sz, sz, f32p, C.c_int,
                                          C.POINTER(C.c_int), C.POINTER(C.c_int)]
         for name in ("to_pack_tq2_0_block", "to_pack_tq1_0_block"):
@@ -274,6 +276,22 @@ class Oracle:
 
     def cpu_linear_a8_planes(self, packed_list, fmt, scales_list, act, m, n, k):
         return self._planes(self.lib.to_cpu_linear_a8_planes, packed_list, fmt, scales_list, act, m, n, k)
+
+    def cpu_projected_vjp(self, packed, fmt, act, scales, grad_output, m, n, k, bias=True, lens=None):
+        """(rc, grad_act [m,k], grad_w [n,k], grad_bias [n] or None); outputs start as NaN so that an
+        early error return is seen to have written nothing. `lens` overrides the output lengths
+        (grad_act, grad_w, grad_bias) to provoke the shape errors."""
+        b = np.ascontiguousarray(packed, np.uint8)
+        a = np.ascontiguousarray(act, np.float32).reshape(-1)
+        s = np.ascontiguousarray(scales, np.float32).reshape(-1)
+        gy = np.ascontiguousarray(grad_output, np.float32).reshape(-1)
+        la, lw, lb = lens or (m * k, n * k, n)
+        ga, gw, gb = (np.full(max(x, 1), np.nan, np.float32) for x in (la, lw, lb))
+        rc = self.lib.to_cpu_projected_vjp(_p(b, u8p), b.size, fmt, _p(a, f32p), a.size, _p(s, f32p), s.size,
+                                           _p(gy, f32p), gy.size, m, n, k, _p(ga, f32p), la, _p(gw, f32p), lw,
+                                           _p(gb, f32p) if bias else None, lb if bias else 0)
+        return rc, ga[:la].reshape(m, k) if la == m * k else ga[:la], \
+            gw[:lw].reshape(n, k) if lw == n * k else gw[:lw], (gb[:lb] if bias else None)
 
     def cpu_mpgemm_fast(self, packed, fmt, act, scales, m, n, k, threads):
         b = np.ascontiguousarray(packed, np.uint8)

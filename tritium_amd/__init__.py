@@ -5,7 +5,7 @@ this package is the thin host mirror of the reference's adapter interface over i
 """
 from . import _lib
 from .backend import (BACKENDS, Backend, BackendEntry, BackendError, DeviceArray, DeviceBuffer, DeviceCaps,
-                      GemmShape, InvalidInput, Linear, Mi355xBackend, Mi355xBuffer, MpGemm, OutOfMemory,
+                      GemmShape, InvalidInput, Linear, Mi355xBackend, Mi355xBuffer, MpGemm, MpGemmProjectedVjp, OutOfMemory,
                       Registry, ShapeMismatch, TernaryFormat, UnsupportedFormat, convert_i2s_to_tq2_0, pack_rows,
                       packed_len, unpack_rows)
 from .linear import TernaryLinear

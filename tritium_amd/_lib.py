@@ -60,6 +60,8 @@ SIGNATURES = {
     "tk_weights_download_trits": (C.c_int, [vp, vp, vp, sz]),
     "tk_mpgemm": (C.c_int, [vp, vp, sz, vp, vp, sz, sz, sz, sz, C.c_int, vp, sz]),
     "tk_mpgemm_with_act_quant": (C.c_int, [vp, vp, sz, vp, vp, sz, sz, sz, sz, C.c_int, vp, sz]),
+    "tk_mpgemm_projected_vjp": (C.c_int, [vp, vp, sz, vp, vp, sz, vp, sz, sz, sz, sz, C.c_int, vp, sz, vp, sz, vp, sz]),
+    "tk_projected_vjp": (C.c_int, [vp, vp, vp, vp, vp, sz, vp, vp, vp]),
     "tk_act_quant_i8": (C.c_int, [vp, vp, C.c_int, sz, sz, vp, vp, vp]),
     "tk_linear_float": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_i2s_payload_len": (sz, [sz, sz]),

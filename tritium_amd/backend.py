@@ -123,6 +123,21 @@ class MpGemm:
     out: np.ndarray          # [M,N] f32, overwritten
 
 
+@dataclass
+class MpGemmProjectedVjp:
+    """Operands of the VJP of one packed ternary mpGEMM (crates/tritium-spec/src/lib.rs:93-117).
+    grad_projected_weight is the gradient with respect to P[n,k] = scales[n] * trit[n,k]."""
+    act: np.ndarray                    # [M,K] f32
+    weights: DeviceBuffer
+    scales: np.ndarray                 # [N] f32
+    grad_output: np.ndarray            # [M,N] f32
+    shape: GemmShape
+    format: TernaryFormat
+    grad_act: np.ndarray               # [M,K] f32, overwritten
+    grad_projected_weight: np.ndarray  # [N,K] f32, overwritten
+    grad_bias: Optional[np.ndarray] = None  # [N] f32, overwritten when given
+
+
 DTYPES = {"f32": L.TK_F32, "bf16": L.TK_BF16, "i8": L.TK_I8, "i32": L.TK_I32}
 _NP = {L.TK_F32: np.float32, L.TK_BF16: np.uint16, L.TK_I8: np.int8, L.TK_I32: np.int32}
 
@@ -339,9 +354,30 @@ class Mi355xBackend:
     def mpgemm_with_act_quant(self, p):
         self._host_call(self._lib.tk_mpgemm_with_act_quant, p)
 
-    def mpgemm_projected_vjp(self, p=None):
-        # the inference-only default (crates/tritium-spec/src/lib.rs:221-226)
-        raise Backend(f"backend `{self.device_id()}` does not implement packed mpGEMM VJP")
+    def mpgemm_projected_vjp(self, p):
+        """grad_act, grad_projected_weight and the optional grad_bias of one packed mpGEMM, with the
+        bits of the CPU backend's scalar path (crates/tritium-cpu/src/kernel.rs:281-317)."""
+        if not isinstance(p.weights, Mi355xBuffer) or p.weights._backend is not self or not p.weights._h:
+            raise InvalidInput("buffer is not a Mi355xBuffer of this backend")
+        outs = [p.grad_act, p.grad_projected_weight] + ([p.grad_bias] if p.grad_bias is not None else [])
+        for o in outs:
+            if not (isinstance(o, np.ndarray) and o.dtype == np.float32 and o.flags.c_contiguous):
+                raise InvalidInput("gradient outputs must be C-contiguous float32 numpy arrays")
+        act = _flat(p.act, np.float32, "act")
+        scales = _flat(p.scales, np.float32, "scales")
+        up = _flat(p.grad_output, np.float32, "grad_output")
+        s = p.shape
+        gb = p.grad_bias
+        _check(self._lib.tk_mpgemm_projected_vjp(
+            self._ctx, act.ctypes.data, act.size, p.weights._h, scales.ctypes.data, scales.size, up.ctypes.data,
+            up.size, s.m, s.n, s.k, int(p.format), p.grad_act.ctypes.data, p.grad_act.size,
+            p.grad_projected_weight.ctypes.data, p.grad_projected_weight.size,
+            gb.ctypes.data if gb is not None else None, gb.size if gb is not None else 0))
+
+    def projected_vjp(self, weights, scales, act, grad_output, m, grad_act, grad_w, grad_bias=None):
+        """The same gradients on device-resident f32 arrays; enqueued, not synchronised."""
+        _check(self._lib.tk_projected_vjp(self._ctx, weights._h, scales.ptr, act.ptr, grad_output.ptr, m, grad_act.ptr,
+                                          grad_w.ptr, grad_bias.ptr if grad_bias is not None else None))
 
     def as_concrete(self):
         return self

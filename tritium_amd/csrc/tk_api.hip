@@ -1051,6 +1051,94 @@ extern "C" int tk_mpgemm_with_act_quant(tk_ctx *ctx, const float *act, size_t ac
 }
 
 // ------------------------------------------------------------------------------------------
+// mpgemm_projected_vjp (crates/tritium-spec/src/lib.rs:217-232)
+// ------------------------------------------------------------------------------------------
+
+static int vjp_weights_ok(tk_ctx *ctx, const tk_weights *weights) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  if (!weights) return tk_fail(TK_ERR_INVALID_INPUT, "buffer is not a tritium-mi355x buffer");
+  if (weights->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "buffer belongs to another context");
+  return TK_OK;
+}
+
+// Zero fill and launches shared by both forms; device pointers, ctx->mu held, device current.
+static int vjp_enqueue(tk_ctx *ctx, const tk_weights *w, const float *scales, const float *act, const float *grad_output,
+                       size_t m, float *grad_act, float *grad_w, float *grad_bias) {
+  const size_t n = w->n, k = w->k;
+  if (m > 0x7fffffffu || n > 0x7fffffffu || k > 0x7fffffffu || (m + 15) / 16 > 65535 || (n + 63) / 64 > 65535)
+    return tk_fail(TK_ERR_INVALID_INPUT, "projected VJP launch bounds exceeded: M=%zu N=%zu K=%zu", m, n, k);
+  // grad_act.fill(0.0); grad_projected_weight.fill(0.0) (crates/tritium-cpu/src/kernel.rs:122-123):
+  // the kernels overwrite every element when m, n and k are all positive
+  if (!(m && n && k)) {
+    if (grad_act && m * k) HIPCHK(hipMemsetAsync(grad_act, 0, m * k * 4, ctx->stream));
+    if (grad_w && n * k) HIPCHK(hipMemsetAsync(grad_w, 0, n * k * 4, ctx->stream));
+  }
+  HIPCHK(tk_launch_projected_vjp(ctx->stream, w->codes, w->nb, n, k, m, scales, act, grad_output, grad_act, grad_w,
+                                 grad_bias));
+  return TK_OK;
+}
+
+extern "C" int tk_projected_vjp(tk_ctx *ctx, const tk_weights *weights, const float *scales, const float *act,
+                                const float *grad_output, size_t m, float *grad_act, float *grad_w,
+                                float *grad_bias) {
+  TKCHK(vjp_weights_ok(ctx, weights));
+  if (weights->invalid_row >= 0)
+    return tk_fail(TK_ERR_BACKEND, "unpack row %ld: decoded value 2 outside ternary range", weights->invalid_row);
+  const size_t n = weights->n, k = weights->k;
+  if ((m * n && (!grad_output || !scales)) || (m * k && !act) || (m * k && !grad_act) || (n * k && !grad_w))
+    return tk_fail(TK_ERR_INVALID_INPUT, "null operand pointer");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return vjp_enqueue(ctx, weights, scales, act, grad_output, m, grad_act, grad_w, grad_bias);
+}
+
+extern "C" int tk_mpgemm_projected_vjp(tk_ctx *ctx, const float *act, size_t act_len, const tk_weights *weights,
+                                       const float *scales, size_t scales_len, const float *grad_output,
+                                       size_t grad_output_len, size_t m, size_t n, size_t k, int format,
+                                       float *grad_act, size_t grad_act_len, float *grad_w, size_t grad_w_len,
+                                       float *grad_bias, size_t grad_bias_len) {
+  TKCHK(vjp_weights_ok(ctx, weights));
+  // CpuBuffer::validate_identity, then the reserved-code refusal, before any length is looked at
+  // (crates/tritium-cpu/src/lib.rs:359-370)
+  if (!fmt_block_bytes(format)) return tk_fail(TK_ERR_UNSUPPORTED_FORMAT, "unsupported ternary format: %d", format);
+  if (weights->n != n || weights->k != k || weights->format != format)
+    return tk_fail(TK_ERR_INVALID_INPUT, "buffer identity N=%zu K=%zu format=%d does not match N=%zu K=%zu format=%d",
+                   weights->n, weights->k, weights->format, n, k, format);
+  if (weights->invalid_row >= 0)
+    return tk_fail(TK_ERR_BACKEND, "unpack row %ld: decoded value 2 outside ternary range", weights->invalid_row);
+  size_t mk, nk, mn;  // crates/tritium-cpu/src/kernel.rs:93-101
+  if (__builtin_mul_overflow(m, k, &mk)) return tk_fail(TK_ERR_INVALID_INPUT, "M*K element count overflows");
+  if (__builtin_mul_overflow(n, k, &nk)) return tk_fail(TK_ERR_INVALID_INPUT, "N*K element count overflows");
+  if (__builtin_mul_overflow(m, n, &mn)) return tk_fail(TK_ERR_INVALID_INPUT, "M*N element count overflows");
+  if (act_len != mk) return tk_fail_mismatch(mk, act_len);  // the reference's order (kernel.rs:102-120)
+  if (scales_len != n) return tk_fail_mismatch(n, scales_len);
+  if (grad_output_len != mn) return tk_fail_mismatch(mn, grad_output_len);
+  if (grad_act_len != mk) return tk_fail_mismatch(mk, grad_act_len);
+  if (grad_w_len != nk) return tk_fail_mismatch(nk, grad_w_len);
+  if (grad_bias && grad_bias_len != n) return tk_fail_mismatch(n, grad_bias_len);
+  if ((mk && (!act || !grad_act)) || (nk && !grad_w) || (n && !scales) || (mn && !grad_output))
+    return tk_fail(TK_ERR_INVALID_INPUT, "null operand pointer");
+
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  auto al = [](size_t x) { return (x + 63) & ~(size_t)63; };  // in floats
+  const size_t in_floats = al(mk) + al(mn) + al(n), out_floats = al(mk) + al(nk) + al(n);
+  TKCHK(ensure(ctx, ctx->h_act, in_floats * 4));
+  TKCHK(ensure(ctx, ctx->h_out, out_floats * 4));
+  float *d_act = (float *)ctx->h_act.p, *d_up = d_act + al(mk), *d_sc = d_up + al(mn);
+  float *d_ga = (float *)ctx->h_out.p, *d_gw = d_ga + al(mk), *d_gb = d_gw + al(nk);
+  if (mk) HIPCHK(hipMemcpyAsync(d_act, act, mk * 4, hipMemcpyHostToDevice, ctx->stream));
+  if (mn) HIPCHK(hipMemcpyAsync(d_up, grad_output, mn * 4, hipMemcpyHostToDevice, ctx->stream));
+  if (n) HIPCHK(hipMemcpyAsync(d_sc, scales, n * 4, hipMemcpyHostToDevice, ctx->stream));
+  TKCHK(vjp_enqueue(ctx, weights, d_sc, d_act, d_up, m, d_ga, d_gw, grad_bias ? d_gb : nullptr));
+  if (mk) HIPCHK(hipMemcpyAsync(grad_act, d_ga, mk * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (nk) HIPCHK(hipMemcpyAsync(grad_w, d_gw, nk * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (grad_bias && n) HIPCHK(hipMemcpyAsync(grad_bias, d_gb, n * 4, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // grouped launches
 // ------------------------------------------------------------------------------------------
 

@@ -121,6 +121,10 @@ hipError_t tk_launch_salt_seq(hipStream_t s, const TkProblem *single);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);
+// The three gradients of one packed mpGEMM (tk_vjp.hip); a null output is skipped.
+hipError_t tk_launch_projected_vjp(hipStream_t s, const uint8_t *codes, size_t nb, size_t n, size_t k, size_t m,
+                                   const float *scales, const float *act, const float *grad_output, float *grad_act,
+                                   float *grad_w, float *grad_bias);
 hipError_t tk_launch_copy(hipStream_t s, void *dst, const void *src, size_t bytes);
 #ifdef __cplusplus
 }

@@ -77,6 +77,25 @@ struct MpGemm {
   size_t out_len;
 };
 
+// Operands of the VJP of one packed mpGEMM (crates/tritium-spec/src/lib.rs:93-117); grad_bias may be null.
+struct MpGemmProjectedVjp {
+  const float *act;
+  size_t act_len;
+  const DeviceBuffer *weights;
+  const float *scales;
+  size_t scales_len;
+  const float *grad_output;
+  size_t grad_output_len;
+  GemmShape shape;
+  TernaryFormat format;
+  float *grad_act;
+  size_t grad_act_len;
+  float *grad_projected_weight;
+  size_t grad_projected_weight_len;
+  float *grad_bias;
+  size_t grad_bias_len;
+};
+
 // Per-token int8 absmax quant of the trait's default fused path (crates/tritium-spec/src/lib.rs:351-378):
 // one divide 127/gamma, one multiply, ties to even, clamp [-128,127]; a zero row gives zeros and scale 0.
 inline void quantize_act_int8(const float *act, size_t m, size_t k, float *q, float *scale) {
@@ -112,7 +131,7 @@ class TernaryBackend {
                                 std::unique_ptr<DeviceBuffer> *out) = 0;
   virtual Status mpgemm(const MpGemm &p) = 0;
   // inference-only default (crates/tritium-spec/src/lib.rs:221-226)
-  virtual Status mpgemm_projected_vjp() {
+  virtual Status mpgemm_projected_vjp(const MpGemmProjectedVjp &) {
     return BackendError{BackendError::Backend, 0, 0, "backend `" + device_id() + "` does not implement packed mpGEMM VJP"};
   }
   // default: host quant -> mpgemm -> fold (crates/tritium-spec/src/lib.rs:266-318)
@@ -178,6 +197,16 @@ class Mi355xBackend : public TernaryBackend {
   }
   Status mpgemm(const MpGemm &p) override { return call(tk_mpgemm, p); }
   Status mpgemm_with_act_quant(const MpGemm &p) override { return call(tk_mpgemm_with_act_quant, p); }
+  Status mpgemm_projected_vjp(const MpGemmProjectedVjp &p) override {
+    auto *buf = dynamic_cast<const Mi355xBuffer *>(p.weights);
+    if (!buf) return BackendError{BackendError::InvalidInput, 0, 0, "buffer is not a Mi355xBuffer"};
+    if (int rc = tk_mpgemm_projected_vjp(ctx_, p.act, p.act_len, buf->handle(), p.scales, p.scales_len, p.grad_output,
+                                         p.grad_output_len, p.shape.m, p.shape.n, p.shape.k, (int)p.format, p.grad_act,
+                                         p.grad_act_len, p.grad_projected_weight, p.grad_projected_weight_len,
+                                         p.grad_bias, p.grad_bias_len))
+      return BackendError::from_status(rc);
+    return std::nullopt;
+  }
   void *as_concrete() override { return this; }
   tk_ctx *ctx() const { return ctx_; }  // the device-resident extension is the C ABI itself
 
