@@ -35,6 +35,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 # profiles/decode_flow_c2_sweep_traffic.txt
 DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_143_859_917
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+FP32_PEAK_TFLOPS = 157.3  # MI355X fp32, published
 
 K2, N2, PLANES2 = 2048, 8192, 2
 SWEEP = (1, 2, 4, 8, 16)
@@ -317,6 +318,32 @@ def bench_salt(T, be, rng, iters=30):
     return res
 
 
+def bench_vjp(T, be, rng, iters=5):
+    """mpgemm_projected_vjp on the configs[2] projection (M=2048 tokens, K=2560, N=6912, one plane),
+    device-resident f32 operands. Each gradient is timed on its own; flops = one multiply and one add
+    per term (kept unfused for the CPU backend's rounding), priced against the published fp32 vector
+    rate, which counts a fused multiply-add per lane and clock."""
+    m, k, n = 2048, 2560, 6912
+    buf = be.upload_weights(T.pack_rows(ternary(rng, n, k, 0.4), n, k), T.GemmShape(0, n, k), T.TernaryFormat.Tq2_0)
+    sc = be.to_device(rng.uniform(0.01, 0.1, n).astype(np.float32), "f32")
+    act = be.to_device(rng.standard_normal((m, k)).astype(np.float32), "f32")
+    gy = be.to_device(rng.standard_normal((m, n)).astype(np.float32), "f32")
+    ga, gw, gb = be.empty(m * k, "f32"), be.empty(n * k, "f32"), be.empty(n, "f32")
+    res = {"workload": f"projected VJP M={m} K={k} N={n}, 1 plane, f32 operands resident on the device"}
+    flops = 2.0 * m * n * k
+    for name, outs in (("grad_act", (ga, None, None)), ("grad_projected_weight", (None, gw, None)),
+                       ("grad_bias", (None, None, gb)), ("all_three", (ga, gw, gb))):
+        ms = time_calls(be, lambda i: be.projected_vjp(buf, sc, act, gy, m, *outs), iters)
+        res[name] = {"ms_per_call": round(ms, 4)}
+        if name != "grad_bias":
+            f = flops * (2 if name == "all_three" else 1)
+            res[name].update({"TFLOP/s": round(f / ms / 1e9, 2), "frac_of_fp32_peak": round(f / ms / 1e9 / FP32_PEAK_TFLOPS, 4)})
+    for a in (sc, act, gy, ga, gw, gb):
+        a.free()
+    buf.free()
+    return res
+
+
 def bench_stack(T, be, rng, iters=100):
     """configs[3]: the 7 ternary projections of 30 decoder layers (hidden 2560, FFN 6912, 20 query
     heads and 5 KV heads of 128), W1.58A8, one launch for the whole stack with given inputs.
@@ -409,7 +436,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,salt",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,salt,vjp",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -464,7 +491,8 @@ def main():
                 "prefill": ("prefill_gemm", lambda: bench_prefill(T, be, rng, 2048, 2560, 6912)),
                 "stack": ("projection_stack", lambda: bench_stack(T, be, rng)),
                 "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng)),
-                "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng))}
+                "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng)),
+                "vjp": ("projected_vjp", lambda: bench_vjp(T, be, rng))}
         out["extra"] = {}
         for leg in [x for x in args.extra_legs.split(",") if x]:
             if leg not in legs:

@@ -239,8 +239,9 @@ int tk_linear_salt_seq(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, 
 /* mpgemm_projected_vjp on device-resident operands (same arithmetic and bits as
  * tk_mpgemm_projected_vjp; precedent for device-resident gradients:
  * crates/tritium-cuda/src/cuda/backend.rs:8755-8830, which stages exactly these buffers). scales [n],
- * act [m,k], grad_output [m,n], grad_act [m,k], grad_w [n,k], grad_bias [n] or NULL, all f32 on
- * ctx's device; enqueued on ctx's stream, not synchronised. */
+ * act [m,k], grad_output [m,n], grad_act [m,k], grad_w [n,k], grad_bias [n], all f32 on ctx's
+ * device; any of the three outputs may be NULL and is then skipped (act is only read for grad_w).
+ * Enqueued on ctx's stream, not synchronised. */
 int tk_projected_vjp(tk_ctx *ctx, const tk_weights *weights, const float *scales, const float *act,
                      const float *grad_output, size_t m, float *grad_act, float *grad_w,
                      float *grad_bias);

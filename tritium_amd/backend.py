@@ -375,9 +375,11 @@ class Mi355xBackend:
             gb.ctypes.data if gb is not None else None, gb.size if gb is not None else 0))
 
     def projected_vjp(self, weights, scales, act, grad_output, m, grad_act, grad_w, grad_bias=None):
-        """The same gradients on device-resident f32 arrays; enqueued, not synchronised."""
-        _check(self._lib.tk_projected_vjp(self._ctx, weights._h, scales.ptr, act.ptr, grad_output.ptr, m, grad_act.ptr,
-                                          grad_w.ptr, grad_bias.ptr if grad_bias is not None else None))
+        """The same gradients on device-resident f32 arrays; enqueued, not synchronised. An output
+        given as None is skipped."""
+        ptr = lambda a: a.ptr if a is not None else None  # noqa: E731
+        _check(self._lib.tk_projected_vjp(self._ctx, weights._h, scales.ptr, ptr(act), grad_output.ptr, m, ptr(grad_act),
+                                          ptr(grad_w), ptr(grad_bias)))
 
     def as_concrete(self):
         return self

@@ -1085,7 +1085,7 @@ extern "C" int tk_projected_vjp(tk_ctx *ctx, const tk_weights *weights, const fl
   if (weights->invalid_row >= 0)
     return tk_fail(TK_ERR_BACKEND, "unpack row %ld: decoded value 2 outside ternary range", weights->invalid_row);
   const size_t n = weights->n, k = weights->k;
-  if ((m * n && (!grad_output || !scales)) || (m * k && !act) || (m * k && !grad_act) || (n * k && !grad_w))
+  if ((m * n && (!grad_output || !scales)) || (m * k && grad_w && !act))
     return tk_fail(TK_ERR_INVALID_INPUT, "null operand pointer");
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
