@@ -91,6 +91,77 @@ size_t tk_i2s_payload_len(size_t n, size_t k); /* n*k/4 + 4; 0 when n*k is not a
 int tk_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k,
                             uint8_t *out, size_t out_len, float *scale);
 
+/* ---- GGUF container (v2/v3): read_gguf and its accessors (crates/tritium-format/src/gguf.rs:
+ *      183-292, 360-400, 460-664). Parses header, metadata table and tensor table of a file held in
+ *      memory; payloads stay in the caller's buffer, which is not retained. Total: no input reads
+ *      out of bounds. A failed parse returns TK_ERR_INVALID_INPUT and reports the GgufError variant
+ *      (and the value UnsupportedVersion / InvalidBoolean / UnknownValueType carry). ---- */
+typedef struct tk_gguf tk_gguf;
+typedef enum tk_gguf_error { /* GgufError (crates/tritium-format/src/gguf.rs:63-96), in its order */
+  TK_GGUF_OK = 0,
+  TK_GGUF_BAD_MAGIC = 1,
+  TK_GGUF_UNSUPPORTED_VERSION = 2,
+  TK_GGUF_TRUNCATED = 3,
+  TK_GGUF_STRING_TOO_LONG = 4,
+  TK_GGUF_DIMS_OVERFLOW = 5,
+  TK_GGUF_INVALID_TENSOR_SHAPE = 6,
+  TK_GGUF_INVALID_ALIGNMENT = 7,
+  TK_GGUF_INVALID_BOOLEAN = 8,
+  TK_GGUF_OFFSET_OUT_OF_BOUNDS = 9,
+  TK_GGUF_UNKNOWN_VALUE_TYPE = 10,
+  TK_GGUF_INVALID_UTF8 = 11
+} tk_gguf_error;
+/* TensorInfo (gguf.rs:360-374). dims are fastest-varying first; offset is relative to
+ * tk_gguf_tensor_data_offset; n_bytes is 0 for a type the reader does not size (I2_S among them).
+ * name points into the tk_gguf and lives as long as it. */
+typedef struct tk_gguf_tensor {
+  const char *name;
+  uint32_t n_dims;
+  uint64_t dims[8];
+  uint32_t ggml_type;
+  uint64_t offset;
+  uint64_t n_bytes;
+} tk_gguf_tensor;
+int tk_gguf_open(const uint8_t *buf, size_t len, tk_gguf **out, int *error_kind, uint64_t *error_detail);
+void tk_gguf_close(tk_gguf *g);
+uint32_t tk_gguf_version(const tk_gguf *g);
+uint64_t tk_gguf_alignment(const tk_gguf *g); /* general.alignment, 32 when absent */
+uint64_t tk_gguf_tensor_data_offset(const tk_gguf *g);
+size_t tk_gguf_tensor_count(const tk_gguf *g);
+size_t tk_gguf_metadata_count(const tk_gguf *g);
+/* The getters below answer like Option: 1 = Some (and *out written), 0 = None. */
+int tk_gguf_tensor_at(const tk_gguf *g, size_t index, tk_gguf_tensor *out);
+int tk_gguf_tensor_find(const tk_gguf *g, const char *name, tk_gguf_tensor *out); /* GgufFile::tensor: first match */
+/* GgufFile::get_metadata(key) followed by GgufValue::as_* with the reference's coercions. index < 0
+ * addresses the key's value, index >= 0 element `index` of its array value. value_type is the GGUF
+ * metadata type id (0..12; 9 = array, for which child_type and array_len are filled). */
+int tk_gguf_meta_type(const tk_gguf *g, const char *key, long long index, uint32_t *value_type,
+                      uint32_t *child_type, uint64_t *array_len);
+int tk_gguf_meta_u64(const tk_gguf *g, const char *key, long long index, uint64_t *out);
+int tk_gguf_meta_i64(const tk_gguf *g, const char *key, long long index, int64_t *out);
+int tk_gguf_meta_f64(const tk_gguf *g, const char *key, long long index, double *out);
+int tk_gguf_meta_f32(const tk_gguf *g, const char *key, long long index, float *out);
+int tk_gguf_meta_bool(const tk_gguf *g, const char *key, long long index, int *out);
+int tk_gguf_meta_str(const tk_gguf *g, const char *key, long long index, const char **out, size_t *len);
+/* TensorInfo::element_count (gguf.rs:392-398); overflow -> TK_ERR_INVALID_INPUT */
+int tk_gguf_element_count(const tk_gguf_tensor *t, uint64_t *out);
+/* Where a tensor's payload lies in the file: the model loader's payload()
+ * (crates/tritium-nn/src/model/weights.rs:146-166), which sizes I2_S as elements/4 + 32. */
+int tk_gguf_tensor_payload(const tk_gguf *g, size_t file_len, const tk_gguf_tensor *t,
+                           uint64_t *abs_offset, uint64_t *len);
+/* ---- ternary tensor -> packed rows + one scale per output row: load_ternary
+ *      (crates/tritium-nn/src/model/weights.rs:177-333). dims must be [k, n]; type I2_S (36), TQ1_0
+ *      (34) or TQ2_0 (35), anything else -> TK_ERR_UNSUPPORTED_FORMAT. I2_S comes out as TQ2_0 rows
+ *      with the tensor's f32 scale on every row. TQ rows are copied in their own format; a block
+ *      whose f16 scale is 0 gets zero trits; block scales must agree within a row (else
+ *      TK_ERR_BACKEND); rows that differ keep their own scales, all-zero rows then take the first
+ *      nonzero one; with one scale for the whole tensor the f32 metadata value
+ *      "tritium.i2s_scale.<name>" replaces it when present (it must round to the same f16).
+ *      packed_len = tk_packed_len(n, k, format) and row_scales_len = n from tk_gguf_ternary_shape. */
+int tk_gguf_ternary_shape(const tk_gguf *g, const char *name, size_t *n, size_t *k, int *format);
+int tk_gguf_load_ternary(const tk_gguf *g, const uint8_t *file, size_t file_len, const char *name,
+                         uint8_t *packed, size_t packed_len, float *row_scales, size_t row_scales_len);
+
 /* ---- TernaryBackend::upload_weights (crates/tritium-spec/src/lib.rs:188-200;
  *      crates/tritium-cpu/src/lib.rs:262-300; crates/tritium-rocm/src/rocm.rs:446-475).
  * Copies; the returned handle owns device memory until tk_free_weights. `packed` is the byte
@@ -104,6 +175,10 @@ int tk_upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len, siz
  * of a BitNet I2_S checkpoint calls per weight tensor. */
 int tk_upload_weights_i2s(tk_ctx *ctx, const uint8_t *payload, size_t payload_len, size_t n, size_t k,
                           tk_weights **out, float *scale);
+/* tk_gguf_load_ternary followed by tk_upload_weights: one weight tensor of a GGUF checkpoint onto
+ * the device; row_scales [n] is what the caller passes as the per-channel scales of mpgemm. */
+int tk_upload_weights_gguf(tk_ctx *ctx, const tk_gguf *g, const uint8_t *file, size_t file_len,
+                           const char *name, tk_weights **out, float *row_scales, size_t row_scales_len);
 void tk_free_weights(tk_weights *w);
 size_t tk_weights_len_bytes(const tk_weights *w); /* DeviceBuffer::len_bytes: the uploaded length */
 size_t tk_weights_n(const tk_weights *w);

@@ -8,6 +8,7 @@ from .backend import (BACKENDS, Backend, BackendEntry, BackendError, DeviceArray
                       GemmShape, InvalidInput, Linear, Mi355xBackend, Mi355xBuffer, MpGemm, MpGemmProjectedVjp, OutOfMemory,
                       Registry, ShapeMismatch, TernaryFormat, UnsupportedFormat, convert_i2s_to_tq2_0, pack_rows,
                       packed_len, unpack_rows)
+from .gguf import GgufError, GgufErrorKind, GgufFile, TensorInfo, read_gguf
 from .linear import TernaryLinear
 
 __all__ = [n for n in dir() if not n.startswith("_")]

@@ -35,6 +35,11 @@ class SaltDesc(C.Structure):
     _fields_ = [("planes", vp * TK_MAX_PLANES), ("n_planes", C.c_int)]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 8), ("ggml_type", C.c_uint32),
+                ("offset", C.c_uint64), ("n_bytes", C.c_uint64)]
+
+
 class RmsNorm(C.Structure):
     _fields_ = [("weight", vp), ("eps", C.c_float), ("zero_centered", C.c_int)]
 
@@ -67,6 +72,28 @@ SIGNATURES = {
     "tk_i2s_payload_len": (sz, [sz, sz]),
     "tk_convert_i2s_to_tq2_0": (C.c_int, [vp, sz, sz, sz, vp, sz, C.POINTER(C.c_float)]),
     "tk_upload_weights_i2s": (C.c_int, [vp, vp, sz, sz, sz, C.POINTER(vp), C.POINTER(C.c_float)]),
+    "tk_gguf_open": (C.c_int, [vp, sz, C.POINTER(vp), C.POINTER(C.c_int), C.POINTER(C.c_uint64)]),
+    "tk_gguf_close": (None, [vp]),
+    "tk_gguf_version": (C.c_uint32, [vp]),
+    "tk_gguf_alignment": (C.c_uint64, [vp]),
+    "tk_gguf_tensor_data_offset": (C.c_uint64, [vp]),
+    "tk_gguf_tensor_count": (sz, [vp]),
+    "tk_gguf_metadata_count": (sz, [vp]),
+    "tk_gguf_tensor_at": (C.c_int, [vp, sz, C.POINTER(GgufTensor)]),
+    "tk_gguf_tensor_find": (C.c_int, [vp, C.c_char_p, C.POINTER(GgufTensor)]),
+    "tk_gguf_meta_type": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32),
+                                    C.POINTER(C.c_uint64)]),
+    "tk_gguf_meta_u64": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_uint64)]),
+    "tk_gguf_meta_i64": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_int64)]),
+    "tk_gguf_meta_f64": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_double)]),
+    "tk_gguf_meta_f32": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_float)]),
+    "tk_gguf_meta_bool": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_int)]),
+    "tk_gguf_meta_str": (C.c_int, [vp, C.c_char_p, C.c_longlong, C.POINTER(C.c_char_p), C.POINTER(sz)]),
+    "tk_gguf_element_count": (C.c_int, [C.POINTER(GgufTensor), C.POINTER(C.c_uint64)]),
+    "tk_gguf_tensor_payload": (C.c_int, [vp, sz, C.POINTER(GgufTensor), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "tk_gguf_ternary_shape": (C.c_int, [vp, C.c_char_p, C.POINTER(sz), C.POINTER(sz), C.POINTER(C.c_int)]),
+    "tk_gguf_load_ternary": (C.c_int, [vp, vp, sz, C.c_char_p, vp, sz, vp, sz]),
+    "tk_upload_weights_gguf": (C.c_int, [vp, vp, vp, sz, C.c_char_p, C.POINTER(vp), vp, sz]),
     "tk_upload_weights_scaled": (C.c_int, [vp, vp, sz, sz, sz, C.POINTER(vp)]),
     "tk_linear_salt": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_salt_seq": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),

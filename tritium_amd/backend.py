@@ -320,6 +320,16 @@ class Mi355xBackend:
                                                C.byref(sc)))
         return Mi355xBuffer(self, h), np.float32(sc.value)
 
+    def upload_weights_gguf(self, gguf, buf, name):
+        """One ternary weight tensor of a GGUF file onto the device -> (device buffer, row scales [n] f32):
+        load_ternary of the model loader (crates/tritium-nn/src/model/weights.rs:177-333)."""
+        b = np.ascontiguousarray(buf, dtype=np.uint8).reshape(-1)
+        n, _, _ = gguf.ternary_shape(name)
+        h, scales = C.c_void_p(), np.zeros(n, np.float32)
+        _check(self._lib.tk_upload_weights_gguf(self._ctx, gguf._h, b.ctypes.data, b.size, name.encode(), C.byref(h),
+                                                scales.ctypes.data, n))
+        return Mi355xBuffer(self, h), scales
+
     def upload_weights_scaled(self, packed, shape):
         """TQ2_0 rows whose f16 block scales are kept on the device (block-scale planes)."""
         b = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)

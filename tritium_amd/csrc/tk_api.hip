@@ -394,6 +394,24 @@ extern "C" int tk_upload_weights_i2s(tk_ctx *ctx, const uint8_t *payload, size_t
   return tk_upload_weights(ctx, packed.data(), len, n, k, TK_FORMAT_TQ2_0, out);
 }
 
+extern "C" int tk_upload_weights_gguf(tk_ctx *ctx, const tk_gguf *g, const uint8_t *file, size_t file_len,
+                                      const char *name, tk_weights **out, float *row_scales, size_t row_scales_len) {
+  if (!ctx || !out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_weights_gguf: null pointer");
+  *out = nullptr;
+  size_t n, k;
+  int format;
+  TKCHK(tk_gguf_ternary_shape(g, name, &n, &k, &format));
+  const size_t len = tk_packed_len(n, k, format);
+  std::vector<uint8_t> packed;
+  try {
+    packed.resize(len);
+  } catch (const std::bad_alloc &) {
+    return tk_fail(TK_ERR_BACKEND, "tk_upload_weights_gguf: host allocation of %zu bytes failed", len);
+  }
+  TKCHK(tk_gguf_load_ternary(g, file, file_len, name, packed.data(), len, row_scales, row_scales_len));
+  return tk_upload_weights(ctx, packed.data(), len, n, k, format, out);
+}
+
 extern "C" void tk_free_weights(tk_weights *w) {
   if (!w) return;
   std::lock_guard<std::mutex> lk(w->ctx->mu);
