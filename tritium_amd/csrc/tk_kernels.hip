@@ -2123,7 +2123,19 @@ __device__ __forceinline__ size_t piece_offset(size_t kb, int q, size_t R, size_
 // workgroup index without the chain of dependent loads the search costs.
 __device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const TkPrep *table, int nprep, int uniform_m,
                                                    int &row) {
-  if (!table) { row = blockIdx.x; return single; }
+  if (!table) {
+    // Workgroups go to the 8 XCDs in turn, and 8 consecutive rows share every 128-byte line of the
+    // operand layout (16 bytes each). With the rows taken in this order a line is written by one XCD,
+    // so its pieces meet in one L2 and leave it as a whole line, not as eight masked writes.
+    const unsigned blk = blockIdx.x;
+    if ((gridDim.x & 63u) == 0) {
+      const unsigned xcd = blk & 7u, slot = blk >> 3;
+      row = (int)((((slot >> 3) * 8u + xcd) * 8u) + (slot & 7u));
+    } else {
+      row = (int)blk;
+    }
+    return single;
+  }
   if (uniform_m > 0) {
     const int t = (int)blockIdx.x / uniform_m;
     row = (int)blockIdx.x - t * uniform_m;
@@ -2153,13 +2165,14 @@ __device__ __forceinline__ void load_piece(const void *act, int dtype, size_t ba
 // Rows of up to TK_PREP_HELD * 256 pieces (K <= 16384) are read from memory once: every thread keeps
 // its pieces in registers between the pass that finds the row maximum and the pass that quantizes.
 #define TK_PREP_HELD 4
+template <int HELD>
 __device__ __forceinline__ void row_absmax_held(const void *act, int dtype, size_t base, size_t k, size_t npieces,
-                                                bool vec, float (&held)[TK_PREP_HELD][16], float *sh, float &gamma,
+                                                bool vec, float (&held)[HELD][16], float *sh, float &gamma,
                                                 int &nonfinite, int *shi) {
   float g = 0.0f;
   int nf = 0;
 #pragma unroll
-  for (int it = 0; it < TK_PREP_HELD; ++it) {
+  for (int it = 0; it < HELD; ++it) {
     const size_t pc = (size_t)threadIdx.x + (size_t)it * TK_WG;
     if (pc < npieces) {
       load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, held[it]);
@@ -2177,6 +2190,9 @@ __device__ __forceinline__ void row_absmax_held(const void *act, int dtype, size
 }
 
 // Per-token int8 absmax quant (crates/tritium-spec/src/lib.rs:351-378) straight into operand order.
+// HELD = pieces a thread keeps in registers: 1 for rows of up to 256 pieces (K <= 4096), 2 up to 512:
+// the registers saved double the resident workgroups, so that 2048 tokens run as one round.
+template <int HELD>
 __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                            int nprep, int uniform_m) {
   __shared__ float shf[4];
@@ -2196,8 +2212,8 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
     nm.inv = row_inv_rms(act, dtype, base, k, pp.norm_eps, part);
   }
   const size_t npieces = nb * 16;
-  const bool resident = !nm.kind && npieces <= (size_t)TK_PREP_HELD * TK_WG;
-  float held[TK_PREP_HELD][16];
+  const bool resident = !nm.kind && npieces <= (size_t)HELD * TK_WG;
+  float held[HELD][16];
   float gamma;
   int nonfinite;
   if (resident)
@@ -2248,7 +2264,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
   };
   if (resident) {
 #pragma unroll
-    for (int it = 0; it < TK_PREP_HELD; ++it) {
+    for (int it = 0; it < HELD; ++it) {
       const size_t pc = (size_t)threadIdx.x + (size_t)it * TK_WG;
       if (pc < npieces) emit(pc, held[it]);
     }
@@ -2452,7 +2468,14 @@ hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const T
   TkPrep dummy = {};
   const TkPrep &sg = single ? *single : dummy;
   switch (kind) {
-    case TK_PREP_A8: hipLaunchKernelGGL(tk_prep_a8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m); break;
+    case TK_PREP_A8:
+      if (single && single->nb * 16 <= (size_t)TK_WG)
+        hipLaunchKernelGGL(tk_prep_a8_kernel<1>, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m);
+      else if (single && single->nb * 16 <= 2 * (size_t)TK_WG)
+        hipLaunchKernelGGL(tk_prep_a8_kernel<2>, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m);
+      else
+        hipLaunchKernelGGL(tk_prep_a8_kernel<TK_PREP_HELD>, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m);
+      break;
     case TK_PREP_DIGITS: hipLaunchKernelGGL(tk_prep_digits_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m); break;
     case TK_PREP_I8: hipLaunchKernelGGL(tk_prep_i8_kernel, dim3(rows), dim3(TK_WG), 0, s, sg, table, nprep, uniform_m); break;
     default: return hipErrorInvalidValue;

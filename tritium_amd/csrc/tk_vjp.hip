@@ -152,12 +152,22 @@ __global__ __launch_bounds__(256) void tk_vjp_weight_kernel(int n, int k, int m,
   }
 }
 
-__global__ __launch_bounds__(256) void tk_vjp_bias_kernel(int n, int m, const float *__restrict__ grad_output,
-                                                          float *__restrict__ grad_bias) {
-  const int ni = blockIdx.x * 256 + threadIdx.x;
+// grad_bias. One thread per column walks the tokens in order; a wave covers 64 adjacent columns, and
+// eight loads are in flight per thread (the additions stay in token order).
+__global__ __launch_bounds__(64) void tk_vjp_bias_kernel(int n, int m, const float *__restrict__ grad_output,
+                                                         float *__restrict__ grad_bias) {
+  const int ni = blockIdx.x * 64 + threadIdx.x;
   if (ni >= n) return;
   float acc = 0.0f;
-  for (int mi = 0; mi < m; ++mi) acc = __fadd_rn(acc, ldg(grad_output + (size_t)mi * n + ni));
+  int mi = 0;
+  for (; mi + 8 <= m; mi += 8) {
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) v[q] = ldg(grad_output + (size_t)(mi + q) * n + ni);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc = __fadd_rn(acc, v[q]);
+  }
+  for (; mi < m; ++mi) acc = __fadd_rn(acc, ldg(grad_output + (size_t)mi * n + ni));
   *(TKV_GLOBAL float *)(grad_bias + ni) = acc;
 }
 
@@ -182,7 +192,7 @@ hipError_t tk_launch_projected_vjp(hipStream_t s, const uint8_t *codes, size_t n
     if (e != hipSuccess) return e;
   }
   if (grad_bias && n) {
-    hipLaunchKernelGGL(tk_vjp_bias_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (int)n, (int)m,
+    hipLaunchKernelGGL(tk_vjp_bias_kernel, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, s, (int)n, (int)m,
                        grad_output, grad_bias);
     return hipGetLastError();
   }
