@@ -3,11 +3,13 @@
 // for the container and load_ternary (crates/tritium-nn/src/model/weights.rs:143-333) for turning a
 // tensor of type I2_S, TQ1_0 or TQ2_0 into packed rows plus one scale per output row.
 // Host code only. Every read is length-checked; no input can make it read out of bounds.
+#include <cstdio>
 #include <cstring>
 #include <map>
 #include <memory>
 #include <new>
 #include <string>
+#include <string_view>
 #include <vector>
 
 #include "tk_host.h"
@@ -164,7 +166,9 @@ float f32_from_bits(uint32_t b) {
 struct tk_gguf {
   uint32_t version = 0;
   uint64_t alignment = kDefaultAlignment, tensor_data_offset = 0;
-  std::map<std::string, Value> metadata;  // a later duplicate key replaces the earlier one, as BTreeMap::insert does
+  // a later duplicate key replaces the earlier one, as BTreeMap::insert does; std::less<> lets the
+  // getters look a C string up without building a std::string (nothing in them can throw)
+  std::map<std::string, Value, std::less<>> metadata;
   std::vector<Tensor> tensors;
 };
 
@@ -236,7 +240,7 @@ const char *kind_text(int kind) {
 // The value a getter addresses: the key's value (index < 0) or element `index` of its array.
 const Value *lookup(const tk_gguf *g, const char *key, long long index) {
   if (!g || !key) return nullptr;
-  auto it = g->metadata.find(key);
+  auto it = g->metadata.find(std::string_view(key));
   if (it == g->metadata.end()) return nullptr;
   const Value *v = &it->second;
   if (index < 0) return v;
@@ -255,8 +259,9 @@ void fill_info(const Tensor &t, tk_gguf_tensor *out) {
 }
 
 const Tensor *find_tensor(const tk_gguf *g, const char *name) {
+  const std::string_view want(name);
   for (const Tensor &t : g->tensors)
-    if (t.name == name) return &t;
+    if (std::string_view(t.name) == want) return &t;
   return nullptr;
 }
 
@@ -437,8 +442,9 @@ extern "C" int tk_gguf_load_ternary(const tk_gguf *g, const uint8_t *file, size_
     float scale;
     const int rc = tk_convert_i2s_to_tq2_0(p, (size_t)len, n, k, packed, packed_len, &scale);
     if (rc == TK_ERR_INVALID_INPUT) {  // the loader reports a bad payload as a backend error (weights.rs:214-216)
-      const std::string why = tk_last_error();
-      return tk_fail(TK_ERR_BACKEND, "%s: %s", name, why.c_str());
+      char why[256];
+      std::snprintf(why, sizeof why, "%s", tk_last_error());
+      return tk_fail(TK_ERR_BACKEND, "%s: %s", name, why);
     }
     if (rc != TK_OK) return rc;
     for (size_t r = 0; r < n; ++r) row_scales[r] = scale;
@@ -501,7 +507,12 @@ extern "C" int tk_gguf_load_ternary(const tk_gguf *g, const uint8_t *file, size_
   // One scale for the tensor. A repacked file keeps the source's exact f32 scale in metadata; it must
   // agree with the block scale to f16 precision (weights.rs:307-329).
   float scale = have_tensor_scale ? tensor_scale : 0.0f;
-  const std::string key = std::string("tritium.i2s_scale.") + name;
+  std::string key;
+  try {
+    key = std::string("tritium.i2s_scale.") + name;
+  } catch (const std::bad_alloc &) {
+    return tk_fail(TK_ERR_BACKEND, "tk_gguf_load_ternary: host allocation failed");
+  }
   float exact;
   if (tk_gguf_meta_f32(g, key.c_str(), -1, &exact)) {
     if (have_tensor_scale) {
