@@ -18,35 +18,42 @@
 #include "tk_internal.h"
 
 #define TKV_GLOBAL __attribute__((address_space(1)))
+#ifndef TKV_ACT_TOK
+#define TKV_ACT_TOK 4  // tokens per thread of the grad_act kernel (2: 3.2 ms, 4: 2.9 ms, 8: 4.5 ms at M=2048 K=2560 N=6912)
+#endif
 
 namespace {
 
 __device__ __forceinline__ float ldg(const float *p) { return *(const TKV_GLOBAL float *)p; }
 
-// grad_act. A workgroup owns 16 tokens x 4 K blocks; a thread owns 4 tokens x the 16 elements of one
-// code dword (piece g, dword j of its K block), the four waves are the four token groups. Per tile of
-// 16 weight rows the upstream values and scales pass through LDS (two buffers, one barrier a tile).
+// grad_act. A workgroup owns 4*TOK tokens x 4 K blocks; a thread owns TOK tokens x the 16 elements of
+// one code dword (piece g, dword j of its K block), the four waves are the four token groups. Per tile
+// of 16 weight rows the upstream values and scales pass through LDS (two buffers, one barrier a tile).
+template <int TOK>
 __global__ __launch_bounds__(256) void tk_vjp_act_kernel(const uint8_t *__restrict__ codes, int nb, int n, int k, int m,
                                                          const float *__restrict__ scales,
                                                          const float *__restrict__ grad_output,
                                                          float *__restrict__ grad_act) {
-  __shared__ float s_up[2][16][16];  // [buffer][token][row of the tile]
+  constexpr int WT = 4 * TOK;            // tokens per workgroup
+  __shared__ float s_up[2][WT][16];      // [buffer][token][row of the tile]
   __shared__ float s_sc[2][16];
   const int tid = threadIdx.x;
   const int set = tid >> 4, ls = tid & 15, g = ls >> 2, j = ls & 3;
   const int kb = blockIdx.x * 4 + (set & 3), mg = set >> 2;
-  const int m0 = blockIdx.y * 16;
+  const int m0 = blockIdx.y * WT;
   const int kbc = min(kb, nb - 1);  // blocks past the end re-read the last one; nothing of them is stored
   const int n_tiles = (n + 15) >> 4;
-  float acc[4][16];
+  float acc[TOK][16];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TOK; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
 
   auto stage = [&](int buf, int t) {
-    const int mi = m0 + (tid >> 4), ni = t * 16 + (tid & 15);
-    s_up[buf][tid >> 4][tid & 15] = (mi < m && ni < n) ? ldg(grad_output + (size_t)mi * n + ni) : 0.0f;
+    if (tid < WT * 16) {
+      const int mi = m0 + (tid >> 4), ni = t * 16 + (tid & 15);
+      s_up[buf][tid >> 4][tid & 15] = (mi < m && ni < n) ? ldg(grad_output + (size_t)mi * n + ni) : 0.0f;
+    }
     if (tid < 16) s_sc[buf][tid] = (t * 16 + tid < n) ? ldg(scales + t * 16 + tid) : 0.0f;
   };
   stage(0, 0);
@@ -63,16 +70,16 @@ __global__ __launch_bounds__(256) void tk_vjp_act_kernel(const uint8_t *__restri
     for (int r = 0; r < 16; ++r) {
       if (r < rmax) {  // uniform
         const float s = s_sc[buf][r];
-        float u[4];
+        float u[TOK];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) u[i] = s_up[buf][mg * 4 + i][r];
+        for (int i = 0; i < TOK; ++i) u[i] = s_up[buf][mg * TOK + i][r];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           // e = b*4 + sl: byte b of the dword, bit pair sl
           const int code = (int)((w[r] >> (8 * (e >> 2) + 2 * (e & 3))) & 3u);
           const float projected = __fmul_rn((float)(code - 1), s);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i][e] = __fadd_rn(acc[i][e], __fmul_rn(u[i], projected));
+          for (int i = 0; i < TOK; ++i) acc[i][e] = __fadd_rn(acc[i][e], __fmul_rn(u[i], projected));
         }
       }
     }
@@ -82,8 +89,8 @@ __global__ __launch_bounds__(256) void tk_vjp_act_kernel(const uint8_t *__restri
   // byte b of this dword is byte i = g*16 + j*4 + b of the block: elements (g/2)*128 + sl*32 + (g%2)*16 + j*4 + b
   const int e0 = kb * 256 + (g >> 1) * 128 + (g & 1) * 16 + j * 4;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int mi = m0 + mg * 4 + i;
+  for (int i = 0; i < TOK; ++i) {
+    const int mi = m0 + mg * TOK + i;
     if (mi >= m) continue;
     float *row = grad_act + (size_t)mi * k;
 #pragma unroll
@@ -153,19 +160,19 @@ __global__ __launch_bounds__(256) void tk_vjp_weight_kernel(int n, int k, int m,
 }
 
 // grad_bias. One thread per column walks the tokens in order; a wave covers 64 adjacent columns, and
-// eight loads are in flight per thread (the additions stay in token order).
+// 32 loads are in flight per thread (the additions stay in token order).
 __global__ __launch_bounds__(64) void tk_vjp_bias_kernel(int n, int m, const float *__restrict__ grad_output,
                                                          float *__restrict__ grad_bias) {
   const int ni = blockIdx.x * 64 + threadIdx.x;
   if (ni >= n) return;
   float acc = 0.0f;
   int mi = 0;
-  for (; mi + 8 <= m; mi += 8) {
-    float v[8];
+  for (; mi + 32 <= m; mi += 32) {
+    float v[32];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) v[q] = ldg(grad_output + (size_t)(mi + q) * n + ni);
+    for (int q = 0; q < 32; ++q) v[q] = ldg(grad_output + (size_t)(mi + q) * n + ni);
 #pragma unroll
-    for (int q = 0; q < 8; ++q) acc = __fadd_rn(acc, v[q]);
+    for (int q = 0; q < 32; ++q) acc = __fadd_rn(acc, v[q]);
   }
   for (; mi < m; ++mi) acc = __fadd_rn(acc, ldg(grad_output + (size_t)mi * n + ni));
   *(TKV_GLOBAL float *)(grad_bias + ni) = acc;
@@ -179,8 +186,9 @@ hipError_t tk_launch_projected_vjp(hipStream_t s, const uint8_t *codes, size_t n
                                    const float *scales, const float *act, const float *grad_output, float *grad_act,
                                    float *grad_w, float *grad_bias) {
   if (grad_act && m && n && k) {
-    dim3 grid((unsigned)((nb + 3) / 4), (unsigned)((m + 15) / 16));
-    hipLaunchKernelGGL(tk_vjp_act_kernel, grid, dim3(256), 0, s, codes, (int)nb, (int)n, (int)k, (int)m, scales,
+    constexpr int TOK = TKV_ACT_TOK;
+    dim3 grid((unsigned)((nb + 3) / 4), (unsigned)((m + 4 * TOK - 1) / (4 * TOK)));
+    hipLaunchKernelGGL(tk_vjp_act_kernel<TOK>, grid, dim3(256), 0, s, codes, (int)nb, (int)n, (int)k, (int)m, scales,
                        grad_output, grad_act);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
