@@ -239,6 +239,45 @@ def test_three_planes_a8(backend, oracle):
         dout.free()
 
 
+@pytest.mark.parametrize("m,n,k,planes", [(56, 48, 3072, 2), (64, 200, 2816, 3), (40, 16400, 4352, 1)])
+def test_single_launch_with_rows_beyond_lds(backend, oracle, m, n, k, planes, decode_kernel):
+    """One launch whose operand rows exceed LDS (more than 48 rows, or more than 32 on a large launch)
+    goes through the prefill kernel by default; forced back onto the decode kernels it gives the same
+    bits, and both equal the CPU backend's."""
+    if decode_kernel != "stream":
+        pytest.skip("single configuration")
+    print("case rows-beyond-lds", m, n, k, planes, flush=True)
+    backend.set_decode_kernel(0)  # automatic choice
+    rng = np.random.default_rng(m + n)
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)[:planes]]
+    scs = [scales(rng, n) for _ in range(planes)]
+    packed, layer = _layer(backend, oracle, ws, scs)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    dact, dout = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    backend.linear_a8(layer, dact, m, dout)
+    a = dout.to_host()
+    backend.set_decode_kernel(2)  # the streaming decode kernel
+    try:
+        backend.linear_a8(layer, dact, m, dout)
+        b = dout.to_host()
+    finally:
+        backend.set_decode_kernel(0)  # the float call below is on the automatic choice too
+    rows = np.arange(m) if n * k <= 1 << 21 else np.array([0, m // 2, m - 1])
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act[rows], len(rows), n, k)
+    assert same_bits(a, b) and same_bits(a.reshape(m, n)[rows], want)
+    if m <= 16 * 4:  # the float contract on the same path: 4 digit rows per token
+        mf = m // 4
+        dout2 = backend.empty(mf * n, "f32")
+        backend.linear_float(layer, dact, mf, dout2)
+        got = dout2.to_host().reshape(mf, n)
+        wantf = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act[:mf], mf, n, k)
+        assert rel_err(got, wantf) <= 1e-3 and accepts(got, wantf, rel=1e-4, floor=1.0).all()
+        dout2.free()
+    dact.free()
+    dout.free()
+    layer.free()
+
+
 def test_gemm_crossover_is_bit_neutral(backend, oracle):
     """Decode kernel and GEMM kernel give identical bits (cuda tests.rs:2100-2190: IMMA == dp4a)."""
     rng = np.random.default_rng(23)

@@ -669,6 +669,17 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
 
   Plan pl;
   plan_shape(ctx, layer, n, k, m, mode, out_dtype, &pl);
+  // Operand rows that do not fit in LDS: beyond 48 rows, or beyond 32 when the launch is large, the
+  // prefill kernel (rows streamed from L2 block by block) beats the decode kernels that re-stage
+  // slices of K behind barriers. Measured with int8 rows on single launches, decode vs prefill
+  // kernel: 64 x 5120 -> 17408, 1/2/3 planes: 63/71/70 -> 37/35/41 us; 64 x 17408 -> 5120: 113-125 ->
+  // 88-108 us; 64 x 6912 -> 2560: 47 -> 42 us; 40 x 5120 -> 17408 x 3 planes: 60 -> 40 us; but
+  // 48 x 6912 -> 2560: 38 -> 42 us and 32 rows always slower (31 -> 42, 71 -> 90 us): those stay.
+  if (pl.skinny && ctx->decode_force == DECODE_AUTO && !pl.flow_ok &&
+      ((size_t)pl.pr.R > 48 || ((size_t)pl.pr.R > 32 && (size_t)pl.pr.n_tiles * (size_t)layer->n_planes >= 1024))) {
+    pl.skinny = false;
+    plan_gemm(&pl);
+  }
   const size_t nb = pl.pr.nb, R = pl.pr.R;
   int variant = DECODE_KSPLIT, run_tiles = 1;
   unsigned flow_groups = 0;
