@@ -568,7 +568,12 @@ static bool prefer_stream(const tk_ctx *ctx, unsigned groups);
 
 // Fills everything of a plan that does not depend on workspace addresses.
 // GEMM form of a planned problem: padded operand row stride, tile grid and its split over the XCDs.
-static void plan_gemm(Plan *pl) {
+// fill > 0 (single launches): one plane normally gives a wave 4 tiles; when that leaves fewer
+// workgroups than `fill` (four per CU), 2 tiles per wave double them. A/B on one box, call incl.
+// quantization, K=2560 N=6912: 64..256 tokens 25 -> 18-19 us, 512: 26.5 -> 23.6, 768: 33.2 -> 28.8,
+// 2048 (864 workgroups): 59.8 -> 58.5; from 1088 workgroups on the 4-tile form wins (1024 x 5120 ->
+// 17408: 100 vs 104 us; 4096 x 5120 -> 17408: 314 vs 362 us).
+static void plan_gemm(Plan *pl, unsigned fill = 0) {
   TkProblem &pr = pl->pr;
   const size_t R = (size_t)pr.R;
   // The GEMM reads, per K block, 16 segments of the operand rows that are exactly rs*16 bytes apart,
@@ -578,7 +583,12 @@ static void plan_gemm(Plan *pl) {
   pl->cfg.rt = 4;
   pl->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();  // three 64-row blocks of 256 k + the row constants
   pl->grid_m = (unsigned)((R + 63) / 64);
-  const unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(pr.planes);
+  unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(pr.planes);
+  pl->cfg.gemm_nt = 0;
+  if (fill && pr.planes == 1 && pl->grid_m * (((unsigned)pr.n_tiles + per_wg - 1) / per_wg) < fill) {
+    per_wg /= 2;
+    pl->cfg.gemm_nt = 2;
+  }
   pl->grid_n = ((unsigned)pr.n_tiles + per_wg - 1) / per_wg;
   // split the tile grid over the 8 XCDs so that each L2 holds few A row blocks and few weight
   // column blocks: minimise bytes touched per XCD = K*(64*sub_m + 4*tiles_per_wg*planes*sub_n)
@@ -643,7 +653,7 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->flow_lds = nb * 256 * R;
     pl->flow_ok = pl->flow_lds <= kLdsFlowMax;
   } else {
-    plan_gemm(pl);
+    plan_gemm(pl, 4u * (unsigned)ctx->info.compute_units);
   }
 }
 
@@ -678,7 +688,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   if (pl.skinny && ctx->decode_force == DECODE_AUTO && !pl.flow_ok &&
       ((size_t)pl.pr.R > 48 || ((size_t)pl.pr.R > 32 && (size_t)pl.pr.n_tiles * (size_t)layer->n_planes >= 1024))) {
     pl.skinny = false;
-    plan_gemm(&pl);
+    plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units);
   }
   const size_t nb = pl.pr.nb, R = pl.pr.R;
   int variant = DECODE_KSPLIT, run_tiles = 1;
