@@ -1325,6 +1325,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   // re-stages slices of K behind barriers.
   if (ctx->decode_force == DECODE_AUTO && !flow_ok && rt >= 2) variant = DECODE_GEMM;
   std::vector<int> wg_prob;
+  int group_gemm_nt = 0;
   unsigned groups_total = 0;
   std::vector<int> flow_wg_prob;
   TkLaunchCfg flow_cfg{};
@@ -1343,6 +1344,20 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       nbs.push_back(plans[i].pr.nb);
       wts.push_back((double)plans[i].pr.n_tiles * (double)plans[i].pr.nb);
     }
+    // one plane: two tiles per wave when four would leave fewer than four workgroups per CU (as for
+    // single launches)
+    bool gemm_nt2 = false;
+    if (planes == 1) {
+      unsigned total = 0;
+      for (size_t i = 0; i < count; ++i) {
+        if (plans[i].flow_ok) continue;
+        Plan tmp = plans[i];
+        plan_gemm(&tmp);
+        total += 8u * (unsigned)tmp.pr.sub_m * (unsigned)tmp.pr.sub_n;
+      }
+      gemm_nt2 = total < 4u * (unsigned)ctx->info.compute_units;
+    }
+    group_gemm_nt = gemm_nt2 ? 2 : 0;
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds);
@@ -1368,7 +1383,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
         }
         continue;
       }
-      plan_gemm(&plans[i]);
+      plan_gemm(&plans[i], gemm_nt2 ? ~0u : 0u);
       const unsigned gi = 8u * (unsigned)plans[i].pr.sub_m * (unsigned)plans[i].pr.sub_n;
       plans[i].pr.group_begin = (int)groups_total;
       for (unsigned j = 0; j < gi; ++j) wg_prob.push_back((int)i);
@@ -1474,6 +1489,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   g->cfg.rt = rt;
   g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
   if (variant == DECODE_GEMM) g->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();
+  g->cfg.gemm_nt = variant == DECODE_GEMM ? group_gemm_nt : 0;
   g->cfg.grid = variant == DECODE_KSPLIT ? tiles : groups_total;
   g->cfg.waves = fw;
   {

@@ -87,7 +87,7 @@ struct TkLaunchCfg {
   int waves;    // flow kernel: waves per workgroup (4, or 8 when the operand rows need > 64 KiB of LDS)
   int ring;     // flow kernel: positions in the prefetch ring (2..5)
   int wide_mfma; // flow kernel: 32x32x32 form (17..64 operand rows, row constants in LDS)
-  int gemm_nt;  // prefill kernel, single launch of one plane: tiles per wave (0 = the default 4, or 2)
+  int gemm_nt;  // prefill kernel, one plane: tiles per wave (0 = the default 4, or 2)
 };
 
 #ifdef __cplusplus

@@ -2725,8 +2725,10 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
 #define TK_GEMM32_CASE(PP, NTT)                                                                              \
   if (table) return gemm_launch_one(tk_gemm32_kernel<PP, NTT, true>, s, sg, table, wg_prob, cfg, wgs);        \
   return gemm_launch_one(tk_gemm32_kernel<PP, NTT, false>, s, sg, table, wg_prob, cfg, wgs);
-  if (!table && cfg.planes == 1 && cfg.gemm_nt == 2)
+  if (cfg.planes == 1 && cfg.gemm_nt == 2) {
+    if (table) return gemm_launch_one(tk_gemm32_kernel<1, 2, true>, s, sg, table, wg_prob, cfg, wgs);
     return gemm_launch_one(tk_gemm32_kernel<1, 2, false>, s, sg, table, wg_prob, cfg, wgs);
+  }
   switch (cfg.planes) {
     case 1: TK_GEMM32_CASE(1, 4)
     case 2: TK_GEMM32_CASE(2, 2)
