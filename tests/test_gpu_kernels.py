@@ -239,10 +239,11 @@ def test_three_planes_a8(backend, oracle):
         dout.free()
 
 
-@pytest.mark.parametrize("m,n,k,planes", [(56, 48, 3072, 2), (64, 200, 2816, 3), (40, 16400, 4352, 1)])
+@pytest.mark.parametrize("m,n,k,planes", [(56, 48, 3072, 2), (64, 200, 2816, 3), (40, 16400, 4352, 1), (36, 48, 4864, 1),
+                                            (28, 16400, 6144, 1)])
 def test_single_launch_with_rows_beyond_lds(backend, oracle, m, n, k, planes, decode_kernel):
-    """One launch whose operand rows exceed LDS (more than 48 rows, or more than 32 on a large launch)
-    goes through the prefill kernel by default; forced back onto the decode kernels it gives the same
+    """One launch whose operand rows exceed LDS (more than 32 rows, or more than 16 on a layer of at
+    least 16384 outputs) goes through the prefill kernel by default; forced back onto the decode kernels it gives the same
     bits, and both equal the CPU backend's."""
     if decode_kernel != "stream":
         pytest.skip("single configuration")

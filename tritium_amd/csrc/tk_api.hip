@@ -679,17 +679,6 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
 
   Plan pl;
   plan_shape(ctx, layer, n, k, m, mode, out_dtype, &pl);
-  // Operand rows that do not fit in LDS: beyond 48 rows, or beyond 32 when the launch is large, the
-  // prefill kernel (rows streamed from L2 block by block) beats the decode kernels that re-stage
-  // slices of K behind barriers. Measured with int8 rows on single launches, decode vs prefill
-  // kernel: 64 x 5120 -> 17408, 1/2/3 planes: 63/71/70 -> 37/35/41 us; 64 x 17408 -> 5120: 113-125 ->
-  // 88-108 us; 64 x 6912 -> 2560: 47 -> 42 us; 40 x 5120 -> 17408 x 3 planes: 60 -> 40 us; but
-  // 48 x 6912 -> 2560: 38 -> 42 us and 32 rows always slower (31 -> 42, 71 -> 90 us): those stay.
-  if (pl.skinny && ctx->decode_force == DECODE_AUTO && !pl.flow_ok &&
-      ((size_t)pl.pr.R > 48 || ((size_t)pl.pr.R > 32 && (size_t)pl.pr.n_tiles * (size_t)layer->n_planes >= 1024))) {
-    pl.skinny = false;
-    plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units);
-  }
   const size_t nb = pl.pr.nb, R = pl.pr.R;
   int variant = DECODE_KSPLIT, run_tiles = 1;
   unsigned flow_groups = 0;
@@ -704,6 +693,18 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
     variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
+    // Operand rows that do not fit in LDS: the prefill kernel (rows streamed from L2 block by block)
+    // beats the decode kernels that re-stage slices of K behind barriers, beyond 32 rows always and
+    // from 17 rows on layers of at least 16384 outputs. A/B on one box, int8 rows,
+    // call incl. quantization, decode kernel -> prefill kernel: 64 x 5120 -> 17408 with 1/2/3 planes
+    // 63/71/70 -> 28/35/41 us; 64 x 17408 -> 5120 113 -> 68 us; 48 x 6912 -> 2560 38 -> 31 us;
+    // 40 x 5120 -> 17408 46 -> 28 us; 32 x 6912 -> 16384 53 -> 32 us; 32 x 5632 -> 17408 x 3 planes
+    // 60 -> 43 us. Narrower launches of up to 32 rows stay on the K-split kernel (32 x 6912 -> 2560: 31
+    // vs 31 us; 24 rows 26 vs 31; 32 x 8192 -> 8192 x 2 planes: 40 vs 45; 17 x 17408 -> 5120: 55 vs 65).
+    if (ctx->decode_force == DECODE_AUTO && !pl.flow_ok && (R > 32 || (R > 16 && pl.pr.n_tiles >= 1024))) {
+      pl.skinny = false;
+      plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units);
+    }
   }
   TKCHK(ensure(ctx, ctx->ap, (size_t)pl.pr.rs * nb * 256));
   TKCHK(ensure(ctx, ctx->rowsum, R * 4));
