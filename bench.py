@@ -273,6 +273,16 @@ def bench_config5(T, be, rng):
                               "ms_per_step": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
                               "frac_of_hbm_peak": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}}
     g.destroy()
+    # the same projections as single calls (one linear per launch, quantization included), rotating over
+    # the 8 layers (535 MB of codes per projection kind): rows beyond LDS -> the prefill kernel
+    single = {}
+    for name, src in (("up", hid), ("down", mid)):
+        n, k = shapes[name]
+        o = outs[0 if name == "up" else 1]
+        ms1 = time_calls(be, lambda i: be.linear_a8(lins[i % layers_n][name], src, m, o), 64)
+        by1 = algorithmic_bytes(m, n, k, 3, 2, 2, a8=True)
+        single[name] = {"us_per_call": round(ms1 * 1e3, 1), "GB/s": round(by1 / ms1 / 1e6, 1)}
+    res["decode_batch64_single_calls"] = dict(single, workload="one projection per call, 3 planes, batch 64, incl. quantization")
     for x in outs + [hid, mid]:
         x.free()
     for L in lins:
