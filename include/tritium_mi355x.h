@@ -257,6 +257,19 @@ int tk_linear_float(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, i
 int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
                  size_t m, void *out, int out_dtype);
 
+/* tk_linear_a8 for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments,
+ * same kernels and same bits as tk_linear_a8; the workspace of the call (operand rows, row sums,
+ * per-token scales and flags) lives in a static device array of TK_NOALLOC_SCRATCH_BYTES that every
+ * GPU the library runs on holds until the process ends, and the call makes no hipMalloc, hipFree or
+ * other allocating call. A shape whose workspace does not fit (about (m + 16) * ceil(k/256) * 256
+ * bytes: e.g. 64 tokens at k = 17408, or 2048 tokens at k = 3584) is answered with
+ * TK_ERR_INVALID_INPUT. Every call on one GPU shares that GPU's array: calls that overlap on one GPU
+ * (two contexts of a device, two threads) race and must be serialised by the caller. */
+#define TK_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
+int tk_linear_a8_noalloc(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
+                         size_t m, void *out, int out_dtype);
+
 /* RMSNorm in front of the per-token int8 quantization, as one launch: what the CUDA decode calls
  * launch_rmsnorm_quant before the q/k/v and gate/up projections
  * (crates/tritium-cuda/src/cuda/mod.rs:1029-1040). y[i] = (x[i] * inv) * s(w[i]),

@@ -98,6 +98,7 @@ SIGNATURES = {
     "tk_linear_salt": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_salt_seq": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
+    "tk_linear_a8_noalloc": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_rmsnorm_quant_i8": (C.c_int, [vp, vp, C.c_int, C.POINTER(RmsNorm), sz, sz, vp, vp, vp]),
     "tk_linear_rmsnorm_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, C.POINTER(RmsNorm), sz, vp, C.c_int]),
     "tk_group_create_normed": (C.c_int, [vp, C.POINTER(GroupMember), C.POINTER(RmsNorm), sz, C.c_int, C.c_int,

@@ -427,6 +427,10 @@ class Mi355xBackend:
     def linear_a8(self, layer, act, m, out):
         self._lin(self._lib.tk_linear_a8, layer, act, m, out)
 
+    def linear_a8_noalloc(self, layer, act, m, out):
+        """linear_a8 on the static device scratch: no allocation; refuses shapes that do not fit."""
+        self._lin(self._lib.tk_linear_a8_noalloc, layer, act, m, out)
+
     def linear_float_seq(self, layer, act, m, out):
         self._lin(self._lib.tk_linear_float_seq, layer, act, m, out)
 

@@ -75,6 +75,7 @@ struct tk_ctx {
   int flow_run_tiles = 0;  // 0 = automatic
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
+  uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum;
   int *d_invalid = nullptr;
 };
@@ -139,6 +140,16 @@ static int choose_decode(const tk_ctx *ctx, bool flow_ok, unsigned flow_groups, 
   if (!flow_ok && prefer_stream(ctx, stream_groups)) return 2;
   return 1;
 }
+
+// ------------------------------------------------------------------------------------------
+// static device scratch: the workspace of the entry point that allocates nothing
+// (tk_linear_a8_noalloc). Every GPU the library runs on holds its own copy of this array until the
+// process ends. In host code the array's name is only a stand-in for the symbol: the device address
+// is resolved once per context by tk_init (hipGetSymbolAddress with the context's device current)
+// and kept in tk_ctx::static_scratch, which is what kernels, and nothing else, receive.
+// ------------------------------------------------------------------------------------------
+#define TK_STATIC_SCRATCH_BYTES TK_NOALLOC_SCRATCH_BYTES  // the stated maximum (include/tritium_mi355x.h)
+static __device__ __align__(256) unsigned char scratch[TK_STATIC_SCRATCH_BYTES];
 
 // ------------------------------------------------------------------------------------------
 // lifetime
@@ -206,6 +217,15 @@ extern "C" int tk_init(int device, tk_ctx **out) {
     return rc;
   }
   ctx->d_invalid = (int *)p;
+  void *sp = nullptr;
+  e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));  // device `device` is current: its copy of the array
+  if (e != hipSuccess || !sp) {
+    (void)hipFree(ctx->d_invalid);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return tk_fail(TK_ERR_BACKEND, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+  }
+  ctx->static_scratch = (uint8_t *)sp;
   *out = ctx;
   return TK_OK;
 }
@@ -215,7 +235,8 @@ extern "C" void tk_destroy(tk_ctx *ctx) {
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
   DevBuf *bufs[] = {&ctx->ap, &ctx->rowsum, &ctx->fscale, &ctx->aux, &ctx->exps,
-                    &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp};
+                    &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp,
+                    &ctx->ynorm, &ctx->blocksum};
   for (DevBuf *b : bufs)
     if (b->p) (void)hipFree(b->p);
   if (ctx->d_invalid) (void)hipFree(ctx->d_invalid);
@@ -664,9 +685,56 @@ static int check_norm(const tk_rmsnorm *norm) {
   return TK_OK;
 }
 
+// The per-call workspace of run_linear: operand rows and the per-row / per-token side arrays.
+struct Workspace {
+  int8_t *ap;
+  int32_t *rowsum;
+  float *fscale, *aux;
+  int32_t *exps;
+  uint32_t *flags;
+  float *ynorm;
+};
+
+// From the context's grow-only buffers (may allocate), or -- static_ws -- carved out of the static
+// device scratch, which allocates nothing and refuses what does not fit.
+static int take_workspace(tk_ctx *ctx, bool static_ws, size_t ap_bytes, size_t R, size_t m, size_t ynorm_bytes,
+                          Workspace *ws) {
+  if (!static_ws) {
+    TKCHK(ensure(ctx, ctx->ap, ap_bytes));
+    TKCHK(ensure(ctx, ctx->rowsum, R * 4));
+    TKCHK(ensure(ctx, ctx->fscale, m * 4));
+    TKCHK(ensure(ctx, ctx->aux, m * 4));
+    TKCHK(ensure(ctx, ctx->exps, m * 4));
+    TKCHK(ensure(ctx, ctx->flags, m * 4));
+    if (ynorm_bytes) TKCHK(ensure(ctx, ctx->ynorm, ynorm_bytes));
+    *ws = Workspace{(int8_t *)ctx->ap.p,   (int32_t *)ctx->rowsum.p, (float *)ctx->fscale.p, (float *)ctx->aux.p,
+                    (int32_t *)ctx->exps.p, (uint32_t *)ctx->flags.p, (float *)ctx->ynorm.p};
+    return TK_OK;
+  }
+  size_t used = 0;
+  auto carve = [&](size_t bytes) {
+    uint8_t *p = ctx->static_scratch + used;
+    used += (bytes + 255) & ~(size_t)255;
+    return p;
+  };
+  ws->ap = (int8_t *)carve(ap_bytes);
+  ws->rowsum = (int32_t *)carve(R * 4);
+  ws->fscale = (float *)carve(m * 4);
+  ws->aux = (float *)carve(m * 4);
+  ws->exps = (int32_t *)carve(m * 4);
+  ws->flags = (uint32_t *)carve(m * 4);
+  ws->ynorm = ynorm_bytes ? (float *)carve(ynorm_bytes) : nullptr;
+  if (used > TK_STATIC_SCRATCH_BYTES || ap_bytes > TK_STATIC_SCRATCH_BYTES)
+    return tk_fail(TK_ERR_INVALID_INPUT,
+                   "this call needs %zu bytes of workspace; the static scratch of the allocation-free entry point "
+                   "holds %zu (operand rows take about tokens * ceil(k/256) * 256 bytes)",
+                   used, (size_t)TK_STATIC_SCRATCH_BYTES);
+  return TK_OK;
+}
+
 static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int prep_kind, const void *act,
                       int act_dtype, const float *act_scale_in, size_t m, void *out, int out_dtype,
-                      const tk_rmsnorm *norm = nullptr) {
+                      const tk_rmsnorm *norm = nullptr, bool static_ws = false) {
   size_t n, k;
   TKCHK(validate_layer(ctx, layer, &n, &k));
   if (m == 0 || n == 0) return TK_OK;  // crates/tritium-rocm/src/rocm.rs:521-523
@@ -706,28 +774,23 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
       plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units);
     }
   }
-  TKCHK(ensure(ctx, ctx->ap, (size_t)pl.pr.rs * nb * 256));
-  TKCHK(ensure(ctx, ctx->rowsum, R * 4));
-  TKCHK(ensure(ctx, ctx->fscale, m * 4));
-  TKCHK(ensure(ctx, ctx->aux, m * 4));
-  TKCHK(ensure(ctx, ctx->exps, m * 4));
-  TKCHK(ensure(ctx, ctx->flags, m * 4));
-  if (norm) TKCHK(ensure(ctx, ctx->ynorm, m * k * 4));
+  Workspace ws;
+  TKCHK(take_workspace(ctx, static_ws, (size_t)pl.pr.rs * nb * 256, R, m, norm ? m * k * 4 : 0, &ws));
 
   TkPrep &pp = pl.prep;
   if (norm) {
     pp.norm_kind = norm->zero_centered ? 2 : 1;
     pp.norm_eps = norm->eps;
     pp.norm_w = norm->weight;
-    pp.ynorm = (float *)ctx->ynorm.p;
+    pp.ynorm = ws.ynorm;
   }
   pp.act = act;
-  pp.ap = (int8_t *)ctx->ap.p;
-  pp.rowsum = (int32_t *)ctx->rowsum.p;
-  pp.act_scale = (float *)ctx->fscale.p;
-  pp.aux = (float *)ctx->aux.p;
-  pp.exps = (int32_t *)ctx->exps.p;
-  pp.flags = (uint32_t *)ctx->flags.p;
+  pp.ap = ws.ap;
+  pp.rowsum = ws.rowsum;
+  pp.act_scale = ws.fscale;
+  pp.aux = ws.aux;
+  pp.exps = ws.exps;
+  pp.flags = ws.flags;
   pp.k = k;
   pp.nb = nb;
   pp.R = R;
@@ -806,6 +869,20 @@ extern "C" int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
   return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, act, act_dtype, nullptr, m, out, out_dtype);
+}
+
+// tk_linear_a8 without any allocation: the workspace is the static device scratch. Calls that
+// overlap on one GPU (other streams, other contexts of the same device, other threads) share that
+// array and race; every element a kernel reads is written by the prep launch of the same call first,
+// so nothing of an earlier call's contents needs clearing.
+extern "C" int tk_linear_a8_noalloc(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype, size_t m,
+                                    void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, act, act_dtype, nullptr, m, out, out_dtype, nullptr, true);
 }
 
 extern "C" int tk_linear_rmsnorm_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *x, int x_dtype,
