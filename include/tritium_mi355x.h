@@ -386,6 +386,10 @@ int tk_set_flow_ring(tk_ctx *ctx, int positions);
  * 32 = 32x32x32 wherever its operand rows fit in LDS. A tuning and test knob: both forms give
  * identical bits. */
 int tk_set_flow_mfma(tk_ctx *ctx, int rows);
+/* Output tiles per wave of the one-plane prefill kernel: 0 = chosen per launch (4, or 2 when 4 would
+ * leave fewer than four workgroups per CU), 2 or 4 to force. A tuning and test knob: both forms give
+ * identical bits. */
+int tk_set_gemm_tiles(tk_ctx *ctx, int tiles);
 /* The K-split decode kernel has the finer grain (a single narrow layer), the streaming and flow
  * kernels walk whole output tiles per wave (launches that fill the chip): the latter are taken when
  * a launch needs at least this many workgroups; default = the device's CU count. No counterpart

@@ -52,3 +52,22 @@ def same_bits(a, b):
     a = np.ascontiguousarray(a, np.float32).reshape(-1)
     b = np.ascontiguousarray(b, np.float32).reshape(-1)
     return bool((a.view(np.uint32) == b.view(np.uint32)).all())
+
+
+def a8_expected(oracle, ws, scs, act):
+    """The W1.58A8 composition for whole tensors: quantize per token with the oracle, contract exactly
+    (integer products summed in f32 BLAS: every partial sum is an integer below 2^24 for K <= 65536, so
+    any summation order gives the exact value), then ((float)acc * s_w[n]) summed over planes in order,
+    times the per-token scale -- every step one f32 rounding, as crates/tritium-cpu/src/kernel.rs:921-922
+    and crates/tritium-nn/src/layers/linear.rs:272-277 do. Tests that use it also compare sampled rows
+    with the C oracle, which pins this restatement."""
+    m, k = act.shape
+    assert k * 128 < (1 << 24)
+    q, s = oracle.quantize_act_int8(act, m, k)
+    qf = np.ascontiguousarray(q, np.float32).reshape(m, k)
+    out = None
+    for w, sc in zip(ws, scs):
+        acc = qf @ np.ascontiguousarray(w.T, np.float32)
+        t = acc * np.asarray(sc, np.float32)[None, :]
+        out = t if out is None else out + t
+    return (out * np.asarray(s, np.float32).reshape(m, 1)).astype(np.float32)

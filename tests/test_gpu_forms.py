@@ -1,0 +1,163 @@
+"""Every kernel instantiation the dispatch can choose, forced at small sizes and compared bit for bit
+with the CPU oracle: the 2-tile and 4-tile forms of the one-plane prefill kernel (single and grouped
+launches), the grouped prefill kernel with one, two and three planes, and the grouped flow kernel on
+the 32x32x32 matrix instruction chosen automatically. Precedent: the reference holds its tensor-core
+kernel to `to_bits` equality with its dp4a kernel (crates/tritium-cuda/src/cuda/tests.rs:2100-2190)."""
+import numpy as np
+import pytest
+
+import tritium_amd as T
+from helpers import accepts, bf16_bits_to_f32, f32_to_bf16_bits, rel_err, same_bits, scales, ternary
+from oracle_lib import FMT_TQ2_0
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def automatic_dispatch(backend):
+    backend.set_decode_kernel(0)
+    backend.set_flow_mfma(0)
+    backend.set_gemm_tiles(0)
+    yield
+    backend.set_decode_kernel(0)
+    backend.set_flow_mfma(0)
+    backend.set_gemm_tiles(0)
+    backend.set_stream_min_groups(backend.info.compute_units)
+
+
+def _planes(rng, n, k, planes):
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)[:planes]]
+    scs = [scales(rng, n) for _ in range(planes)]
+    packed = [T.pack_rows(w, n, k) for w in ws]
+    return ws, scs, packed
+
+
+@pytest.mark.parametrize("tiles", [2, 4])
+@pytest.mark.parametrize("m,n,k", [(65, 8, 256), (130, 257, 512), (200, 129, 300), (128, 1040, 2560), (300, 2100, 768)])
+def test_one_plane_prefill_kernel_both_tile_counts(backend, oracle, tiles, m, n, k):
+    """tk_gemm32_kernel<1,2,false> and <1,4,false>: ragged tile counts (partial workgroups, partial
+    pairs), several row blocks, every output type."""
+    print("case gemm-tiles", tiles, m, n, k, flush=True)
+    backend.set_gemm_tiles(tiles)
+    rng = np.random.default_rng(tiles * 1000 + m + n + k)
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[m // 2] = 0.0
+    dact = backend.to_device(act, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    dout = backend.empty(m * n, "f32")
+    backend.linear_a8(layer, dact, m, dout)
+    assert same_bits(dout.to_host(), want)
+    dob = backend.empty(m * n, "bf16")
+    backend.linear_a8(layer, dact, m, dob)
+    assert (dob.to_host() == f32_to_bf16_bits(want).reshape(-1)).all()
+    # raw accumulators (the int32 the CPU's integer kernel holds before its two multiplies)
+    q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    dq, dacc = backend.to_device(q, "i8"), backend.empty(m * n, "i32")
+    backend.linear_i8(layer, dq, None, m, dacc)
+    assert (dacc.to_host().reshape(m, n) == oracle.int8_accumulators(packed[0], FMT_TQ2_0, q, m, n, k)).all()
+    # the float contract through the same instantiation
+    mf = min(m, 40)
+    dof = backend.empty(mf * n, "f32")
+    backend.linear_float(layer, dact, mf, dof)
+    got = dof.to_host().reshape(mf, n)
+    rc, wantf = oracle.cpu_mpgemm(packed[0], FMT_TQ2_0, act[:mf], scs[0], mf, n, k)
+    assert rc == 0 and accepts(got, wantf, rel=1e-4, floor=1.0).all()
+    for a in (dact, dout, dob, dq, dacc, dof):
+        a.free()
+    layer.free()
+
+
+@pytest.mark.parametrize("planes,tiles", [(1, 2), (1, 4), (2, 0), (3, 0)])
+def test_grouped_prefill_kernel_every_plane_count(backend, oracle, planes, tiles):
+    """A grouped decode launch whose operand rows exceed LDS runs the prefill kernel from a problem
+    table: tk_gemm32_kernel<1,2,true>, <1,4,true>, <2,2,true>, <3,2,true>. Members of different widths
+    (ragged tile counts), two sharing an activation; one member short enough for the flow kernel's
+    share of the group. Bits equal the single launches and the CPU composition."""
+    print("case grouped-prefill", planes, tiles, flush=True)
+    backend.set_gemm_tiles(tiles)
+    rng = np.random.default_rng(planes * 10 + tiles)
+    m, k_long, k_short = 40, 4500, 768  # 40 rows x 18 K blocks = 184 KiB of operand rows: beyond LDS
+    acts = {"a": rng.standard_normal((m, k_long)).astype(np.float32),
+            "b": rng.standard_normal((m, k_long)).astype(np.float32),
+            "c": rng.standard_normal((m, k_short)).astype(np.float32)}
+    dev = {key: backend.to_device(v, "f32") for key, v in acts.items()}
+    members, checks = [], []
+    for n, key in ((136, "a"), (200, "c"), (72, "a"), (1050, "b"), (48, "c")):
+        k = acts[key].shape[1]
+        ws, scs, packed = _planes(rng, n, k, planes)
+        layer = backend.linear(packed, scs, n, k)
+        out_g, out_s = backend.empty(m * n, "f32"), backend.empty(m * n, "f32")
+        members.append((layer, dev[key], m, out_g))
+        checks.append((layer, dev[key], out_g, out_s, packed, scs, acts[key], n, k))
+    grp = backend.group(members, 1, "f32", "f32")
+    grp.launch()
+    grp.launch()
+    for layer, src, out_g, out_s, packed, scs, act, n, k in checks:
+        backend.linear_a8(layer, src, m, out_s)
+        got = out_g.to_host()
+        assert same_bits(got, out_s.to_host())
+        assert same_bits(got, oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+    grp.destroy()
+    for layer, _, out_g, out_s, *_ in checks:
+        out_g.free()
+        out_s.free()
+        layer.free()
+    for d in dev.values():
+        d.free()
+
+
+@pytest.mark.parametrize("mode,m,planes", [(1, 28, 2), (1, 32, 1), (0, 8, 2), (0, 7, 1)])
+def test_grouped_flow_kernel_wide_form_chosen_automatically(backend, oracle, mode, m, planes):
+    """25..32 operand rows that take at most 64 KiB of LDS: the flow kernel picks the 32x32x32 matrix
+    instruction by itself (tk_flow32_kernel<P,1,*,true> from a problem table: the headline's batch 8 is
+    8 tokens x 4 digit rows x 2 planes). The group is made wide enough for the flow kernel by lowering
+    the workgroup threshold, not by forcing a kernel. Forced onto the 16x16x64 form it gives the same
+    bits."""
+    print("case grouped-flow32", mode, m, planes, flush=True)
+    backend.set_stream_min_groups(1)
+    rng = np.random.default_rng(mode * 100 + m + planes)
+    k = 2048
+    act_a = rng.standard_normal((m, k)).astype(np.float32)
+    act_b = rng.standard_normal((m, k)).astype(np.float32)
+    da, db = backend.to_device(f32_to_bf16_bits(act_a), "bf16"), backend.to_device(f32_to_bf16_bits(act_b), "bf16")
+    act_a = bf16_bits_to_f32(f32_to_bf16_bits(act_a)).reshape(m, k)
+    act_b = bf16_bits_to_f32(f32_to_bf16_bits(act_b)).reshape(m, k)
+    members, checks = [], []
+    for n, src, act in ((520, da, act_a), (136, db, act_b), (1029, da, act_a)):
+        ws, scs, packed = _planes(rng, n, k, planes)
+        layer = backend.linear(packed, scs, n, k)
+        out_g, out_s = backend.empty(m * n, "f32"), backend.empty(m * n, "f32")
+        members.append((layer, src, m, out_g))
+        checks.append((layer, src, out_g, out_s, packed, scs, act, n))
+    grp = backend.group(members, mode, "bf16", "f32")
+    grp.launch()
+    grp.launch()
+    backend.set_flow_mfma(16)
+    grp16 = backend.group([(l, s, m, o) for (l, s, _, o, *_r) in checks], mode, "bf16", "f32")
+    for layer, src, out_g, out_s, packed, scs, act, n in checks:
+        got = out_g.to_host()
+        if mode == 1:
+            assert same_bits(got, oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+        else:
+            want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+            assert rel_err(got.reshape(m, n), want) <= 1e-3
+            assert accepts(got.reshape(m, n), want, rel=1e-4, floor=1.0).all()
+    grp16.launch()
+    for layer, src, out_g, out_s, *_ in checks:
+        assert same_bits(out_g.to_host(), out_s.to_host())  # out_s: the 16x16x64 form's result
+    grp.destroy()
+    grp16.destroy()
+    for layer, _, out_g, out_s, *_ in checks:
+        out_g.free()
+        out_s.free()
+        layer.free()
+    da.free()
+    db.free()
+
+
+def test_gemm_tiles_knob_rejects_other_values(backend):
+    for bad in (1, 3, 8, -2):
+        with pytest.raises(T.InvalidInput):
+            backend.set_gemm_tiles(bad)

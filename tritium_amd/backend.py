@@ -504,6 +504,10 @@ class Mi355xBackend:
     def set_flow_mfma(self, rows):
         _check(self._lib.tk_set_flow_mfma(self._ctx, rows))
 
+    def set_gemm_tiles(self, tiles):
+        """0 automatic, 2 or 4 output tiles per wave of the one-plane prefill kernel."""
+        _check(self._lib.tk_set_gemm_tiles(self._ctx, tiles))
+
     def set_stream_min_groups(self, groups):
         _check(self._lib.tk_set_stream_min_groups(self._ctx, groups))
 

@@ -75,6 +75,7 @@ struct tk_ctx {
   int flow_run_tiles = 0;  // 0 = automatic
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
+  int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum;
   int *d_invalid = nullptr;
@@ -284,6 +285,15 @@ extern "C" int tk_set_flow_mfma(tk_ctx *ctx, int rows) {
     return tk_fail(TK_ERR_INVALID_INPUT, "flow_mfma=%d - use 0 (automatic), 16 or 32", rows);
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->flow_mfma = rows;
+  return TK_OK;
+}
+
+extern "C" int tk_set_gemm_tiles(tk_ctx *ctx, int tiles) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_tiles: null context");
+  if (tiles != 0 && tiles != 2 && tiles != 4)
+    return tk_fail(TK_ERR_INVALID_INPUT, "gemm_tiles=%d - use 0 (automatic), 2 or 4", tiles);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->gemm_tiles = tiles;
   return TK_OK;
 }
 
@@ -594,7 +604,7 @@ static bool prefer_stream(const tk_ctx *ctx, unsigned groups);
 // quantization, K=2560 N=6912: 64..256 tokens 25 -> 18-19 us, 512: 26.5 -> 23.6, 768: 33.2 -> 28.8,
 // 2048 (864 workgroups): 59.8 -> 58.5; from 1088 workgroups on the 4-tile form wins (1024 x 5120 ->
 // 17408: 100 vs 104 us; 4096 x 5120 -> 17408: 314 vs 362 us).
-static void plan_gemm(Plan *pl, unsigned fill = 0) {
+static void plan_gemm(Plan *pl, unsigned fill = 0, int force_nt = 0) {
   TkProblem &pr = pl->pr;
   const size_t R = (size_t)pr.R;
   // The GEMM reads, per K block, 16 segments of the operand rows that are exactly rs*16 bytes apart,
@@ -606,7 +616,8 @@ static void plan_gemm(Plan *pl, unsigned fill = 0) {
   pl->grid_m = (unsigned)((R + 63) / 64);
   unsigned per_wg = (unsigned)tk_gemm_tiles_per_wg(pr.planes);
   pl->cfg.gemm_nt = 0;
-  if (fill && pr.planes == 1 && pl->grid_m * (((unsigned)pr.n_tiles + per_wg - 1) / per_wg) < fill) {
+  const bool few = fill && pl->grid_m * (((unsigned)pr.n_tiles + per_wg - 1) / per_wg) < fill;
+  if (pr.planes == 1 && (force_nt == 2 || (force_nt == 0 && few))) {
     per_wg /= 2;
     pl->cfg.gemm_nt = 2;
   }
@@ -674,7 +685,7 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
     pl->flow_lds = nb * 256 * R;
     pl->flow_ok = pl->flow_lds <= kLdsFlowMax;
   } else {
-    plan_gemm(pl, 4u * (unsigned)ctx->info.compute_units);
+    plan_gemm(pl, 4u * (unsigned)ctx->info.compute_units, ctx->gemm_tiles);
   }
 }
 
@@ -771,7 +782,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     // vs 31 us; 24 rows 26 vs 31; 32 x 8192 -> 8192 x 2 planes: 40 vs 45; 17 x 17408 -> 5120: 55 vs 65).
     if (ctx->decode_force == DECODE_AUTO && !pl.flow_ok && (R > 32 || (R > 16 && pl.pr.n_tiles >= 1024))) {
       pl.skinny = false;
-      plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units);
+      plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units, ctx->gemm_tiles);
     }
   }
   Workspace ws;
@@ -1433,7 +1444,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
         plan_gemm(&tmp);
         total += 8u * (unsigned)tmp.pr.sub_m * (unsigned)tmp.pr.sub_n;
       }
-      gemm_nt2 = total < 4u * (unsigned)ctx->info.compute_units;
+      gemm_nt2 = ctx->gemm_tiles == 2 || (ctx->gemm_tiles == 0 && total < 4u * (unsigned)ctx->info.compute_units);
     }
     group_gemm_nt = gemm_nt2 ? 2 : 0;
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
@@ -1461,7 +1472,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
         }
         continue;
       }
-      plan_gemm(&plans[i], gemm_nt2 ? ~0u : 0u);
+      plan_gemm(&plans[i], 0u, gemm_nt2 ? 2 : 4);
       const unsigned gi = 8u * (unsigned)plans[i].pr.sub_m * (unsigned)plans[i].pr.sub_n;
       plans[i].pr.group_begin = (int)groups_total;
       for (unsigned j = 0; j < gi; ++j) wg_prob.push_back((int)i);
