@@ -247,7 +247,19 @@ int tk_act_quant_i8(tk_ctx *ctx, const void *act, int act_dtype, size_t m, size_
                     float *act_scale, uint32_t *nonfinite_rows);
 
 /* Float-activation linear (BASELINE configs 1 and 2): act [m,k] f32 or bf16,
- * out[m,n] = Σ_p scales_p[n] · Σ_k act[m,k]·trit_p[n,k], f32 accumulate, out f32 or bf16. */
+ * out[m,n] = Σ_p scales_p[n] · Σ_k act[m,k]·trit_p[n,k], out f32 or bf16.
+ * Accuracy. A token is contracted exactly on a 31-bit fixed-point grid of spacing 2^(E-30),
+ * 2^(E-1) <= max|act[m,:]| < 2^E. With D the exact dot product of an output of one plane,
+ *     |value - D| <= n_poor · 2^(E-31) + 1.5 ulp(value),
+ * n_poor = the non-zero elements under the output's non-zero trits that neither lie on the grid
+ * exactly (as int8-valued activations and most of a bf16 token do) nor reach 2^(E-15) in magnitude.
+ * The reference's k-ordered f32 fold (crates/tritium-core/src/reference.rs:42-51) is itself only within
+ * ~sqrt(K)·2^-24·|partial sums| of D; on ordinary tokens the two agree to ~1e-6 of the largest output.
+ * A zero trit makes the fold skip an activation, so an output can miss a token's largest elements and be
+ * small next to its maximum. Tokens where that would show -- the rounding noise n_poor·2^(2E-62)/3 of the
+ * token exceeds 2^-30 of the energy left without its 96 largest elements, e.g. one activation 2^15 or more
+ * times the rest -- and tokens holding NaN or Inf are computed in the reference's own order instead
+ * (bit-identical to the CPU backend, and slow: one sequential walk over K per output). */
 int tk_linear_float(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
                     size_t m, void *out, int out_dtype);
 

@@ -61,7 +61,8 @@ def test_mfma_float_path_on_conformance_sets(backend, oracle):
         epilogue plus the fixed-point grid (K·max|a|·2^-30 per output before the channel scale).
     On other seeds a handful of near-zero outputs differ from the CPU's k-order f32 fold by a little
     more than 1e-4: that is the fold's own rounding (crates/tritium-cpu/src/kernel.rs:686-693 says the
-    same of any wider reduction), which the float64 check makes visible."""
+    same of any wider reduction). Every such output must be closer to the float64 value than the fold
+    is: then no output is off by more than the reference is itself."""
     backend.set_exact_max_macs(0)
     try:
         misses = total = 0
@@ -81,7 +82,9 @@ def test_mfma_float_path_on_conformance_sets(backend, oracle):
                 gamma = np.abs(a).max(axis=1)[:, None]
                 bound = 3 * 2.0 ** -24 * np.abs(exact) + k * gamma * 2.0 ** -30 * v["scales"][None, :] + 1e-30
                 assert (np.abs(out.reshape(m, n) - exact) <= bound).all(), (seed, v["id"])
-        print(f"outputs beyond 1e-4 of the f32 fold: {misses} of {total}")
+                closer = np.abs(out.reshape(m, n) - exact) <= np.abs(want.reshape(m, n) - exact)
+                assert (ok4.reshape(m, n) | closer).all(), (seed, v["id"])
+        print(f"outputs beyond 1e-4 of the f32 fold, all of them closer to the exact value than the fold: {misses} of {total}")
         assert misses <= total * 1e-3
     finally:
         backend.set_exact_max_macs(1 << 20)

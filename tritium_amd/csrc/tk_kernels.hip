@@ -1981,18 +1981,20 @@ __device__ void block_max_any(float &v, int &flag, float *sh, int *shi) {
   __syncthreads();
 }
 
-// Four block sums at once (the four digit rows of a token); sh4 holds 16 ints.
-__device__ void block_sum4(int (&v)[4], int *sh4) {
+// NV block sums at once (the four digit rows of a token, and its two element counts); sh holds
+// 4 * NV ints.
+template <int NV>
+__device__ void block_sums(int (&v)[NV], int *sh) {
 #pragma unroll
-  for (int d = 0; d < 4; ++d)
+  for (int d = 0; d < NV; ++d)
     for (int o = 32; o > 0; o >>= 1) v[d] += __shfl_xor(v[d], o);
   if ((threadIdx.x & 63) == 0) {
 #pragma unroll
-    for (int d = 0; d < 4; ++d) sh4[(threadIdx.x >> 6) * 4 + d] = v[d];
+    for (int d = 0; d < NV; ++d) sh[(threadIdx.x >> 6) * NV + d] = v[d];
   }
   __syncthreads();
 #pragma unroll
-  for (int d = 0; d < 4; ++d) v[d] = sh4[d] + sh4[4 + d] + sh4[8 + d] + sh4[12 + d];
+  for (int d = 0; d < NV; ++d) v[d] = sh[d] + sh[NV + d] + sh[2 * NV + d] + sh[3 * NV + d];
   __syncthreads();
 }
 
@@ -2295,10 +2297,25 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
 // Float token -> four balanced base-256 digit rows of round(a * 2^(30-E)), 2^(E-1) <= max|a| < 2^E.
 // Scaling a float by a power of two is exact, so the rounding to an integer happens once, in
 // single precision.
+//
+// Dynamic range. The grid is 2^(E-30) wide against the token's own maximum. An element that lies on
+// the grid exactly, or is at least 2^(E-15) in magnitude (rounding error at most 2^-16 of itself), is
+// carried faithfully; any other ("poor") element is rounded by up to 2^(E-31), which can be all of
+// it. The reference's k-ordered f32 fold skips an activation under a zero trit
+// (crates/tritium-core/src/reference.rs:42-51), so an output can miss the largest elements of a token
+// and consist of small ones only: its value is then small next to the token's maximum, and the
+// rounding of the poor elements shows. The prep therefore compares the rounding noise of a token,
+// n_poor * 2^(2(E-31)) / 3, with the energy that is left when its TK_DIGITS_TRIM largest elements
+// are all skipped (a lower bound from counts per 4-bit magnitude band below 2^E): where the noise
+// exceeds 2^-30 of that energy (2^-15 in amplitude, i.e. 3e-5 of a typical output that misses the
+// top elements), the token is flagged like one holding NaN or Inf and its outputs are computed in
+// the reference's order. For every other token and every output, unconditionally,
+//   |value - exact dot product| <= n * 2^(E-31)  (+ 1.5 ulp),  n = poor elements under its non-zero trits.
+#define TK_DIGITS_TRIM 96
 __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                                int nprep, int uniform_m) {
   __shared__ float shf[4];
-  __shared__ int shi[16];
+  __shared__ int shi[52];
   int rowi;
   const TkPrep &pp = find_prep(single, table, nprep, uniform_m, rowi);
   const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
@@ -2320,7 +2337,9 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
   if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
   const int shift = 30 - E;
   const bool live = gamma != 0.0f && !nonfinite;
-  int sums[4] = {0, 0, 0, 0};
+  int sums[13] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};  // four digit-row sums, poor elements, eight band counts
+  int &n_poor = sums[4];
+  unsigned long long bands_lo = 0, bands_hi = 0;  // 16-bit counters of bands 0..3 and 4..7
   // split the 16 values of piece pc into their four digit rows and store those in operand order
   auto emit = [&](size_t pc, const float (&v)[16]) {
     const size_t kb = pc >> 4;
@@ -2334,7 +2353,16 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         int q = 0;
-        if (live && e + b < k) q = __float2int_rn(ldexpf(v[sl * 4 + b], shift));  // |q| <= 2^30
+        if (live && e + b < k) {
+          const float r = ldexpf(v[sl * 4 + b], shift);
+          q = __float2int_rn(r);  // |q| <= 2^30
+          n_poor += (fabsf(r) >= 32768.0f || r == (float)q) ? 0 : 1;
+          // band b: 2^(30-4b-4) <= |r| < 2^(30-4b); below 2^-2 (and zero) none
+          const int band = (156 - (int)((__float_as_uint(r) >> 23) & 0xFFu)) >> 2;
+          const unsigned long long one = 1ull << (16 * (band & 3));
+          bands_lo += band < 4 ? one : 0ull;
+          bands_hi += (band >= 4 && band < 8) ? one : 0ull;
+        }
 #pragma unroll
         for (int dg = 0; dg < 4; ++dg) {
           int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
@@ -2382,14 +2410,32 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
       emit(pc, v);
     }
   }
-  block_sum4(sums, shi);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    sums[5 + b] = (int)((bands_lo >> (16 * b)) & 0xFFFFu);
+    sums[9 + b] = (int)((bands_hi >> (16 * b)) & 0xFFFFu);
+  }
+  block_sums<13>(sums, shi);
   if (threadIdx.x < 4) {
     const int t = threadIdx.x;
     pp.rowsum[tok * 4 + t] = t == 0 ? sums[0] : t == 1 ? sums[1] : t == 2 ? sums[2] : sums[3];
   }
   if (threadIdx.x == 0) {
+    // energy left without the TK_DIGITS_TRIM largest elements, in units of 2^(2E): band b counts at
+    // its lower edge 2^(-4b-4); the grid does not carry the token when n_poor * 2^-62 / 3 exceeds
+    // 2^-30 of it
+    float left = 0.0f, edge2 = 0.00390625f;  // 2^-8
+    int trim = TK_DIGITS_TRIM;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int c = sums[5 + b], cut = c < trim ? c : trim;
+      trim -= cut;
+      left += (float)(c - cut) * edge2;
+      edge2 *= 0.00390625f;
+    }
+    const bool narrow = sums[4] > 0 && (float)sums[4] > 3.0f * 4294967296.0f * left;
     pp.exps[tok] = -shift;
-    pp.flags[tok] = nonfinite ? 1u : 0u;
+    pp.flags[tok] = (nonfinite || narrow) ? 1u : 0u;
   }
 }
 
