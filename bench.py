@@ -63,6 +63,46 @@ def algorithmic_bytes(m, n, k, planes, act_bytes, out_bytes, a8=False):
 PREWARM_S = 0.25  # untimed: the clock governor needs some tens of milliseconds of load to settle
 
 
+def bf16_to_f32(bits):
+    return (np.ascontiguousarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def check_a8(name, got_bits_or_f32, ws, scs, act, out_dtype):
+    """Every leg that reports a W1.58A8 number checks sampled tokens of one member against the exact
+    composition, computed here with numpy alone: per-token absmax int8 quantization (one f32 divide
+    127/gamma, one multiply, ties to even), integer contraction (f32 BLAS on integers below 2^24 is
+    exact), ((float)acc * s_w[n]) summed over planes in order, times the per-token scale. The contract
+    is bit-exact, so any difference stops the benchmark."""
+    act = np.ascontiguousarray(act, np.float32)
+    gamma = np.abs(act).max(axis=1, keepdims=True)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        s = np.where(gamma > 0, np.float32(127.0) / gamma, np.float32(0.0)).astype(np.float32)
+    q = np.clip(np.rint(act * s), -128, 127).astype(np.float32)
+    scale = (gamma / np.float32(127.0)).astype(np.float32)
+    out = None
+    for w, sc in zip(ws, scs):
+        t = (q @ np.ascontiguousarray(w.T, np.float32)) * np.asarray(sc, np.float32)[None, :]
+        out = t if out is None else out + t
+    want = (out * scale).astype(np.float32)
+    if out_dtype == "bf16":
+        ok = (np.asarray(got_bits_or_f32, np.uint16).reshape(want.shape) == f32_to_bf16_bits(want).reshape(want.shape)).all()
+    else:
+        ok = (np.asarray(got_bits_or_f32, np.float32).reshape(want.shape).view(np.uint32) == want.view(np.uint32)).all()
+    if not ok:
+        sys.exit(f"bench.py: leg `{name}` produced outputs that differ from the exact W1.58A8 composition")
+    return f"{want.shape[0]} token(s) x {want.shape[1]} outputs bit-exact"
+
+
+def check_float(name, got, ws, scs, act):
+    """Float-contract legs: sampled tokens of one member against a float64 evaluation, at the bound the
+    contract states (1e-3 of the largest output; the kernels are normally ~1e-6)."""
+    exact = sum((act.astype(np.float64) @ w.T.astype(np.float64)) * np.asarray(sc, np.float64)[None, :] for w, sc in zip(ws, scs))
+    err = np.abs(np.asarray(got, np.float64).reshape(exact.shape) - exact).max() / max(np.abs(exact).max(), 1e-30)
+    if not err <= 1e-3:
+        sys.exit(f"bench.py: leg `{name}` is off by {err:.3e} of the largest output (bound 1e-3)")
+    return f"{exact.shape[0]} token(s) x {exact.shape[1]} outputs within {err:.1e} of float64"
+
+
 def prewarm(be, fn, seconds=PREWARM_S):
     """Run fn() untimed until `seconds` of wall clock have passed (at least once)."""
     t0 = time.perf_counter()
@@ -75,19 +115,24 @@ def prewarm(be, fn, seconds=PREWARM_S):
 
 def time_steps(be, steps, warmup, step_fn):
     """Untimed: a fixed pre-warm, then W steps. Timed: exactly K steps between two events on the
-    library's stream."""
+    library's stream (`value`). Then the same K steps once more with an event pair around every launch of
+    the decode kernel (`roofline`): event markers between dependent launches cost a few microseconds
+    each, so they stay out of the region `value` is taken from."""
     start, stop = be.event(), be.event()
     prewarm(be, lambda: step_fn(None))
     for _ in range(warmup):
         step_fn(None)
     be.sync()
-    marks = []
     start.record()
     for _ in range(steps):
-        step_fn(marks)
+        step_fn(None)
     stop.record()
     be.sync()
     total_ms = start.elapsed_ms(stop)
+    marks = []
+    for _ in range(steps):
+        step_fn(marks)
+    be.sync()
     kernel_ms = sum(a.elapsed_ms(b) for a, b in marks)
     for a, b in marks:
         a.destroy()
@@ -98,15 +143,23 @@ def time_steps(be, steps, warmup, step_fn):
 def bench_decode(T, be, steps, warmup, rng):
     host = []
     for _ in range(2):  # two distinct host layers, replicated to COPIES distinct device copies
-        planes = [T.pack_rows(ternary(rng, N2, K2, p0), N2, K2) for p0 in (0.4, 0.7)]
+        trits = [ternary(rng, N2, K2, p0) for p0 in (0.4, 0.7)]
+        planes = [T.pack_rows(w, N2, K2) for w in trits]
         scs = [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)]
-        host.append((planes, scs))
-    layers = [be.linear(*host[i % 2], N2, K2) for i in range(COPIES)]
+        host.append((planes, scs, trits))
+    layers = [be.linear(host[i % 2][0], host[i % 2][1], N2, K2) for i in range(COPIES)]
     mmax = max(SWEEP)
-    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((mmax, K2)).astype(np.float32)), "bf16")
-            for _ in range(COPIES)]
+    act_bits = [f32_to_bf16_bits(rng.standard_normal((mmax, K2)).astype(np.float32)) for _ in range(COPIES)]
+    acts = [be.to_device(b, "bf16") for b in act_bits]
     outs = [be.empty(mmax * N2, "f32") for _ in range(COPIES)]
     groups = {m: be.group([(layers[i], acts[i], m, outs[i]) for i in range(COPIES)], 0, "bf16", "f32") for m in SWEEP}
+    verified = {}
+    for m in SWEEP:  # the last copy of every batch size against float64
+        groups[m].launch()
+        be.sync()
+        c = COPIES - 1
+        verified[str(m)] = check_float(f"decode sweep batch {m}", outs[c].to_host()[: m * N2], host[c % 2][2], host[c % 2][1],
+                                       bf16_to_f32(act_bits[c]).reshape(mmax, K2)[:m])
 
     def step(marks):
         for m in SWEEP:
@@ -137,7 +190,8 @@ def bench_decode(T, be, steps, warmup, rng):
         b = be.event().record()
         be.sync()
         ms = a.elapsed_ms(b) / 50
-        per_m[str(m)] = {"GB/s": round(per_launch[m] / ms / 1e6, 1), "us_per_layer": round(ms * 1e3 / COPIES, 3)}
+        per_m[str(m)] = {"kernel_GB/s": round(per_launch[m] / ms / 1e6, 1), "frac_of_hbm_peak": round(per_launch[m] / ms / 1e6 / HBM_PEAK_GBS, 4),
+                         "kernel_us_per_layer": round(ms * 1e3 / COPIES, 3)}
     res = {
         "ms_per_step": total_ms / steps,
         "value": step_bytes * steps / total_ms / 1e6,
@@ -145,6 +199,7 @@ def bench_decode(T, be, steps, warmup, rng):
         "kernel_avg_ms": kernel_ms / launches,
         "bytes_per_launch_avg": step_bytes / len(SWEEP),
         "per_batch": per_m,
+        "verified": verified,
     }
     for g in groups.values():
         g.destroy()
@@ -170,48 +225,86 @@ def bench_prefill(T, be, rng, m, k, n, planes=1, iters=100):
     """Prefill GEMM: bf16 activations quantized per token to int8 (fused prep launch), int8 MFMA with
     int32 accumulation over `planes` additive planes, bf16 output after per-channel x per-token scale."""
     p0s = (0.4, 0.7, 0.85)[:planes]
-    layers = [be.linear([T.pack_rows(ternary(rng, n, k, p0), n, k) for p0 in p0s],
-                        [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in p0s], n, k) for _ in range(2)]
-    act = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32)), "bf16")
+    hostw = []
+    for _ in range(2):
+        hostw.append(([ternary(rng, n, k, p0) for p0 in p0s], [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in p0s]))
+    layers = [be.linear([T.pack_rows(w, n, k) for w in ws], scs, n, k) for ws, scs in hostw]
+    abits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    act = be.to_device(abits, "bf16")
     out = be.empty(m * n, "bf16")
+    be.linear_a8(layers[1], act, m, out)
+    tok = [0, m // 2 + 1, m - 1]
+    verified = check_a8(f"prefill M={m} K={k} N={n}", out.to_host().reshape(m, n)[tok], hostw[1][0], hostw[1][1],
+                        bf16_to_f32(abits).reshape(m, k)[tok], "bf16")
     ms = time_calls(be, lambda i: be.linear_a8(layers[i % 2], act, m, out), iters)
+    # the contraction alone: the same call on already-quantized int8 rows (their re-ordering launch stays in)
+    q = be.to_device(rng.integers(-127, 128, (m, k)).astype(np.int8), "i8")
+    qs = be.to_device(rng.uniform(0.01, 0.05, m).astype(np.float32), "f32")
+    ms_i8 = time_calls(be, lambda i: be.linear_i8(layers[i % 2], q, qs, m, out), iters)
     ops = 2.0 * m * n * k * planes
     for l in layers:
         l.free()
-    act.free()
-    out.free()
+    for x in (act, out, q, qs):
+        x.free()
     return {"workload": f"prefill GEMM M={m} K={k} N={n} {planes} plane(s), bf16 act -> int8 per token -> int32 acc -> bf16",
             "ms_per_call_incl_quant": round(ms, 4), "TOPS": round(ops / ms / 1e9, 1),
-            "frac_of_int8_peak": round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4)}
+            "frac_of_int8_peak": round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4),
+            "int8_input_call": {"ms_per_call": round(ms_i8, 4), "TOPS": round(ops / ms_i8 / 1e9, 1),
+                                "frac_of_int8_peak": round(ops / ms_i8 / 1e9 / INT8_PEAK_TOPS, 4),
+                                "note": "activations already int8 (no absmax pass; the operand re-ordering launch included)"},
+            "verified": verified}
 
 
 def bench_config1(T, be, rng, iters=200):
     """configs[0]: one ternary linear, K=2560 N=6912, one plane, f32 N(0,1) activation, batch 1.
-    Through the adapter call on host slices (upload, kernel, download, sync per call) and through the
-    device-resident call (one launch of prep + decode kernel, back to back)."""
+    (a) the HBM figure: COPIES distinct resident copies of the layer (0.57 GB of codes, above the 256 MB
+        last-level cache) in one grouped launch; kernel alone and the whole step with its digit-split launch;
+    (b) one device-resident call on a single 4.4 MB layer (digit split + decode kernel back to back: cache
+        resident and launch-bound, so a latency figure, not a bandwidth one);
+    (c) the adapter call on host slices (upload, kernels, download, sync per call)."""
     n, k = 6912, 2560
-    w = T.pack_rows(ternary(rng, n, k, 0.4), n, k)
-    sc = rng.uniform(0.01, 0.1, n).astype(np.float32)
-    act = rng.standard_normal((1, k)).astype(np.float32)
-    buf = be.upload_weights(w, T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0)
+    trits = [ternary(rng, n, k, 0.4) for _ in range(2)]
+    packed = [T.pack_rows(w, n, k) for w in trits]
+    scs = [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in range(2)]
+    layers = [be.linear([packed[i % 2]], [scs[i % 2]], n, k) for i in range(COPIES)]
+    act_h = [rng.standard_normal((1, k)).astype(np.float32) for _ in range(COPIES)]
+    acts = [be.to_device(a, "f32") for a in act_h]
+    outs = [be.empty(n, "f32") for _ in range(COPIES)]
+    g = be.group([(layers[i], acts[i], 1, outs[i]) for i in range(COPIES)], 0, "f32", "f32")
+    g.launch()
+    be.sync()
+    c = COPIES - 1
+    verified = check_float("config1 grouped", outs[c].to_host(), [trits[c % 2]], [scs[c % 2]], act_h[c])
+    ms_step = time_calls(be, lambda i: g.launch(), iters)
+    g.launch_parts(True, False)
+    ms_kernel = time_calls(be, lambda i: g.launch_parts(False, True), iters)
+    by = COPIES * algorithmic_bytes(1, n, k, 1, 4, 4)
+    g.destroy()
+    ms_single = time_calls(be, lambda i: be.linear_float(layers[0], acts[0], 1, outs[0]), iters)
+    buf = be.upload_weights(packed[0], T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0)
     out = np.zeros(n, np.float32)
-    call = T.MpGemm(act.reshape(-1), buf, sc, T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0, out)
+    call = T.MpGemm(act_h[0].reshape(-1), buf, scs[0], T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0, out)
     for _ in range(20):
         be.mpgemm(call)
     t0 = time.perf_counter()
     for _ in range(iters):
         be.mpgemm(call)
     host_us = (time.perf_counter() - t0) / iters * 1e6
-    layer = be.linear([w], [sc], n, k)
-    dact, dout = be.to_device(act, "f32"), be.empty(n, "f32")
-    ms = time_calls(be, lambda i: be.linear_float(layer, dact, 1, dout), iters)
-    by = algorithmic_bytes(1, n, k, 1, 4, 4)
-    layer.free()
-    dact.free()
-    dout.free()
-    return {"workload": "K=2560 N=6912 1 plane, f32 activation, batch 1 (a single 4.4 MB layer: launch-bound)",
-            "adapter_call_on_host_slices_us": round(host_us, 1), "device_resident_call_us": round(ms * 1e3, 2),
-            "device_resident_GB/s": round(by / ms / 1e6, 1)}
+    buf.free()
+    for x in acts + outs:
+        x.free()
+    for l in layers:
+        l.free()
+    by1 = algorithmic_bytes(1, n, k, 1, 4, 4)
+    return {"workload": f"K=2560 N=6912 1 plane, f32 activation, batch 1; {COPIES} resident layer copies per grouped launch",
+            "kernel_GB/s": round(by / ms_kernel / 1e6, 1), "kernel_frac_of_hbm_peak": round(by / ms_kernel / 1e6 / HBM_PEAK_GBS, 4),
+            "kernel_us_per_layer": round(ms_kernel * 1e3 / COPIES, 3),
+            "step_GB/s_incl_digit_split": round(by / ms_step / 1e6, 1),
+            "step_frac_of_hbm_peak": round(by / ms_step / 1e6 / HBM_PEAK_GBS, 4),
+            "single_layer_device_resident_call_us": round(ms_single * 1e3, 2),
+            "single_layer_GB/s": round(by1 / ms_single / 1e6, 1),
+            "adapter_call_on_host_slices_us": round(host_us, 1),
+            "verified": verified}
 
 
 def bench_sweep_a8(T, be, rng, iters=100):
@@ -221,74 +314,111 @@ def bench_sweep_a8(T, be, rng, iters=100):
     of the sweep stays in the bandwidth regime. Kernel only, like `per_batch`."""
     host = []
     for _ in range(2):
-        planes = [T.pack_rows(ternary(rng, N2, K2, p0), N2, K2) for p0 in (0.4, 0.7)]
-        host.append((planes, [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)]))
-    layers = [be.linear(*host[i % 2], N2, K2) for i in range(COPIES)]
+        trits = [ternary(rng, N2, K2, p0) for p0 in (0.4, 0.7)]
+        host.append(([T.pack_rows(w, N2, K2) for w in trits], [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(PLANES2)], trits))
+    layers = [be.linear(host[i % 2][0], host[i % 2][1], N2, K2) for i in range(COPIES)]
     mmax = max(SWEEP)
-    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((mmax, K2)).astype(np.float32)), "bf16")
-            for _ in range(COPIES)]
+    act_bits = [f32_to_bf16_bits(rng.standard_normal((mmax, K2)).astype(np.float32)) for _ in range(COPIES)]
+    acts = [be.to_device(b, "bf16") for b in act_bits]
     outs = [be.empty(mmax * N2, "f32") for _ in range(COPIES)]
-    res, tot_b, tot_ms = {}, 0, 0.0
+    res, tot_b, tot_ms, tot_step = {}, 0, 0.0, 0.0
+    c = COPIES - 1
     for m in SWEEP:
         g = be.group([(layers[i], acts[i], m, outs[i]) for i in range(COPIES)], 1, "bf16", "f32")
+        g.launch()
+        be.sync()
+        ver = check_a8(f"int8 sweep batch {m}", outs[c].to_host()[: m * N2], host[c % 2][2], host[c % 2][1],
+                       bf16_to_f32(act_bits[c]).reshape(mmax, K2)[:m], "f32")
+        ms_step = time_calls(be, lambda i: g.launch(), iters)
         g.launch_parts(True, False)
         ms = time_calls(be, lambda i: g.launch_parts(False, True), iters)
         by = COPIES * algorithmic_bytes(m, N2, K2, PLANES2, 2, 4, a8=True)
-        res[str(m)] = {"GB/s": round(by / ms / 1e6, 1), "us_per_layer": round(ms * 1e3 / COPIES, 3)}
+        res[str(m)] = {"kernel_GB/s": round(by / ms / 1e6, 1), "kernel_us_per_layer": round(ms * 1e3 / COPIES, 3),
+                       "step_GB/s_incl_quant": round(by / ms_step / 1e6, 1), "verified": ver}
         tot_b += by
         tot_ms += ms
+        tot_step += ms_step
         g.destroy()
     for x in acts + outs:
         x.free()
     for l in layers:
         l.free()
-    return {"workload": "the headline sweep with per-token int8 activations (W1.58A8), decode kernel only",
-            "per_batch": res, "sweep_GB/s": round(tot_b / tot_ms / 1e6, 1),
-            "frac_of_hbm_peak": round(tot_b / tot_ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return {"workload": "the headline sweep with per-token int8 activations (W1.58A8): decode kernel alone, and the step with its quantization launch",
+            "per_batch": res, "kernel_sweep_GB/s": round(tot_b / tot_ms / 1e6, 1),
+            "kernel_frac_of_hbm_peak": round(tot_b / tot_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "step_sweep_GB/s_incl_quant": round(tot_b / tot_step / 1e6, 1),
+            "step_frac_of_hbm_peak": round(tot_b / tot_step / 1e6 / HBM_PEAK_GBS, 4)}
 
 
 def bench_config5(T, be, rng):
-    """configs[4]: three additive planes (P(0)=0.4/0.7/0.85), hidden 5120, FFN 17408. Decode at batch
-    64 over the up and down projections of 8 distinct layers in one grouped launch (W1.58A8, bf16 in
-    and out), and the 4096-token prefill GEMM of the up projection."""
-    h, f, layers_n, m = 5120, 17408, 8, 64
-    shapes = {"up": (f, h), "down": (h, f)}
-    lins = []
-    for _ in range(layers_n):
-        lins.append({name: be.linear([T.pack_rows(ternary(rng, n, k, p0), n, k) for p0 in (0.4, 0.7, 0.85)],
-                                     [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in range(3)], n, k)
-                     for name, (n, k) in shapes.items()})
-    hid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
-    mid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, f)).astype(np.float32)), "bf16")
+    """configs[4]: 27B-class dense ternary projections, three additive planes (P(0)=0.4/0.7/0.85), hidden
+    5120, FFN 17408, 64 layers. The config does not give the attention shapes; assumed here: 40 query heads
+    and 8 KV heads of 128, i.e. q and o 5120 x 5120, k and v 1024 x 5120 (with gate/up 17408 x 5120 and down
+    5120 x 17408 that is 330 M weights per layer and plane, 15.9 GB of 2-bit codes for the stack).
+    Decode: all 64 layers x 7 projections at batch 64 (W1.58A8, bf16 in and out) on given inputs in ONE
+    grouped launch, quantization included. The layers are 64 distinct device copies of one host set per
+    shape. Prefill: the 4096-token GEMM of the up and of the down projection."""
+    h, f, kvd, layers_n, m = 5120, 17408, 1024, 64, 64
+    shapes = {"q": (h, h), "k": (kvd, h), "v": (kvd, h), "o": (h, h), "gate": (f, h), "up": (f, h), "down": (h, f)}
+    hostw = {}
+    for n, k in sorted(set(shapes.values())):
+        ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)]
+        hostw[(n, k)] = (ws, [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in range(3)], [T.pack_rows(w, n, k) for w in ws])
+    lins = [{name: be.linear(hostw[sh][2], hostw[sh][1], *sh) for name, sh in shapes.items()} for _ in range(layers_n)]
+    srcs_h = {key: f32_to_bf16_bits(rng.standard_normal((m, kk)).astype(np.float32)) for key, kk in (("hid", h), ("att", h), ("mid", f))}
+    srcs = {key: be.to_device(v, "bf16") for key, v in srcs_h.items()}
+    wiring = (("q", "hid"), ("k", "hid"), ("v", "hid"), ("o", "att"), ("gate", "hid"), ("up", "hid"), ("down", "mid"))
     members, outs = [], []
     for L in lins:
-        for name, src in (("up", hid), ("down", mid)):
+        for name, key in wiring:
             o = be.empty(m * shapes[name][0], "bf16")
             outs.append(o)
-            members.append((L[name], src, m, o))
+            members.append((L[name], srcs[key], m, o))
     g = be.group(members, 1, "bf16", "bf16")
-    ms = time_calls(be, lambda i: g.launch(), 30)
+    g.launch()
+    be.sync()
+    verified = {}
+    tok = [0, 33, m - 1]
+    for j, (name, key) in enumerate(wiring):  # the last layer's seven projections
+        idx = (layers_n - 1) * len(wiring) + j
+        n, k = shapes[name]
+        ws, scs, _ = hostw[shapes[name]]
+        verified[name] = check_a8(f"config5 decode {name}", outs[idx].to_host().reshape(m, n)[tok], ws, scs,
+                                  bf16_to_f32(srcs_h[key]).reshape(m, k)[tok], "bf16")
+    ms = time_calls(be, lambda i: g.launch(), 10)
+    g.launch_parts(True, False)
+    ms_k = time_calls(be, lambda i: g.launch_parts(False, True), 10)
     by = layers_n * sum(algorithmic_bytes(m, n, k, 3, 2, 2, a8=True) for n, k in shapes.values())
-    res = {"decode_batch64": {"workload": f"{layers_n} layers x (up, down), 3 planes, batch 64, one grouped launch incl. quantization",
-                              "ms_per_step": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
-                              "frac_of_hbm_peak": round(by / ms / 1e6 / HBM_PEAK_GBS, 4)}}
+    ops = layers_n * sum(2.0 * m * n * k * 3 for n, k in shapes.values())
+    res = {"assumed_attention_shapes": "40 query heads, 8 KV heads of 128: q,o 5120x5120; k,v 1024x5120 (not given by the config)",
+           "decode_batch64": {"workload": f"{layers_n} layers x (q,k,v,o,gate,up,down), 3 planes, batch 64, one grouped launch on given inputs",
+                              "ms_per_step_incl_quant": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+                              "frac_of_hbm_peak": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+                              "tokens_per_s": round(m / ms * 1e3, 1),
+                              "kernels_only": {"ms": round(ms_k, 4), "GB/s": round(by / ms_k / 1e6, 1),
+                                               "frac_of_hbm_peak": round(by / ms_k / 1e6 / HBM_PEAK_GBS, 4),
+                                               "TOPS": round(ops / ms_k / 1e9, 1)},
+                              "code_bytes": int(layers_n * sum(3 * n * ((k + 255) // 256) * 64 for n, k in shapes.values())),
+                              "verified": verified}}
     g.destroy()
     # the same projections as single calls (one linear per launch, quantization included), rotating over
-    # the 8 layers (535 MB of codes per projection kind): rows beyond LDS -> the prefill kernel
+    # the 64 layers: rows beyond LDS -> the prefill kernel
     single = {}
-    for name, src in (("up", hid), ("down", mid)):
+    for name, key in (("q", "hid"), ("k", "hid"), ("up", "hid"), ("down", "mid")):
         n, k = shapes[name]
-        o = outs[0 if name == "up" else 1]
-        ms1 = time_calls(be, lambda i: be.linear_a8(lins[i % layers_n][name], src, m, o), 64)
+        o = outs[[w[0] for w in wiring].index(name)]
+        ms1 = time_calls(be, lambda i: be.linear_a8(lins[i % layers_n][name], srcs[key], m, o), 64)
         by1 = algorithmic_bytes(m, n, k, 3, 2, 2, a8=True)
-        single[name] = {"us_per_call": round(ms1 * 1e3, 1), "GB/s": round(by1 / ms1 / 1e6, 1)}
+        single[name] = {"us_per_call_incl_quant": round(ms1 * 1e3, 1), "GB/s": round(by1 / ms1 / 1e6, 1),
+                        "frac_of_hbm_peak": round(by1 / ms1 / 1e6 / HBM_PEAK_GBS, 4)}
     res["decode_batch64_single_calls"] = dict(single, workload="one projection per call, 3 planes, batch 64, incl. quantization")
-    for x in outs + [hid, mid]:
+    for x in outs + list(srcs.values()):
         x.free()
     for L in lins:
         for l in L.values():
             l.free()
-    res["prefill_4096"] = bench_prefill(T, be, rng, 4096, h, f, planes=3, iters=30)
+    res["prefill_4096_up"] = bench_prefill(T, be, rng, 4096, h, f, planes=3, iters=20)
+    res["prefill_4096_down"] = bench_prefill(T, be, rng, 4096, f, h, planes=3, iters=20)
     return res
 
 
@@ -360,11 +490,12 @@ def bench_stack(T, be, rng, iters=100):
     tokens/s = batch / time of the projection path only."""
     h, f, kv, layers_n = 2560, 6912, 640, 30
     shapes = {"q": (h, h), "k": (kv, h), "v": (kv, h), "o": (h, h), "gate": (f, h), "up": (f, h), "down": (h, f)}
-    hostw = {}
+    hostw, hostt = {}, {}
     for name, (n, k) in shapes.items():
         key = (n, k)
         if key not in hostw:
-            hostw[key] = (T.pack_rows(ternary(rng, n, k, 0.4), n, k), rng.uniform(0.01, 0.1, n).astype(np.float32))
+            hostt[key] = ternary(rng, n, k, 0.4)
+            hostw[key] = (T.pack_rows(hostt[key], n, k), rng.uniform(0.01, 0.1, n).astype(np.float32))
     res = {}
     lins = []
     for _ in range(layers_n):
@@ -372,19 +503,34 @@ def bench_stack(T, be, rng, iters=100):
     code_bytes = layers_n * sum(n * ((k + 255) // 256) * 64 for n, k in shapes.values())
     nw = [[be.to_device(rng.uniform(0.5, 1.5, h).astype(np.float32), "f32") for _ in range(2)] for _ in range(layers_n)]
     for m in (1, 32):
-        hid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
-        att = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, h)).astype(np.float32)), "bf16")
-        mid = be.to_device(f32_to_bf16_bits(rng.standard_normal((m, f)).astype(np.float32)), "bf16")
+        src_h = {key: f32_to_bf16_bits(rng.standard_normal((m, kk)).astype(np.float32)) for key, kk in (("hid", h), ("att", h), ("mid", f))}
+        hid, att, mid = (be.to_device(src_h[key], "bf16") for key in ("hid", "att", "mid"))
+        wiring = (("q", hid, "hid"), ("k", hid, "hid"), ("v", hid, "hid"), ("o", att, "att"), ("gate", hid, "hid"),
+                  ("up", hid, "hid"), ("down", mid, "mid"))
         members, outs = [], []
         for L in lins:
-            for name, src in (("q", hid), ("k", hid), ("v", hid), ("o", att), ("gate", hid), ("up", hid), ("down", mid)):
+            for name, src, _ in wiring:
                 o = be.empty(m * shapes[name][0], "bf16")
                 outs.append(o)
                 members.append((L[name], src, m, o))
         g = be.group(members, 1, "bf16", "bf16")
+        g.launch()
+        be.sync()
+        tok = sorted({0, m // 2, m - 1})
+        ver = {}
+        for j, (name, _, key) in enumerate(wiring):  # the last layer's seven projections
+            n, k = shapes[name]
+            ver[name] = check_a8(f"stack batch {m} {name}", outs[(layers_n - 1) * 7 + j].to_host().reshape(m, n)[tok],
+                                 [hostt[(n, k)]], [hostw[(n, k)][1]], bf16_to_f32(src_h[key]).reshape(m, k)[tok], "bf16")
         ms = time_calls(be, lambda i: g.launch(), iters)
-        res[f"batch{m}"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1),
-                            "code_GB/s": round(code_bytes / ms / 1e6, 1)}
+        g.launch_parts(True, False)
+        ms_k = time_calls(be, lambda i: g.launch_parts(False, True), iters)
+        res[f"batch{m}"] = {"ms_per_step_incl_quant": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1),
+                            "code_GB/s": round(code_bytes / ms / 1e6, 1),
+                            "frac_of_hbm_peak": round(code_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                            "kernels_only_ms": round(ms_k, 4),
+                            "kernels_only_frac_of_hbm_peak": round(code_bytes / ms_k / 1e6 / HBM_PEAK_GBS, 4),
+                            "verified": ver}
         g.destroy()
         # the same step with the attention / FFN RMSNorms fused into the quantization of q,k,v and gate,up
         norms = []
@@ -392,7 +538,7 @@ def bench_stack(T, be, rng, iters=100):
             norms += [(nw[li][0], 1e-5, False)] * 3 + [None] + [(nw[li][1], 1e-5, False)] * 2 + [None]
         g = be.group(members, 1, "bf16", "bf16", norms=norms)
         ms = time_calls(be, lambda i: g.launch(), iters)
-        res[f"batch{m}_rmsnorm_fused"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1)}
+        res[f"batch{m}_rmsnorm_fused"] = {"ms_per_step_incl_norm_and_quant": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1)}
         g.destroy()
         for x in outs + [hid, att, mid]:
             x.free()
@@ -483,6 +629,7 @@ def main():
                      "kernel": "tk_flow_kernel<2,1,1,4> (batch 1-4), tk_flow32_kernel<2,1,4> (batch 8), tk_flow_kernel<2,4,2,2> (batch 16)", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
                      "algorithmic_bytes_per_launch": int(dec["bytes_per_launch_avg"])},
         "per_batch": dec["per_batch"],
+        "verified": dec["verified"],
         "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
                    "clock_mhz": info.clock_khz / 1000, "memory_clock_mhz": info.memory_clock_khz / 1000,
                    "memory_bus_bits": info.memory_bus_bits},

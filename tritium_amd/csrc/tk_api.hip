@@ -539,11 +539,12 @@ static bool flow_wide(const tk_ctx *ctx, int planes, int rt, size_t nb, size_t r
   if (ctx->flow_mfma == 32) return true;
   return rt == 2 && rows > 24 && flow_wide_lds(rt, nb) <= 64 * 1024;
 }
-static int flow_runs_per_wave(bool wide, int planes, int rt) {
-  return wide ? tk_flow32_runs_per_wave() : tk_flow_runs_per_wave(planes, rt);
+static int flow_runs_per_wave(bool wide, int planes, int rt, size_t rows) {
+  return wide ? tk_flow32_runs_per_wave() : tk_flow_runs_per_wave(planes, rt, (int)rows);
 }
-static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds) {
+static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds, size_t rows) {
   cfg->wide_mfma = wide ? 1 : 0;
+  cfg->tw = flow_runs_per_wave(wide, cfg->planes, cfg->rt, rows);
   cfg->lds_bytes = flow_lds + (wide ? kFlowWideExtraLds : 0);
   if (wide && cfg->ring > 4) cfg->ring = 4;
 }
@@ -557,9 +558,9 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds) {
 // operand rows (8-16 KiB staged) are 5-8% faster with runs of ONE tile (64 KiB per workgroup), 16
 // rows stay at 2.
 static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
-                          size_t nb, bool wide) {
+                          size_t nb, bool wide, size_t rows) {
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
-  const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, planes, rt);
+  const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, planes, rt, rows);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
   size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 ? 2 : 4);
   if (target < 64 * 1024) target = 64 * 1024;
@@ -767,8 +768,8 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     wide = pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R);
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
     const int fw = flow_waves(flow_lds);
-    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide);
-    const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt) * (unsigned)run_tiles;
+    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, R);
+    const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
     variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
@@ -833,8 +834,8 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
     cfg.waves = flow_waves(flow_lds);
-    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R);
-    flow_cfg_form(&cfg, wide, flow_lds);
+    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R));
+    flow_cfg_form(&cfg, wide, flow_lds, R);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -1276,6 +1277,7 @@ struct tk_group {
   void *tables = nullptr;    // TkProblem[count], TkPrep[nprep], then int wg_prob[] (streaming form)
   int nprobs = 0, nprep = 0, prep_kind = 0;
   int prep_uniform_m = 0;    // > 0: prep entry j starts at token j * prep_uniform_m
+  int prep_wave_pieces = 0;  // > 0: every entry fits the one-wave-per-token prep kernels; the largest piece count
   unsigned prep_rows = 0;
   int variant = 1;
   size_t wg_prob_off = 0;
@@ -1395,13 +1397,13 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   const bool wide = flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
   if (wide) flds = flow_wide_lds(rt, nb_max);
   const int fw = flow_waves(flds);
-  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide);
+  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, rows_max);
   {
     std::vector<unsigned> member_tiles(count);
     for (size_t i = 0; i < count; ++i) member_tiles[i] = (unsigned)plans[i].pr.n_tiles;
-    run_tiles = trim_run_tiles(ctx, run_tiles, (size_t)fw * (size_t)flow_runs_per_wave(wide, planes, rt), member_tiles);
+    run_tiles = trim_run_tiles(ctx, run_tiles, (size_t)fw * (size_t)flow_runs_per_wave(wide, planes, rt, rows_max), member_tiles);
   }
-  const unsigned fper = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, planes, rt) * (unsigned)run_tiles;
+  const unsigned fper = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, planes, rt, rows_max) * (unsigned)run_tiles;
   unsigned fgroups = 0;
   for (size_t i = 0; i < count; ++i) {
     sgroups += ((unsigned)plans[i].pr.n_tiles + tpw - 1) / tpw;
@@ -1450,14 +1452,14 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds);
-    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide) : 1;
+    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, prows_max) : 1;
     {
       std::vector<unsigned> member_tiles;
       for (size_t i = 0; i < count; ++i)
         if (plans[i].flow_ok) member_tiles.push_back((unsigned)plans[i].pr.n_tiles);
-      prun = trim_run_tiles(ctx, prun, (size_t)pfw * (size_t)flow_runs_per_wave(pwide, planes, rt), member_tiles);
+      prun = trim_run_tiles(ctx, prun, (size_t)pfw * (size_t)flow_runs_per_wave(pwide, planes, rt, prows_max), member_tiles);
     }
-    const unsigned pper = (unsigned)pfw * (unsigned)flow_runs_per_wave(pwide, planes, rt) * (unsigned)prun;
+    const unsigned pper = (unsigned)pfw * (unsigned)flow_runs_per_wave(pwide, planes, rt, prows_max) * (unsigned)prun;
     unsigned flow_total = 0;
     for (size_t i = 0; i < count; ++i) {
       if (plans[i].flow_ok) {
@@ -1485,8 +1487,8 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.lds_bytes = pflds;
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
-      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max);
-      flow_cfg_form(&flow_cfg, pwide, pflds);
+      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, planes, rt, prows_max));
+      flow_cfg_form(&flow_cfg, pwide, pflds, prows_max);
     }
   } else if (variant != DECODE_KSPLIT) {
     const unsigned per = variant == DECODE_FLOW ? fper : tpw;
@@ -1574,6 +1576,16 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     if (preps[j].m != preps[0].m || preps[j].row_begin != (int)j * preps[0].m) g->prep_uniform_m = 0;
   g->prep_kind = prep_kind;
   g->prep_rows = rows;
+  g->prep_wave_pieces = 0;
+  {
+    size_t pieces = 0;
+    bool ok = true;
+    for (const TkPrep &pp : preps) {
+      ok = ok && pp.nb * 16 <= 256 && !pp.norm_kind && !pp.blocksum;
+      if (pp.nb * 16 > pieces) pieces = pp.nb * 16;
+    }
+    if (ok) g->prep_wave_pieces = (int)pieces;
+  }
   g->cfg.planes = planes;
   g->cfg.rt = rt;
   g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
@@ -1588,9 +1600,9 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       nbs[i] = plans[i].pr.nb;
       wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
     }
-    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max);
+    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, planes, rt, rows_max));
   }
-  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds);
+  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds, rows_max);
   *out = g;
   return TK_OK;
 }
@@ -1601,7 +1613,9 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   HIPCHK(hipSetDevice(ctx->device));
   const TkProblem *probs = (const TkProblem *)g->tables;
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
-  if (do_prep) HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows));
+  if (do_prep)
+    HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows,
+                          g->prep_wave_pieces));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
   if (do_main && g->has_flow_part)
     HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),

@@ -88,6 +88,7 @@ struct TkLaunchCfg {
   int ring;     // flow kernel: positions in the prefetch ring (2..5)
   int wide_mfma; // flow kernel: 32x32x32 form (17..64 operand rows, row constants in LDS)
   int gemm_nt;  // prefill kernel, one plane: tiles per wave (0 = the default 4, or 2)
+  int tw;       // flow kernel, 16x16x64 form: runs per wave (tk_flow_runs_per_wave)
 };
 
 #ifdef __cplusplus
@@ -100,20 +101,22 @@ hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *co
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
                                   int8_t *trits);
 // uniform_m > 0 says that entry j of the table starts at token j * uniform_m (all tensors equally long).
+// table_wave_pieces: for a table, the largest piece count (16 * K blocks) of its entries when every entry can
+// take the one-wave-per-token kernels (at most 256 pieces, no norm, no per-block sums), else 0.
 hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
-                          unsigned rows);
+                          unsigned rows, int table_wave_pieces = 0);
 hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
                             const TkLaunchCfg &cfg);
 // streaming decode kernel: tiles per workgroup for a (planes, rt) pair, and the launcher
 int tk_stream_tiles_per_wg(int planes, int rt);
 hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                             const TkLaunchCfg &cfg);
-int tk_flow_runs_per_wave(int planes, int rt);
+int tk_flow_runs_per_wave(int planes, int rt, int rows);
 hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
 int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
-int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows);
+int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows, int tw);
 int tk_flow32_runs_per_wave(void);
 // block-scale planes (float activations): flow form for <= 64 operand rows resident in LDS, and the
 // reference-order kernel for everything else

@@ -16,6 +16,8 @@
 //
 // Compiled with -ffp-contract=off: the epilogue multiplies must round exactly as the CPU's do.
 
+#include <cstdlib>
+
 #include "tk_internal.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -2294,6 +2296,39 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
   }
 }
 
+// An element scaled onto the grid (r = a * 2^(30-E), q = its rounding) is carried faithfully when it
+// lies on the grid or its rounding error is at most 2^-16 of it.
+__device__ __forceinline__ bool digit_poor(float r, int q) { return !(fabsf(r) >= 32768.0f || r == (float)q); }
+
+// Counts of the elements of one piece per magnitude band: band b holds 2^(30-4b-4) <= |r| < 2^(30-4b);
+// elements below the eighth band (and zeros) are not counted.
+__device__ __forceinline__ void count_bands(const float (&v)[16], int shift, int (&bands)[8]) {
+#pragma unroll
+  for (int x = 0; x < 16; ++x) {
+    const float r = ldexpf(v[x], shift);
+    const int band = (156 - (int)((__float_as_uint(r) >> 23) & 0xFFu)) >> 2;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) bands[b] += band == b ? 1 : 0;
+  }
+}
+
+#define TK_DIGITS_TRIM 96
+// Energy left without the TK_DIGITS_TRIM largest elements, in units of 2^(2E): band b counts at its
+// lower edge 2^(-4b-4). The grid does not carry the token when its rounding noise n_poor * 2^-62 / 3
+// exceeds 2^-30 of that.
+__device__ __forceinline__ bool digits_narrow(int n_poor, const int (&bands)[8]) {
+  float left = 0.0f, edge2 = 0.00390625f;  // 2^-8
+  int trim = TK_DIGITS_TRIM;
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+    const int c = bands[b], cut = c < trim ? c : trim;
+    trim -= cut;
+    left += (float)(c - cut) * edge2;
+    edge2 *= 0.00390625f;
+  }
+  return n_poor > 0 && (float)n_poor > 3.0f * 4294967296.0f * left;
+}
+
 // Float token -> four balanced base-256 digit rows of round(a * 2^(30-E)), 2^(E-1) <= max|a| < 2^E.
 // Scaling a float by a power of two is exact, so the rounding to an integer happens once, in
 // single precision.
@@ -2311,11 +2346,10 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_kernel(TkPrep single, const 
 // top elements), the token is flagged like one holding NaN or Inf and its outputs are computed in
 // the reference's order. For every other token and every output, unconditionally,
 //   |value - exact dot product| <= n * 2^(E-31)  (+ 1.5 ulp),  n = poor elements under its non-zero trits.
-#define TK_DIGITS_TRIM 96
 __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                                int nprep, int uniform_m) {
   __shared__ float shf[4];
-  __shared__ int shi[52];
+  __shared__ int shi[32];
   int rowi;
   const TkPrep &pp = find_prep(single, table, nprep, uniform_m, rowi);
   const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
@@ -2337,9 +2371,8 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
   if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
   const int shift = 30 - E;
   const bool live = gamma != 0.0f && !nonfinite;
-  int sums[13] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};  // four digit-row sums, poor elements, eight band counts
+  int sums[5] = {0, 0, 0, 0, 0};  // four digit-row sums, poor elements
   int &n_poor = sums[4];
-  unsigned long long bands_lo = 0, bands_hi = 0;  // 16-bit counters of bands 0..3 and 4..7
   // split the 16 values of piece pc into their four digit rows and store those in operand order
   auto emit = [&](size_t pc, const float (&v)[16]) {
     const size_t kb = pc >> 4;
@@ -2356,12 +2389,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
         if (live && e + b < k) {
           const float r = ldexpf(v[sl * 4 + b], shift);
           q = __float2int_rn(r);  // |q| <= 2^30
-          n_poor += (fabsf(r) >= 32768.0f || r == (float)q) ? 0 : 1;
-          // band b: 2^(30-4b-4) <= |r| < 2^(30-4b); below 2^-2 (and zero) none
-          const int band = (156 - (int)((__float_as_uint(r) >> 23) & 0xFFu)) >> 2;
-          const unsigned long long one = 1ull << (16 * (band & 3));
-          bands_lo += band < 4 ? one : 0ull;
-          bands_hi += (band >= 4 && band < 8) ? one : 0ull;
+          n_poor += digit_poor(r, q) ? 1 : 0;
         }
 #pragma unroll
         for (int dg = 0; dg < 4; ++dg) {
@@ -2410,30 +2438,249 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
       emit(pc, v);
     }
   }
+  block_sums<5>(sums, shi);
+  // Only a token that has poor elements needs the magnitude bands (the same answer in every thread, so
+  // the barriers inside are reached by all or by none).
+  bool narrow = false;
+  if (sums[4] > 0) {
+    int bands[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (resident) {
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    sums[5 + b] = (int)((bands_lo >> (16 * b)) & 0xFFFFu);
-    sums[9 + b] = (int)((bands_hi >> (16 * b)) & 0xFFFFu);
+      for (int it = 0; it < TK_PREP_HELD; ++it) {
+        const size_t pc = (size_t)threadIdx.x + (size_t)it * TK_WG;
+        if (pc < npieces) count_bands(held[it], shift, bands);
+      }
+    } else {
+      for (size_t pc = threadIdx.x; pc < npieces; pc += TK_WG) {
+        float v[16];
+        load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, v);
+        count_bands(v, shift, bands);
+      }
+    }
+    block_sums<8>(bands, shi);
+    narrow = digits_narrow(sums[4], bands);
   }
-  block_sums<13>(sums, shi);
   if (threadIdx.x < 4) {
     const int t = threadIdx.x;
     pp.rowsum[tok * 4 + t] = t == 0 ? sums[0] : t == 1 ? sums[1] : t == 2 ? sums[2] : sums[3];
   }
   if (threadIdx.x == 0) {
-    // energy left without the TK_DIGITS_TRIM largest elements, in units of 2^(2E): band b counts at
-    // its lower edge 2^(-4b-4); the grid does not carry the token when n_poor * 2^-62 / 3 exceeds
-    // 2^-30 of it
-    float left = 0.0f, edge2 = 0.00390625f;  // 2^-8
-    int trim = TK_DIGITS_TRIM;
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const int c = sums[5 + b], cut = c < trim ? c : trim;
-      trim -= cut;
-      left += (float)(c - cut) * edge2;
-      edge2 *= 0.00390625f;
+    pp.exps[tok] = -shift;
+    pp.flags[tok] = (nonfinite || narrow) ? 1u : 0u;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// activation prep, one WAVE per token: rows of up to HELD * 64 pieces (K <= 4096 at HELD = 4). Same
+// arithmetic and the same bytes out as the one-workgroup-per-token kernels above; what changes is the
+// shape of the work: a token's pieces sit in the registers of one wave, the row maximum and the row
+// sums are wave shuffles, nothing waits at a barrier, every lane has pieces to work on (a K = 2048
+// row has 128 pieces: half a workgroup's threads idle), and a launch has a quarter of the workgroups.
+// Not for rows that are normalized first (the canonical sum of squares has 256 slots) nor for the
+// per-block row sums of the block-scale planes.
+// ------------------------------------------------------------------------------------------
+
+// The token a wave works on, and its tensor. Single tensor, workgroup count a multiple of 16: eight
+// consecutive rows share every 128-byte line of the operand layout, and workgroups go to the 8 XCDs
+// in turn, so the two workgroups that cover rows 8j..8j+7 are taken from the same XCD.
+__device__ __forceinline__ const TkPrep &find_prep_wave(const TkPrep &single, const TkPrep *table, int nprep,
+                                                        int uniform_m, int wave, int &row, int &gt) {
+  const unsigned blk = blockIdx.x;
+  if (!table) {
+    if ((gridDim.x & 15u) == 0) {
+      const unsigned xcd = blk & 7u, slot = blk >> 3;
+      gt = (int)((((slot >> 1) * 8u + xcd) * 8u) + (slot & 1u) * 4u) + wave;
+    } else {
+      gt = (int)blk * 4 + wave;
     }
-    const bool narrow = sums[4] > 0 && (float)sums[4] > 3.0f * 4294967296.0f * left;
+    row = gt;
+    return single;
+  }
+  gt = (int)blk * 4 + wave;
+  if (uniform_m > 0) {
+    const int t = min(gt / uniform_m, nprep - 1);
+    row = gt - t * uniform_m;
+    return table[t];
+  }
+  int lo = 0, hi = nprep - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (table[mid].row_begin <= gt) lo = mid; else hi = mid - 1;
+  }
+  row = gt - table[lo].row_begin;
+  return table[lo];
+}
+
+__device__ __forceinline__ int wave_sum(int v) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+template <int HELD>
+__device__ __forceinline__ void wave_absmax_held(const void *act, int dtype, size_t base, size_t k, size_t npieces, bool vec,
+                                                 int lane, float (&held)[HELD][16], float &gamma, int &nonfinite) {
+  float g = 0.0f;
+  int nf = 0;
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 64;
+    if (pc < npieces) {
+      load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, held[it]);
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const float a = fabsf(held[it][x]);  // elements past k were loaded as 0
+        if (a > g) g = a;                    // NaN never wins (crates/tritium-spec/src/lib.rs:351-360)
+        nf |= !(a <= 3.402823466e38f);
+      }
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    g = fmaxf(g, __shfl_xor(g, o));
+    nf |= __shfl_xor(nf, o);
+  }
+  gamma = g;
+  nonfinite = nf != 0;
+}
+
+template <int HELD>
+__global__ __launch_bounds__(TK_WG) void tk_prep_a8_wave_kernel(TkPrep single, const TkPrep *__restrict__ table, int nprep,
+                                                                int uniform_m, unsigned rows) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int rowi, gt;
+  const TkPrep &pp = find_prep_wave(single, table, nprep, uniform_m, wave, rowi, gt);
+  if ((unsigned)gt >= rows) return;  // no barrier anywhere below
+  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
+  const size_t base = row * k;
+  const void *act = pp.act;
+  const int dtype = pp.act_dtype;
+  int8_t *ap = pp.ap, *qrm = pp.q_rowmajor;
+  const bool vec = act_rows_vectorizable(act, dtype, k);
+  const size_t npieces = nb * 16;
+  float held[HELD][16];
+  float gamma;
+  int nonfinite;
+  wave_absmax_held<HELD>(act, dtype, base, k, npieces, vec, lane, held, gamma, nonfinite);
+  const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
+  const bool live = gamma != 0.0f && !nonfinite;
+  int sum = 0;
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 64;
+    if (pc >= npieces) continue;
+    const size_t kb = pc >> 4;
+    const int q16 = (int)(pc & 15);
+    const size_t e0 = piece_elem0(kb, q16);
+    v4u piece;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const size_t e = e0 + (size_t)sl * 32;
+      uint32_t packed = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        int q = 0;
+        if (live && e + b < k) {
+          float r = rintf(__fmul_rn(held[it][sl * 4 + b], s));  // one multiply, ties to even
+          r = r < -128.0f ? -128.0f : (r > 127.0f ? 127.0f : r);
+          q = (int)r;
+        }
+        sum += q;
+        packed |= ((uint32_t)q & 0xFFu) << (8 * b);
+      }
+      piece[sl] = packed;
+      if (qrm) {
+        if (vec && e + 4 <= k) {
+          *(TK_GLOBAL uint32_t *)(qrm + base + e) = packed;
+        } else {
+          for (int b = 0; b < 4; ++b)
+            if (e + b < k) qrm[base + e + b] = (int8_t)(packed >> (8 * b));
+        }
+      }
+    }
+    if (ap) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, row)) = piece;
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) {
+    if (pp.rowsum) pp.rowsum[row] = sum;
+    pp.act_scale[row] = gamma == 0.0f ? 0.0f : __fdiv_rn(gamma, 127.0f);
+    if (pp.aux) pp.aux[row] = s;
+    if (pp.flags) pp.flags[row] = nonfinite ? 1u : 0u;
+  }
+}
+
+template <int HELD>
+__global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep single, const TkPrep *__restrict__ table,
+                                                                    int nprep, int uniform_m, unsigned rows) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int rowi, gt;
+  const TkPrep &pp = find_prep_wave(single, table, nprep, uniform_m, wave, rowi, gt);
+  if ((unsigned)gt >= rows) return;
+  const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
+  const size_t base = tok * k;
+  const void *act = pp.act;
+  const int dtype = pp.act_dtype;
+  int8_t *ap = pp.ap;
+  const bool vec = act_rows_vectorizable(act, dtype, k);
+  const size_t npieces = nb * 16;
+  float held[HELD][16];
+  float gamma;
+  int nonfinite;
+  wave_absmax_held<HELD>(act, dtype, base, k, npieces, vec, lane, held, gamma, nonfinite);
+  int E = 0;
+  if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
+  const int shift = 30 - E;
+  const bool live = gamma != 0.0f && !nonfinite;
+  int sums[4] = {0, 0, 0, 0}, n_poor = 0;
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 64;
+    if (pc >= npieces) continue;
+    const size_t kb = pc >> 4;
+    const int q16 = (int)(pc & 15);
+    const size_t e0 = piece_elem0(kb, q16);
+    v4u piece[4];
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const size_t e = e0 + (size_t)sl * 32;
+      uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        int q = 0;
+        if (live && e + b < k) {
+          const float r = ldexpf(held[it][sl * 4 + b], shift);
+          q = __float2int_rn(r);  // |q| <= 2^30
+          n_poor += digit_poor(r, q) ? 1 : 0;
+        }
+#pragma unroll
+        for (int dg = 0; dg < 4; ++dg) {
+          int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
+          q = (q - dv) >> 8;
+          sums[dg] += dv;
+          packed[dg] |= ((uint32_t)dv & 0xFFu) << (8 * b);
+        }
+      }
+#pragma unroll
+      for (int dg = 0; dg < 4; ++dg) piece[dg][sl] = packed[dg];
+    }
+#pragma unroll
+    for (int dg = 0; dg < 4; ++dg) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, tok * 4 + dg)) = piece[dg];
+  }
+#pragma unroll
+  for (int dg = 0; dg < 4; ++dg) sums[dg] = wave_sum(sums[dg]);
+  n_poor = wave_sum(n_poor);
+  bool narrow = false;
+  if (n_poor > 0) {  // wave-uniform
+    int bands[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int it = 0; it < HELD; ++it) {
+      const size_t pc = (size_t)lane + (size_t)it * 64;
+      if (pc < npieces) count_bands(held[it], shift, bands);
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) bands[b] = wave_sum(bands[b]);
+    narrow = digits_narrow(n_poor, bands);
+  }
+  if (lane < 4) pp.rowsum[tok * 4 + lane] = lane == 0 ? sums[0] : lane == 1 ? sums[1] : lane == 2 ? sums[2] : sums[3];
+  if (lane == 0) {
     pp.exps[tok] = -shift;
     pp.flags[tok] = (nonfinite || narrow) ? 1u : 0u;
   }
@@ -2509,10 +2756,29 @@ hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n,
 }
 
 hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
-                          unsigned rows) {
+                          unsigned rows, int table_wave_pieces) {
   if (!rows) return hipSuccess;
   TkPrep dummy = {};
   const TkPrep &sg = single ? *single : dummy;
+  // one wave per token where every row has at most 256 pieces and needs neither a norm nor per-block sums
+  size_t wave_pieces = (size_t)(table_wave_pieces > 0 ? table_wave_pieces : 0);
+  if (single) wave_pieces = (single->nb * 16 <= 256 && !single->norm_kind && !single->blocksum) ? single->nb * 16 : 0;
+  // a handful of tokens is a latency problem: a whole workgroup per token finishes a row sooner
+  if (rows < 32) wave_pieces = 0;
+  if (wave_pieces && (kind == TK_PREP_A8 || kind == TK_PREP_DIGITS)) {
+    const dim3 grid((rows + 3) / 4), block(TK_WG);
+    const int held = wave_pieces <= 64 ? 1 : (wave_pieces <= 128 ? 2 : 4);
+    if (kind == TK_PREP_A8) {
+      if (held == 1) hipLaunchKernelGGL(tk_prep_a8_wave_kernel<1>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+      else if (held == 2) hipLaunchKernelGGL(tk_prep_a8_wave_kernel<2>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+      else hipLaunchKernelGGL(tk_prep_a8_wave_kernel<4>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+    } else {
+      if (held == 1) hipLaunchKernelGGL(tk_prep_digits_wave_kernel<1>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+      else if (held == 2) hipLaunchKernelGGL(tk_prep_digits_wave_kernel<2>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+      else hipLaunchKernelGGL(tk_prep_digits_wave_kernel<4>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+    }
+    return hipGetLastError();
+  }
   switch (kind) {
     case TK_PREP_A8:
       if (single && single->nb * 16 <= (size_t)TK_WG)
@@ -2618,6 +2884,17 @@ static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkPro
                                  const TkLaunchCfg &cfg) {
   constexpr int TW = ((RT >= 4 && P <= 2) || (RT == 2 && P == 1)) ? 2 : 1;
   const int threads = cfg.waves * 64;
+  if constexpr (P <= 2 && RT == 1) {  // one row tile: one or two runs per wave, the host's choice by row count
+    if (cfg.tw == 2) {
+      switch (cfg.ring) {
+        case 2: return table ? flow_launch_one(tk_flow_kernel<P, RT, 2, 2, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, RT, 2, 2, false>, s, sg, table, wg_prob, cfg, threads);
+        case 3: return table ? flow_launch_one(tk_flow_kernel<P, RT, 2, 3, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, RT, 2, 3, false>, s, sg, table, wg_prob, cfg, threads);
+        case 4: return table ? flow_launch_one(tk_flow_kernel<P, RT, 2, 4, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, RT, 2, 4, false>, s, sg, table, wg_prob, cfg, threads);
+        case 5: return table ? flow_launch_one(tk_flow_kernel<P, RT, 2, 5, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, RT, 2, 5, false>, s, sg, table, wg_prob, cfg, threads);
+        default: return hipErrorInvalidValue;
+      }
+    }
+  }
   switch (cfg.ring) {
     case 2:
       if (table) return flow_launch_one(tk_flow_kernel<P, RT, TW, 2, true>, s, sg, table, wg_prob, cfg, threads);
@@ -2675,10 +2952,17 @@ static hipError_t launch_flow_p(hipStream_t s, const TkProblem &sg, const TkProb
   }
 }
 
-// lock-step runs per wave of the flow kernel for a (planes, rt) pair: two where registers allow and a
+// lock-step runs per wave of the flow kernel for a (planes, rt, rows) triple: two where registers allow and a
 // single run would keep too few bytes in flight (four row tiles of one or two planes; two row
 // tiles of one plane: K=2048 N=8192, 32 int8 rows, one plane went from 263 to 228 us)
-int tk_flow_runs_per_wave(int planes, int rt) { return ((rt >= 4 && planes <= 2) || (rt == 2 && planes == 1)) ? 2 : 1; }
+int tk_flow_runs_per_wave(int planes, int rt, int rows) {
+  // One row tile: a second run doubles the loads a wave keeps in flight and costs registers, i.e. waves
+  // per SIMD. Measured over 128 layer copies per launch: one plane (K=2560 N=6912) 4 / 4 / 16 rows
+  // +5% / +10% / +7% with two runs, a single row -1.5%; two planes (K=2048 N=8192) 4..8 rows -3%,
+  // 16 rows +2.4%.
+  if (rt == 1) return (planes == 1 && rows >= 2) || (planes == 2 && rows >= 9) ? 2 : 1;
+  return ((rt >= 4 && planes <= 2) || (rt == 2 && planes == 1)) ? 2 : 1;
+}
 // ... of the 32x32x32 form: always a pair of adjacent tiles
 int tk_flow32_runs_per_wave(void) { return 2; }
 
@@ -2691,12 +2975,14 @@ int tk_flow32_runs_per_wave(void) { return 2; }
 // (one row tile: K=2560 runs 2% faster on 5 positions than on 4 padded to 12) or a quarter (more
 // row tiles) of the positions, weighted by each problem's chunk count; if all do, the one that
 // pads least.
-int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows) {
+int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows, int tw) {
   // one row tile: 4 positions with runs of one tile (up to 8 rows), 5 with runs of two (9..16 rows)
   const int pref1a[4] = {4, 5, 3, 2}, pref1b[4] = {5, 4, 3, 2}, pref2[4] = {4, 5, 3, 2}, pref4[4] = {2, 3, 4, 5};
-  const int *pref1 = rows <= 8 ? pref1a : pref1b;
-  const double limit = rt == 1 ? 0.10 : 0.25;
-  const int *cand = rt == 1 ? pref1 : (rt == 2 ? pref2 : pref4);
+  const int *pref1 = rows <= 8 ? pref1a : pref1b;  // (one plane with two runs per wave: 4 positions at every row count; see the caller)
+  // one row tile with two runs per wave: 4 positions measured best even where they pad K (K = 2560, ten
+  // blocks: 4 positions 97.9 us, 3: 98.6, 5: 99.1; 16 int8 rows: 128.5 / 131 / 130.5)
+  const double limit = (rt == 1 && tw < 2) ? 0.10 : 0.25;
+  const int *cand = rt == 1 ? (tw >= 2 ? pref2 : pref1) : (rt == 2 ? pref2 : pref4);
   int best = cand[0];
   double best_waste = -1.0;
   for (int c = 0; c < 4; ++c) {
