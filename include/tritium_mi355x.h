@@ -63,6 +63,8 @@ typedef struct tk_device_info {
 /* ---- lifetime: BackendEntry::init (crates/tritium-runtime/src/lib.rs:73-110) and
  *      RocmBackend::new(ordinal) (crates/tritium-rocm/src/rocm.rs:234-300) ---- */
 int tk_init(int device, tk_ctx **out);
+/* Frees the context's workspaces. Weight buffers and groups created on it stay valid to FREE (not to
+ * use) afterwards, in any order: the stream lives until the last of them is gone. */
 void tk_destroy(tk_ctx *ctx);
 const char *tk_last_error(void);
 /* expected/got of the last ShapeMismatch, or requested/0 of the last OutOfMemory, on this thread */
@@ -310,6 +312,17 @@ int tk_linear_rmsnorm_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *x
  * raw int32 accumulators Σ_k q·trit instead of the scaled output. */
 int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
                  size_t m, void *out, int out_dtype);
+
+/* The same two calls with a fused residual add, out[m,n] = residual[m,n] + value (one f32 add after the
+ * scale multiplies): the epilogue of tq2_0_add_mpgemm_tiled_i8_scaled_residual and its TQ1_0 twin
+ * (crates/tritium-cuda/kernels/tq2_0_add.cu:577-637,856-913), which saves the decode step a separate
+ * residual_add launch and memory pass after the o and down projections. residual is a device pointer to
+ * [m,n] elements of the output's type (f32 or bf16; bf16 is widened, added in f32, rounded once) and may
+ * be the output itself. */
+int tk_linear_a8_residual(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
+                          size_t m, const void *residual, void *out, int out_dtype);
+int tk_linear_i8_residual(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
+                          size_t m, const void *residual, void *out, int out_dtype);
 
 /* ---- block-scale additive planes (SALT): every plane is a TQ2_0 tensor whose per-256-block f16
  *      scales count, W[n,k] = Σ_p s_p[n, k/256] · trit_p[n,k] (crates/tritium-format/src/salt.rs:1-19),

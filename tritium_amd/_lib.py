@@ -104,6 +104,8 @@ SIGNATURES = {
     "tk_group_create_normed": (C.c_int, [vp, C.POINTER(GroupMember), C.POINTER(RmsNorm), sz, C.c_int, C.c_int,
                                          C.POINTER(vp)]),
     "tk_linear_i8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, vp, sz, vp, C.c_int]),
+    "tk_linear_a8_residual": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, vp, C.c_int]),
+    "tk_linear_i8_residual": (C.c_int, [vp, C.POINTER(LinearDesc), vp, vp, sz, vp, vp, C.c_int]),
     "tk_linear_float_seq": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_group_create": (C.c_int, [vp, C.POINTER(GroupMember), sz, C.c_int, C.c_int, C.c_int, C.POINTER(vp)]),
     "tk_group_launch": (C.c_int, [vp, vp]),

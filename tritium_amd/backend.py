@@ -431,6 +431,16 @@ class Mi355xBackend:
         """linear_a8 on the static device scratch: no allocation; refuses shapes that do not fit."""
         self._lin(self._lib.tk_linear_a8_noalloc, layer, act, m, out)
 
+    def linear_a8_residual(self, layer, act, m, residual, out):
+        """out = residual + linear_a8(act); residual has the output's dtype and may be `out` itself."""
+        _check(self._lib.tk_linear_a8_residual(self._ctx, C.byref(layer.desc), act.ptr, act.dtype, m, residual.ptr,
+                                               out.ptr, out.dtype))
+
+    def linear_i8_residual(self, layer, q, act_scale, m, residual, out):
+        _check(self._lib.tk_linear_i8_residual(self._ctx, C.byref(layer.desc), q.ptr,
+                                               act_scale.ptr if act_scale is not None else None, m, residual.ptr,
+                                               out.ptr, out.dtype))
+
     def linear_float_seq(self, layer, act, m, out):
         self._lin(self._lib.tk_linear_float_seq, layer, act, m, out)
 

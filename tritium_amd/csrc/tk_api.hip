@@ -1,5 +1,6 @@
 // Host side of the C ABI: validation in the reference's order, device buffers, dispatch between the
 // decode GEMV and the prefill GEMM, and the trait-shaped host-slice entry points.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -79,7 +80,18 @@ struct tk_ctx {
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum;
   int *d_invalid = nullptr;
+  // The context itself plus every weight buffer and group created on it: tk_destroy gives up the
+  // context's own reference, the stream and this record live until the last of them is released, so
+  // buffers and groups may be freed after tk_destroy.
+  std::atomic<int> refs{1};
 };
+
+static void ctx_release(tk_ctx *ctx) {
+  if (ctx->refs.fetch_sub(1) != 1) return;
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+}
 
 struct tk_weights {
   tk_ctx *ctx;
@@ -233,16 +245,22 @@ extern "C" int tk_init(int device, tk_ctx **out) {
 
 extern "C" void tk_destroy(tk_ctx *ctx) {
   if (!ctx) return;
-  (void)hipSetDevice(ctx->device);
-  (void)hipStreamSynchronize(ctx->stream);
-  DevBuf *bufs[] = {&ctx->ap, &ctx->rowsum, &ctx->fscale, &ctx->aux, &ctx->exps,
-                    &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp,
-                    &ctx->ynorm, &ctx->blocksum};
-  for (DevBuf *b : bufs)
-    if (b->p) (void)hipFree(b->p);
-  if (ctx->d_invalid) (void)hipFree(ctx->d_invalid);
-  (void)hipStreamDestroy(ctx->stream);
-  delete ctx;
+  {
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    DevBuf *bufs[] = {&ctx->ap, &ctx->rowsum, &ctx->fscale, &ctx->aux, &ctx->exps,
+                      &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp,
+                      &ctx->ynorm, &ctx->blocksum};
+    for (DevBuf *b : bufs) {
+      if (b->p) (void)hipFree(b->p);
+      b->p = nullptr;
+      b->cap = 0;
+    }
+    if (ctx->d_invalid) (void)hipFree(ctx->d_invalid);
+    ctx->d_invalid = nullptr;
+  }
+  ctx_release(ctx);
 }
 
 extern "C" const char *tk_device_id(const tk_ctx *ctx) { return ctx ? ctx->device_id.c_str() : ""; }
@@ -406,6 +424,7 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
   w->len_bytes = packed_len;
   w->format = format;
   w->invalid_row = invalid == INT32_MAX ? -1 : invalid;
+  ctx->refs.fetch_add(1);
   *out = w;
   return TK_OK;
 }
@@ -414,11 +433,18 @@ extern "C" int tk_upload_weights_i2s(tk_ctx *ctx, const uint8_t *payload, size_t
                                      tk_weights **out, float *scale) {
   if (!ctx || !out || !scale) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_weights_i2s: null pointer");
   *out = nullptr;
+  // the payload must hold the tensor before anything is sized from the caller's n and k
+  // (the converter's own checks, in its order and with its errors: crates/tritium-format/src/i2s.rs:122-135)
+  size_t elems;
+  if (__builtin_mul_overflow(n, k, &elems)) return tk_fail(TK_ERR_INVALID_INPUT, "I2_S element count overflows");
+  if (elems % 128 != 0) return tk_fail(TK_ERR_INVALID_INPUT, "I2_S tensor of %zu elements is not a multiple of 128", elems);
+  if (payload_len < elems / 4 + 4) return tk_fail_mismatch(elems / 4 + 4, payload_len);
   const size_t len = tk_packed_len(n, k, TK_FORMAT_TQ2_0);
+  if (!len && n && k) return tk_fail(TK_ERR_INVALID_INPUT, "packed weight byte count overflows");
   std::vector<uint8_t> packed;
   try {
     packed.resize(len);
-  } catch (const std::bad_alloc &) {
+  } catch (const std::exception &) {
     return tk_fail(TK_ERR_BACKEND, "tk_upload_weights_i2s: host allocation of %zu bytes failed", len);
   }
   TKCHK(tk_convert_i2s_to_tq2_0(payload, payload_len, n, k, packed.data(), len, scale));
@@ -432,11 +458,25 @@ extern "C" int tk_upload_weights_gguf(tk_ctx *ctx, const tk_gguf *g, const uint8
   size_t n, k;
   int format;
   TKCHK(tk_gguf_ternary_shape(g, name, &n, &k, &format));
+  // the dims of a tensor are the file's word: check them against the bytes the file really holds
+  // before sizing anything from them (a crafted header may claim 2^62 rows)
+  {
+    tk_gguf_tensor info;
+    uint64_t off = 0, plen = 0;
+    if (!tk_gguf_tensor_find(g, name, &info)) return tk_fail(TK_ERR_INVALID_INPUT, "tensor `%s` not found", name);
+    TKCHK(tk_gguf_tensor_payload(g, file_len, &info, &off, &plen));
+    size_t nk;
+    if (__builtin_mul_overflow(n, k, &nk) || nk / 5 > plen)  // the densest packing holds 5 trits per byte
+      return tk_fail(TK_ERR_INVALID_INPUT, "tensor `%s` claims %zu x %zu elements but its payload holds %llu bytes", name, n, k,
+                     (unsigned long long)plen);
+  }
   const size_t len = tk_packed_len(n, k, format);
+  if (!len && n && k) return tk_fail(TK_ERR_INVALID_INPUT, "packed weight byte count overflows");
+  if (row_scales_len != n) return tk_fail_mismatch(n, row_scales_len);
   std::vector<uint8_t> packed;
   try {
     packed.resize(len);
-  } catch (const std::bad_alloc &) {
+  } catch (const std::exception &) {
     return tk_fail(TK_ERR_BACKEND, "tk_upload_weights_gguf: host allocation of %zu bytes failed", len);
   }
   TKCHK(tk_gguf_load_ternary(g, file, file_len, name, packed.data(), len, row_scales, row_scales_len));
@@ -445,12 +485,16 @@ extern "C" int tk_upload_weights_gguf(tk_ctx *ctx, const tk_gguf *g, const uint8
 
 extern "C" void tk_free_weights(tk_weights *w) {
   if (!w) return;
-  std::lock_guard<std::mutex> lk(w->ctx->mu);
-  (void)hipSetDevice(w->ctx->device);
-  (void)hipStreamSynchronize(w->ctx->stream);
-  (void)hipFree(w->codes);
-  if (w->block_scales) (void)hipFree(w->block_scales);
-  delete w;
+  tk_ctx *ctx = w->ctx;
+  {
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(w->codes);
+    if (w->block_scales) (void)hipFree(w->block_scales);
+    delete w;
+  }
+  ctx_release(ctx);
 }
 extern "C" size_t tk_weights_len_bytes(const tk_weights *w) { return w ? w->len_bytes : 0; }
 extern "C" size_t tk_weights_n(const tk_weights *w) { return w ? w->n : 0; }
@@ -746,7 +790,7 @@ static int take_workspace(tk_ctx *ctx, bool static_ws, size_t ap_bytes, size_t R
 
 static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int prep_kind, const void *act,
                       int act_dtype, const float *act_scale_in, size_t m, void *out, int out_dtype,
-                      const tk_rmsnorm *norm = nullptr, bool static_ws = false) {
+                      const tk_rmsnorm *norm = nullptr, bool static_ws = false, const void *residual = nullptr) {
   size_t n, k;
   TKCHK(validate_layer(ctx, layer, &n, &k));
   if (m == 0 || n == 0) return TK_OK;  // crates/tritium-rocm/src/rocm.rs:521-523
@@ -815,6 +859,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   pr.ap = pp.ap;
   pr.rowsum = pp.rowsum;
   pr.out = out;
+  pr.residual = residual;
   if (prep_kind == TK_PREP_A8) {
     pr.act_scale = pp.act_scale;
     pr.aux = pp.aux;
@@ -1039,6 +1084,31 @@ extern "C" int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
   return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_I8, q, TK_I8, act_scale, m, out, out_dtype);
+}
+
+// out = residual + linear(act): the fused residual-add epilogue of the reference's decode kernels
+// (crates/tritium-cuda/kernels/tq2_0_add.cu:577-637,856-913)
+extern "C" int tk_linear_a8_residual(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype, size_t m,
+                                     const void *residual, void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_act_dtype(act_dtype));
+  TKCHK(check_out_dtype(out_dtype, false));
+  if (!residual && m && layer && layer->n_planes > 0 && layer->planes[0] && layer->planes[0]->n)
+    return tk_fail(TK_ERR_INVALID_INPUT, "null residual pointer");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_A8, act, act_dtype, nullptr, m, out, out_dtype, nullptr, false, residual);
+}
+
+extern "C" int tk_linear_i8_residual(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
+                                     size_t m, const void *residual, void *out, int out_dtype) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");
+  TKCHK(check_out_dtype(out_dtype, false));
+  if (!residual && m && layer && layer->n_planes > 0 && layer->planes[0] && layer->planes[0]->n)
+    return tk_fail(TK_ERR_INVALID_INPUT, "null residual pointer");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  return run_linear(ctx, layer, TK_MODE_INT8, TK_PREP_I8, q, TK_I8, act_scale, m, out, out_dtype, nullptr, false, residual);
 }
 
 extern "C" int tk_linear_float_seq(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype, size_t m,
@@ -1603,6 +1673,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, planes, rt, rows_max));
   }
   if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds, rows_max);
+  ctx->refs.fetch_add(1);
   *out = g;
   return TK_OK;
 }
@@ -1635,14 +1706,16 @@ extern "C" int tk_group_launch(tk_ctx *ctx, tk_group *g) { return tk_group_launc
 
 extern "C" void tk_group_destroy(tk_group *g) {
   if (!g) return;
+  tk_ctx *ctx = g->ctx;
   {
-    std::lock_guard<std::mutex> lk(g->ctx->mu);
-    (void)hipSetDevice(g->ctx->device);
-    (void)hipStreamSynchronize(g->ctx->stream);
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
     if (g->ws) (void)hipFree(g->ws);
     if (g->tables) (void)hipFree(g->tables);
   }
   delete g;
+  ctx_release(ctx);
 }
 
 // ------------------------------------------------------------------------------------------

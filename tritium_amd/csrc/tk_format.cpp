@@ -78,7 +78,12 @@ bool unpack_block(const uint8_t *blk, int format, int8_t *t) {
 }  // namespace
 
 extern "C" size_t tk_packed_len(size_t n, size_t k, int format) {
-  return n * ((k + kBlock - 1) / kBlock) * block_bytes(format);
+  // 0 for an unsupported format and for a shape whose byte count does not fit size_t
+  size_t row, total;
+  if (k > (size_t)-1 - kBlock) return 0;
+  if (__builtin_mul_overflow((k + kBlock - 1) / kBlock, block_bytes(format), &row)) return 0;
+  if (__builtin_mul_overflow(n, row, &total)) return 0;
+  return total;
 }
 
 extern "C" int tk_pack_rows(const int8_t *trits, size_t trits_len, size_t n, size_t k, int format, uint8_t *out,

@@ -40,6 +40,7 @@ struct TkProblem {
   const float *bscale[TK_MAX_PLANES];
   const int32_t *blocksum;
   void *out;                 // [M,N]
+  const void *residual;      // [M,N] in the output's element type, added to every output (one f32 add), or null
   int n, k, nb, R, M;
   int rs;                    // row stride of `ap` in rows (>= R; the GEMM pads it, see tk_api.hip)
   int mode, raw_dtype, out_dtype, planes;

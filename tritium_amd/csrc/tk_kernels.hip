@@ -66,6 +66,15 @@ __device__ __forceinline__ void store_out(void *out, int dtype, size_t idx, floa
     gstore((float *)out + idx, v);
 }
 
+// Fused residual add: out = residual + value, one f32 add (the epilogue of the reference's
+// tq2_0_add_mpgemm_tiled_i8_scaled_residual, crates/tritium-cuda/kernels/tq2_0_add.cu:577-637).
+// The residual has the layout and element type of the output; null = no residual.
+__device__ __forceinline__ float with_residual(const void *residual, int dtype, size_t idx, float v) {
+  if (!residual) return v;
+  const float r = dtype == TK_BF16 ? bf16_to_f32(gload((const uint16_t *)residual + idx)) : gload((const float *)residual + idx);
+  return __fadd_rn(r, v);
+}
+
 __device__ __forceinline__ v4i expand_codes(uint32_t w) {
   v4i b;
   b.x = (int)(w & 0x03030303u);
@@ -171,7 +180,7 @@ __device__ __forceinline__ void finish_lane(const TkProblem &pr, int n, int rowb
         }
       }
       if (pr.act_scale) f = __fmul_rn(f, pr.act_scale[m]);
-      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, with_residual(pr.residual, pr.out_dtype, (size_t)m * pr.n + n, f));
     }
   } else {
     int tok = rowbase >> 2;
@@ -184,7 +193,7 @@ __device__ __forceinline__ void finish_lane(const TkProblem &pr, int n, int rowb
         f = p == 0 ? t : __fadd_rn(f, t);
       }
     }
-    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, with_residual(pr.residual, pr.out_dtype, (size_t)tok * pr.n + n, f));
   }
 }
 
@@ -423,6 +432,7 @@ __global__ __launch_bounds__(TK_WG) void tk_stream_kernel(TkProblem single, cons
 // a pointer into a problem table they would be fetched again after every store.
 struct TkHot {
   void *out;
+  const void *residual;
   const int32_t *rowsum;
   const float *act_scale;
   const int32_t *exps;
@@ -432,6 +442,7 @@ struct TkHot {
 __device__ __forceinline__ TkHot make_hot(const TkProblem &pr) {
   TkHot h;
   h.out = pr.out;
+  h.residual = pr.residual;
   h.rowsum = pr.rowsum;
   h.act_scale = pr.act_scale;
   h.exps = pr.exps;
@@ -551,12 +562,14 @@ __device__ __forceinline__ void flow_epilogue(const PR &pr, int n, int rowbase, 
     for (int r = 0; r < 4; ++r) {
       const int m = rowbase + r;
       if (m >= pr.R || (rc.flag & (1u << r))) continue;
-      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, int8_value<P>(acc, r, sc, rc, pr.act_scale != nullptr));
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n,
+                with_residual(pr.residual, pr.out_dtype, (size_t)m * pr.n + n, int8_value<P>(acc, r, sc, rc, pr.act_scale != nullptr)));
     }
   } else {
     const int tok = rowbase >> 2;
     if (tok >= pr.M || rc.flag) return;
-    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, digits_value<P>(acc, sc, rc));
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n,
+              with_residual(pr.residual, pr.out_dtype, (size_t)tok * pr.n + n, digits_value<P>(acc, sc, rc)));
   }
 }
 
@@ -573,7 +586,7 @@ __device__ __forceinline__ void exact_rows(const TkProblem &pr, int n, int rowba
         f = p == 0 ? t : __fadd_rn(f, t);
       }
       if (pr.act_scale) f = __fmul_rn(f, pr.act_scale[m]);
-      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, f);
+      store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, with_residual(pr.residual, pr.out_dtype, (size_t)m * pr.n + n, f));
     }
   } else {
     const int tok = rowbase >> 2;
@@ -583,7 +596,7 @@ __device__ __forceinline__ void exact_rows(const TkProblem &pr, int n, int rowba
       float t = __fmul_rn(seq_dot(pr, p, n, tok, 0), pr.scales[p][n]);
       f = p == 0 ? t : __fadd_rn(f, t);
     }
-    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, f);
+    store_out(pr.out, pr.out_dtype, (size_t)tok * pr.n + n, with_residual(pr.residual, pr.out_dtype, (size_t)tok * pr.n + n, f));
   }
 }
 
@@ -1404,7 +1417,8 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, const TkHo
   // last barrier of the main loop) and leave as whole 16-byte pieces of contiguous row segments:
   // every store instruction of a wave then covers full cache lines.
   const int esz = hot.out_dtype == TK_BF16 ? 2 : 4;
-  const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0;
+  // (a call with a fused residual add takes the direct stores: the residual is read where the value is formed)
+  const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0 && !hot.residual;
   if (staged) {
     constexpr int WG_COLS = TK_GEMM_WAVES * NT * 16;
     const bool int8_mode = hot.mode == TK_MODE_INT8 || hot.out_dtype == TK_I32;
@@ -1767,7 +1781,8 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
   };
 
   const int esz = hot.out_dtype == TK_BF16 ? 2 : 4;
-  const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0;
+  // (a call with a fused residual add takes the direct stores: the residual is read where the value is formed)
+  const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0 && !hot.residual;
   if (staged) {
     constexpr int WG_COLS = TK_GEMM_WAVES * NT * 16;
     const bool int8_mode = hot.mode == TK_MODE_INT8 || hot.out_dtype == TK_I32;
