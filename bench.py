@@ -422,6 +422,56 @@ def bench_config5(T, be, rng):
     return res
 
 
+def bench_zero_skip(T, be, rng, iters=60):
+    """Zero-chunk skip on the headline shape (two planes, K=2048, N=8192, W1.58A8, batch 1 and 4, 128 layer
+    copies per launch). Plane 2 has P(0)=0.85 in two forms: block-structured (75% of its 16-row x 256-trit
+    chunks all zero, the rest i.i.d. with P(0)=0.4) and i.i.d. Each is timed with the map the upload keeps
+    by the 0.5% rule and with maps disabled; for the i.i.d. plane also with a map forced on (it has no
+    zero chunk: the rule keeps none, so the default costs nothing). GB/s are the dense algorithmic bytes
+    over time, so a skip shows as a figure above what the memory could deliver for the full planes."""
+    nt, nb = N2 // 16, K2 // 256
+    p1 = ternary(rng, N2, K2, 0.4)
+    structured = ternary(rng, N2, K2, 0.4)
+    z = rng.random((nt, nb)) < 0.75
+    structured.reshape(nt, 16, nb, 256)[z[:, None, :, None].repeat(16, 1).repeat(256, 3)] = 0
+    iid = ternary(rng, N2, K2, 0.85)
+    scs = [rng.uniform(0.01, 0.1, N2).astype(np.float32) for _ in range(2)]
+    res = {"workload": f"two planes K={K2} N={N2}, plane 2 with P(0)=0.85 block-structured ({z.mean():.2f} of its chunks zero) or i.i.d.; "
+                       f"W1.58A8, {COPIES} layer copies per launch, decode kernel alone",
+           "zero_fraction_of_plane2": {"structured": round(float((structured == 0).mean()), 3), "iid": round(float((iid == 0).mean()), 3)}}
+    packed1 = T.pack_rows(p1, N2, K2)
+    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((4, K2)).astype(np.float32)), "bf16") for _ in range(COPIES)]
+    outs = [be.empty(4 * N2, "f32") for _ in range(COPIES)]
+    ref_out = {}
+    for name, plane2, modes in (("structured", structured, (0, 1)), ("iid", iid, (0, 1, 2))):
+        packed2 = T.pack_rows(plane2, N2, K2)
+        for mode in modes:
+            be.set_zero_skip(mode)
+            layers = [be.linear([packed1, packed2], scs, N2, K2) for _ in range(COPIES)]
+            kept = layers[0].planes[1].zero_chunks()
+            tag = f"{name}_{('by_rule', 'maps_off', 'map_forced')[mode]}"
+            res[tag] = {"plane2_zero_chunks": kept[0], "chunks": kept[1], "map_kept": kept[2]}
+            for m in (1, 4):
+                g = be.group([(layers[i], acts[i], m, outs[i]) for i in range(COPIES)], 1, "bf16", "f32")
+                g.launch()
+                be.sync()
+                got = outs[COPIES - 1].to_host()[: m * N2].copy()
+                if (name, m) in ref_out and not (got.view(np.uint32) == ref_out[(name, m)].view(np.uint32)).all():
+                    sys.exit(f"bench.py: zero-skip leg: bits differ between map settings ({tag}, batch {m})")
+                ref_out[(name, m)] = got
+                ms = time_calls(be, lambda i: g.launch_parts(False, True), iters)
+                by = COPIES * algorithmic_bytes(m, N2, K2, PLANES2, 2, 4, a8=True)
+                res[tag][f"batch{m}"] = {"kernel_us_per_launch": round(ms * 1e3, 1), "dense_GB/s": round(by / ms / 1e6, 1)}
+                g.destroy()
+            for l in layers:
+                l.free()
+    be.set_zero_skip(0)
+    res["bits"] = "identical across map settings (checked on the last layer copy of every launch)"
+    for x in acts + outs:
+        x.free()
+    return res
+
+
 def bench_salt(T, be, rng, iters=30):
     """Block-scale additive planes (SALT): the headline shape K=2048 x 2 planes with per-256-block f16
     scales, one tall layer of N = 262,144 output channels per launch (2 x 134 MB of codes; two
@@ -592,7 +642,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,salt,vjp",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,salt,vjp",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -648,6 +698,7 @@ def main():
                 "prefill": ("prefill_gemm", lambda: bench_prefill(T, be, rng, 2048, 2560, 6912)),
                 "stack": ("projection_stack", lambda: bench_stack(T, be, rng)),
                 "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng)),
+                "zero_skip": ("zero_chunk_skip", lambda: bench_zero_skip(T, be, rng)),
                 "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng)),
                 "vjp": ("projected_vjp", lambda: bench_vjp(T, be, rng))}
         out["extra"] = {}

@@ -83,6 +83,16 @@ int tk_pack_rows(const int8_t *trits, size_t trits_len, size_t n, size_t k, int 
 int tk_unpack_rows(const uint8_t *packed, size_t packed_len, size_t n, size_t k, int format,
                    int8_t *trits, size_t trits_len);
 
+/* ---- zero-block bitmaps of packed TQ2_0 rows: compute_zero_bitmaps
+ *      (crates/tritium-format/src/tq2.rs:101-181). words [n * ceil(nb/32)], nb = ceil(k/256): bit b%32 of
+ *      word r*ceil(nb/32) + b/32 is set when block b of row r holds only zero trits (64 code bytes 0x55;
+ *      the scale bytes do not count). Rows are row_bytes apart. Short rows or buffers ->
+ *      TK_ERR_INVALID_INPUT; k == 0 -> TK_OK, nothing written. This is the per-row map the reference's
+ *      sparse decode kernels take; the device keeps its own map at the granularity it streams
+ *      (tk_set_zero_skip). ---- */
+int tk_compute_zero_bitmaps(const uint8_t *packed, size_t packed_len, size_t n, size_t k, size_t row_bytes,
+                            uint32_t *words, size_t words_len);
+
 /* ---- I2_S ingest: convert_i2s_to_tq2_0 (crates/tritium-format/src/i2s_int8.rs:36-68) over
  *      unpack_i2s_tensor (crates/tritium-format/src/i2s.rs:70-158). payload = n*k/4 quant bytes
  *      (32-byte blocks of 128 elements of the flat [n,k] tensor, code = trit + 1, code 3 rejected)
@@ -186,6 +196,17 @@ size_t tk_weights_len_bytes(const tk_weights *w); /* DeviceBuffer::len_bytes: th
 size_t tk_weights_n(const tk_weights *w);
 size_t tk_weights_k(const tk_weights *w);
 int tk_weights_format(const tk_weights *w);
+/* Zero-chunk skip: what the reference's sparse decode kernels do with per-row bitmaps
+ * (crates/tritium-cuda/kernels/tq2_0_add.cu:330-401,504-571), at the granularity this layout streams.
+ * At upload every 1-KiB chunk (16 rows x 256 trits) that holds only zero trits is marked; when at least
+ * 0.5% of a plane's chunks are (the reference's BITMAP_MIN_ZERO_BLOCK_FRAC,
+ * crates/tritium-cuda/src/cuda/mod.rs:384-405) the map is kept, and the bandwidth-bound decode kernel
+ * then fetches such chunks from one resident all-zero chunk instead of from memory: same bytes, same
+ * arithmetic, identical bits, less traffic. Planes without such structure (i.i.d. trits have none)
+ * carry no map and take the plain path. tk_set_zero_skip acts on later uploads: 0 = by the threshold,
+ * 1 = never keep a map, 2 = always. tk_weights_zero_chunks reports what an upload found. */
+int tk_set_zero_skip(tk_ctx *ctx, int mode);
+int tk_weights_zero_chunks(const tk_weights *w, size_t *zero, size_t *total, int *map_kept);
 /* Debug/parity aid: decode the device-resident planes back to [n,k] trits. */
 int tk_weights_download_trits(tk_ctx *ctx, const tk_weights *w, int8_t *trits, size_t trits_len);
 

@@ -253,6 +253,44 @@ int to_unpack_i2s_tensor(const uint8_t *payload, size_t payload_len, size_t n_el
   return TO_OK;
 }
 
+/* tq2.rs:101-122 : bit b of word b/32 is set iff every qs byte of block b is 0x55. */
+static size_t sat_mul(size_t a, size_t b) {
+  size_t r;
+  return __builtin_mul_overflow(a, b, &r) ? (size_t)-1 : r;
+}
+
+int to_compute_zero_bitmap(const uint8_t *packed_row, size_t row_len, size_t k, uint32_t *words, size_t words_len) {
+  const size_t nb = k / TO_QK_K + (k % TO_QK_K != 0);
+  const size_t need = sat_mul(nb, TO_TQ2_0_BLOCK_BYTES); /* tq2.rs:105 */
+  if (row_len < need) return TO_ERR_SHAPE;               /* FormatError::WrongBlockLen */
+  const size_t nwords = nb / 32 + (nb % 32 != 0);
+  if (words_len < nwords) return TO_ERR_SHAPE;
+  for (size_t w = 0; w < nwords; ++w) words[w] = 0;
+  for (size_t b = 0; b < nb; ++b) {
+    const uint8_t *qs = packed_row + b * TO_TQ2_0_BLOCK_BYTES;
+    int all = 1;
+    for (size_t i = 0; i < 64; ++i) all &= qs[i] == 0x55;
+    if (all) words[b / 32] |= (uint32_t)1 << (b % 32);
+  }
+  return TO_OK;
+}
+
+/* tq2.rs:134-181 */
+int to_compute_zero_bitmaps(const uint8_t *packed, size_t packed_len, size_t n, size_t k, size_t row_bytes,
+                            uint32_t *words, size_t words_len) {
+  const size_t nb = k / TO_QK_K + (k % TO_QK_K != 0);
+  const size_t wpr = nb / 32 + (nb % 32 != 0);
+  if (nb == 0) return TO_OK;                                          /* tq2.rs:146-148 */
+  if (row_bytes < sat_mul(nb, TO_TQ2_0_BLOCK_BYTES)) return TO_ERR_SHAPE; /* :155-161 */
+  if (packed_len < sat_mul(n, row_bytes)) return TO_ERR_SHAPE;           /* :165-171 */
+  if (words_len != sat_mul(n, wpr)) return TO_ERR_SHAPE;
+  for (size_t r = 0; r < n; ++r) {
+    int rc = to_compute_zero_bitmap(packed + r * row_bytes, row_bytes, k, words + r * wpr, wpr);
+    if (rc) return rc;
+  }
+  return TO_OK;
+}
+
 /* i2s_int8.rs:47-68 : decode, then pack_tq2_0_row of every row with unit block scales. */
 int to_convert_i2s_to_tq2_0(const uint8_t *payload, size_t payload_len, size_t n, size_t k, uint8_t *out,
                             size_t out_len, float *scale) {

@@ -176,6 +176,17 @@ uint64_t to_xorshift64_next(uint64_t *state);
 uint16_t to_f32_to_bf16(float x);
 float to_bf16_to_f32(uint16_t h);
 
+/* ---- zero-block bitmaps: crates/tritium-format/src/tq2.rs:101-181 ----
+ * One bit per 256-trit block of a packed TQ2_0 row, SET when all 64 code bytes are 0x55 (every trit
+ * zero; the scale bytes do not matter); ceil(nb/32) words per row, padding bits never set.
+ * to_compute_zero_bitmap: TO_ERR_SHAPE when the row is shorter than nb*66 bytes, or `words` than
+ * ceil(nb/32). to_compute_zero_bitmaps: rows `row_bytes` apart; k == 0 -> TO_OK with nothing written;
+ * TO_ERR_SHAPE when row_bytes < nb*66, packed_len < n*row_bytes (saturating), or words_len is not
+ * n*ceil(nb/32). */
+int to_compute_zero_bitmap(const uint8_t *packed_row, size_t row_len, size_t k, uint32_t *words, size_t words_len);
+int to_compute_zero_bitmaps(const uint8_t *packed, size_t packed_len, size_t n, size_t k, size_t row_bytes,
+                            uint32_t *words, size_t words_len);
+
 /* ---- timed CPU baseline: crates/tritium-cpu/src/kernel.rs:49-78,568-573,577-664,824-1003 ----
  * Same dispatch as the reference: unpack every call; rows chunked at clamp(65536/(n*k),1,m)
  * across `threads` workers; AVX-VNNI/AVX2 int8 kernel when every activation is an integer in

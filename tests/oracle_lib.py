@@ -86,6 +86,9 @@ class Oracle:
                                            f32p, sz]
         L.to_cpu_mpgemm_fast.argtypes = [u8p, sz, C.c_int, f32p, f32p, sz, sz, sz, f32p, C.c_int,
                                          C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        u32p = C.POINTER(C.c_uint32)
+        L.to_compute_zero_bitmap.argtypes = [u8p, sz, sz, u32p, sz]
+        L.to_compute_zero_bitmaps.argtypes = [u8p, sz, sz, sz, sz, u32p, sz]
         for name in ("to_pack_tq2_0_block", "to_pack_tq1_0_block"):
             getattr(L, name).argtypes = [i8p, C.c_uint16, u8p]
         for name in ("to_unpack_tq2_0_block", "to_unpack_tq1_0_block"):
@@ -226,6 +229,23 @@ class Oracle:
         s = np.zeros(m, np.float32)
         self.lib.to_rmsnorm_quant(_p(a, f32p), _p(ww, f32p), m, k, eps, int(zero_centered), _p(q, f32p), _p(s, f32p))
         return q.reshape(m, k), s
+
+    def compute_zero_bitmap(self, packed_row, k):
+        b = np.ascontiguousarray(packed_row, np.uint8).reshape(-1)
+        nb = (k + 255) // 256
+        words = np.zeros((nb + 31) // 32, np.uint32)
+        rc = self.lib.to_compute_zero_bitmap(_p(b, u8p), b.size, k, words.ctypes.data_as(C.POINTER(C.c_uint32)), words.size)
+        return rc, words
+
+    def compute_zero_bitmaps(self, packed, n, k, row_bytes, words_len=None):
+        b = np.ascontiguousarray(packed, np.uint8).reshape(-1)
+        nb = (k + 255) // 256
+        if words_len is None:
+            words_len = n * ((nb + 31) // 32)
+        words = np.zeros(max(words_len, 1), np.uint32)
+        rc = self.lib.to_compute_zero_bitmaps(_p(b, u8p), b.size, n, k, row_bytes,
+                                              words.ctypes.data_as(C.POINTER(C.c_uint32)), words_len)
+        return rc, words[:words_len]
 
     def upload_check(self, packed, n, k, fmt):
         b = np.ascontiguousarray(packed, np.uint8)

@@ -6,7 +6,8 @@ this package is the thin host mirror of the reference's adapter interface over i
 from . import _lib
 from .backend import (BACKENDS, Backend, BackendEntry, BackendError, DeviceArray, DeviceBuffer, DeviceCaps,
                       GemmShape, InvalidInput, Linear, Mi355xBackend, Mi355xBuffer, MpGemm, MpGemmProjectedVjp, OutOfMemory,
-                      Registry, ShapeMismatch, TernaryFormat, UnsupportedFormat, convert_i2s_to_tq2_0, pack_rows,
+                      Registry, ShapeMismatch, TernaryFormat, UnsupportedFormat, compute_zero_bitmaps, convert_i2s_to_tq2_0,
+                      pack_rows,
                       packed_len, unpack_rows)
 from .gguf import GgufError, GgufErrorKind, GgufFile, TensorInfo, read_gguf
 from .linear import TernaryLinear

@@ -56,12 +56,15 @@ SIGNATURES = {
     "tk_packed_len": (sz, [sz, sz, C.c_int]),
     "tk_pack_rows": (C.c_int, [vp, sz, sz, sz, C.c_int, vp, sz]),
     "tk_unpack_rows": (C.c_int, [vp, sz, sz, sz, C.c_int, vp, sz]),
+    "tk_compute_zero_bitmaps": (C.c_int, [vp, sz, sz, sz, sz, vp, sz]),
     "tk_upload_weights": (C.c_int, [vp, vp, sz, sz, sz, C.c_int, C.POINTER(vp)]),
     "tk_free_weights": (None, [vp]),
     "tk_weights_len_bytes": (sz, [vp]),
     "tk_weights_n": (sz, [vp]),
     "tk_weights_k": (sz, [vp]),
     "tk_weights_format": (C.c_int, [vp]),
+    "tk_set_zero_skip": (C.c_int, [vp, C.c_int]),
+    "tk_weights_zero_chunks": (C.c_int, [vp, C.POINTER(sz), C.POINTER(sz), C.POINTER(C.c_int)]),
     "tk_weights_download_trits": (C.c_int, [vp, vp, vp, sz]),
     "tk_mpgemm": (C.c_int, [vp, vp, sz, vp, vp, sz, sz, sz, sz, C.c_int, vp, sz]),
     "tk_mpgemm_with_act_quant": (C.c_int, [vp, vp, sz, vp, vp, sz, sz, sz, sz, C.c_int, vp, sz]),

@@ -190,6 +190,12 @@ class Mi355xBuffer(DeviceBuffer):
     def format(self):
         return TernaryFormat(L.load().tk_weights_format(self._h))
 
+    def zero_chunks(self):
+        """(all-zero 1-KiB chunks, chunks, whether the upload kept a skip map for them)."""
+        z, t, kept = C.c_size_t(0), C.c_size_t(0), C.c_int(0)
+        _check(L.load().tk_weights_zero_chunks(self._h, C.byref(z), C.byref(t), C.byref(kept)))
+        return z.value, t.value, bool(kept.value)
+
     def download_trits(self):
         out = np.empty(self.n * self.k, np.int8)
         _check(L.load().tk_weights_download_trits(self._backend._ctx, self._h, out.ctypes.data, out.size))
@@ -518,6 +524,10 @@ class Mi355xBackend:
         """0 automatic, 2 or 4 output tiles per wave of the one-plane prefill kernel."""
         _check(self._lib.tk_set_gemm_tiles(self._ctx, tiles))
 
+    def set_zero_skip(self, mode):
+        """Later uploads: 0 keep a zero-chunk map by the 0.5% threshold, 1 never, 2 always."""
+        _check(self._lib.tk_set_zero_skip(self._ctx, mode))
+
     def set_stream_min_groups(self, groups):
         _check(self._lib.tk_set_stream_min_groups(self._ctx, groups))
 
@@ -548,6 +558,20 @@ def pack_rows(trits, n, k, format=TernaryFormat.Tq2_0):
     out = np.empty(packed_len(n, k, format), np.uint8)
     _check(L.load().tk_pack_rows(t.ctypes.data, t.size, n, k, int(format), out.ctypes.data, out.size))
     return out
+
+
+def compute_zero_bitmaps(packed, n, k, row_bytes):
+    """Per-row zero-block bitmaps of packed TQ2_0 rows (crates/tritium-format/src/tq2.rs:134-181):
+    uint32 words, ceil(nb/32) per row."""
+    b = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+    nb = (k + 255) // 256
+    want = n * ((nb + 31) // 32)
+    # the library checks the rows against the buffer before it touches the words: an absurd n is
+    # refused there, so only a believable word count is allocated here
+    words = np.zeros(want if nb and n * row_bytes <= b.size else 0, np.uint32)
+    _check(L.load().tk_compute_zero_bitmaps(b.ctypes.data, b.size, n, k, row_bytes, words.ctypes.data,
+                                            min(want, (1 << 63) - 1)))
+    return words
 
 
 def convert_i2s_to_tq2_0(payload, n, k):

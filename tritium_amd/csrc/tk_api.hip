@@ -77,6 +77,8 @@ struct tk_ctx {
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
   int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
+  int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
+  unsigned *d_count = nullptr;  // a device counter for the uploads
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum;
   int *d_invalid = nullptr;
@@ -95,7 +97,9 @@ static void ctx_release(tk_ctx *ctx) {
 
 struct tk_weights {
   tk_ctx *ctx;
-  uint8_t *codes;
+  uint8_t *codes;           // n_tiles * nb chunks of 1 KiB, then one chunk of all-zero trits (0x55)
+  uint32_t *zero_map;       // one bit per chunk, set = all-zero trits; null when too few chunks are zero
+  size_t zero_chunks;       // how many chunks are zero (counted at upload whether or not the map is kept)
   float *block_scales;  // [(tile, K block), 16 rows] f32, only for uploads that keep the block scales
   size_t n, k, nb, n_tiles, len_bytes;
   int format;
@@ -223,13 +227,14 @@ extern "C" int tk_init(int device, tk_ctx **out) {
     return tk_fail(TK_ERR_BACKEND, "hipStreamCreate: %s", hipGetErrorString(e));
   }
   void *p = nullptr;
-  int rc = dev_malloc(sizeof(int), &p);
+  int rc = dev_malloc(2 * sizeof(int), &p);
   if (rc) {
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return rc;
   }
   ctx->d_invalid = (int *)p;
+  ctx->d_count = (unsigned *)p + 1;
   void *sp = nullptr;
   e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));  // device `device` is current: its copy of the array
   if (e != hipSuccess || !sp) {
@@ -315,6 +320,14 @@ extern "C" int tk_set_gemm_tiles(tk_ctx *ctx, int tiles) {
   return TK_OK;
 }
 
+extern "C" int tk_set_zero_skip(tk_ctx *ctx, int mode) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_zero_skip: null context");
+  if (mode < 0 || mode > 2) return tk_fail(TK_ERR_INVALID_INPUT, "zero_skip=%d - use 0 (by threshold), 1 (never) or 2 (always)", mode);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->zero_skip = mode;
+  return TK_OK;
+}
+
 extern "C" int tk_set_flow_ring(tk_ctx *ctx, int positions) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_ring: null context");
   if (positions != 0 && (positions < 2 || positions > 5))
@@ -379,18 +392,24 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
   const size_t n_tiles = (n + 15) / 16;
-  const size_t code_bytes = n_tiles * nb * TK_CHUNK_BYTES;
-  void *codes = nullptr, *raw = nullptr, *bscales = nullptr;
-  TKCHK(dev_malloc(code_bytes, &codes));
+  const size_t n_chunks = n_tiles * nb, code_bytes = n_chunks * TK_CHUNK_BYTES;
+  const size_t map_words = (n_chunks + 31) / 32;
+  void *codes = nullptr, *raw = nullptr, *bscales = nullptr, *zmap = nullptr;
+  TKCHK(dev_malloc(code_bytes + TK_CHUNK_BYTES, &codes));  // + the resident all-zero chunk
   int rc = dev_malloc(packed_len, &raw);
   if (!rc && keep_block_scales) rc = dev_malloc(n_tiles * nb * 16 * sizeof(float), &bscales);
+  if (!rc && ctx->zero_skip != 1 && n_chunks) rc = dev_malloc(map_words * 4, &zmap);
   if (rc) {
     (void)hipFree(codes);
     if (raw) (void)hipFree(raw);
+    if (bscales) (void)hipFree(bscales);
     return rc;
   }
   int invalid = INT32_MAX;
-  hipError_t e = hipSuccess;
+  unsigned zero_chunks = 0;
+  hipError_t e = hipMemsetAsync((uint8_t *)codes + code_bytes, 0x55, TK_CHUNK_BYTES, ctx->stream);
+  if (e == hipSuccess && zmap) e = hipMemsetAsync(zmap, 0, map_words * 4, ctx->stream);
+  if (e == hipSuccess && zmap) e = hipMemsetAsync(ctx->d_count, 0, sizeof(unsigned), ctx->stream);
   if (packed_len) e = hipMemcpyAsync(raw, packed, packed_len, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) e = hipMemcpyAsync(ctx->d_invalid, &invalid, sizeof invalid, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) {
@@ -400,20 +419,35 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
     else
       e = tk_launch_relayout_tq1(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb);
   }
+  if (e == hipSuccess && zmap)
+    e = tk_launch_zero_chunk_map(ctx->stream, (const uint8_t *)codes, n_chunks, (uint32_t *)zmap, ctx->d_count);
+  if (e == hipSuccess && zmap)
+    e = hipMemcpyAsync(&zero_chunks, ctx->d_count, sizeof zero_chunks, hipMemcpyDeviceToHost, ctx->stream);
   if (e == hipSuccess) e = hipMemcpyAsync(&invalid, ctx->d_invalid, sizeof invalid, hipMemcpyDeviceToHost, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   (void)hipFree(raw);
+  // The map is worth carrying when enough chunks are zero: the reference's threshold for its per-row
+  // bitmaps, BITMAP_MIN_ZERO_BLOCK_FRAC = 0.005 (crates/tritium-cuda/src/cuda/mod.rs:384-405), applied
+  // to the 16-row chunks this layout streams.
+  if (zmap && !(ctx->zero_skip == 2 || (double)zero_chunks >= 0.005 * (double)n_chunks)) {
+    (void)hipFree(zmap);
+    zmap = nullptr;
+  }
   if (e != hipSuccess) {
     (void)hipFree(codes);
     if (bscales) (void)hipFree(bscales);
+    if (zmap) (void)hipFree(zmap);
     return tk_fail(TK_ERR_BACKEND, "upload_weights: %s", hipGetErrorString(e));
   }
   tk_weights *w = new (std::nothrow) tk_weights();
   if (!w) {
     (void)hipFree(codes);
     if (bscales) (void)hipFree(bscales);
+    if (zmap) (void)hipFree(zmap);
     return tk_fail(TK_ERR_BACKEND, "tk_upload_weights: host allocation failed");
   }
+  w->zero_map = (uint32_t *)zmap;
+  w->zero_chunks = zero_chunks;
   w->ctx = ctx;
   w->codes = (uint8_t *)codes;
   w->block_scales = (float *)bscales;
@@ -492,11 +526,19 @@ extern "C" void tk_free_weights(tk_weights *w) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(w->codes);
     if (w->block_scales) (void)hipFree(w->block_scales);
+    if (w->zero_map) (void)hipFree(w->zero_map);
     delete w;
   }
   ctx_release(ctx);
 }
 extern "C" size_t tk_weights_len_bytes(const tk_weights *w) { return w ? w->len_bytes : 0; }
+extern "C" int tk_weights_zero_chunks(const tk_weights *w, size_t *zero, size_t *total, int *map_kept) {
+  if (!w) return tk_fail(TK_ERR_INVALID_INPUT, "tk_weights_zero_chunks: null buffer");
+  if (zero) *zero = w->zero_chunks;
+  if (total) *total = w->n_tiles * w->nb;
+  if (map_kept) *map_kept = w->zero_map ? 1 : 0;
+  return TK_OK;
+}
 extern "C" size_t tk_weights_n(const tk_weights *w) { return w ? w->n : 0; }
 extern "C" size_t tk_weights_k(const tk_weights *w) { return w ? w->k : 0; }
 extern "C" int tk_weights_format(const tk_weights *w) { return w ? w->format : 0; }
@@ -586,10 +628,14 @@ static bool flow_wide(const tk_ctx *ctx, int planes, int rt, size_t nb, size_t r
 static int flow_runs_per_wave(bool wide, int planes, int rt, size_t rows) {
   return wide ? tk_flow32_runs_per_wave() : tk_flow_runs_per_wave(planes, rt, (int)rows);
 }
-static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds, size_t rows) {
+// zmap_tiles > 0: some plane of the launch carries a zero-chunk map; a workgroup of that many tiles stages
+// the words of its chunks behind the operand rows (16x16x64 form only; the other kernels ignore the maps)
+static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds, size_t rows, size_t zmap_tiles = 0,
+                          size_t zmap_nb = 0) {
   cfg->wide_mfma = wide ? 1 : 0;
   cfg->tw = flow_runs_per_wave(wide, cfg->planes, cfg->rt, rows);
   cfg->lds_bytes = flow_lds + (wide ? kFlowWideExtraLds : 0);
+  if (!wide && zmap_tiles) cfg->lds_bytes += (size_t)cfg->planes * tk_flow_zmap_words(zmap_tiles, zmap_nb) * 4;
   if (wide && cfg->ring > 4) cfg->ring = 4;
 }
 
@@ -696,6 +742,8 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
   for (int p = 0; p < layer->n_planes; ++p) {
     pr.codes[p] = layer->planes[p]->codes;
     pr.scales[p] = layer->scales[p];
+    pr.zmap[p] = layer->planes[p]->zero_map;
+    if (pr.zmap[p]) pr.zskip = 1;
   }
   pr.n = (int)n;
   pr.k = (int)k;
@@ -880,7 +928,10 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.lds_bytes = flow_lds;
     cfg.waves = flow_waves(flow_lds);
     cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R));
-    flow_cfg_form(&cfg, wide, flow_lds, R);
+    size_t ztiles = pr.zskip && !wide ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0;
+    if (ztiles && flow_lds + (size_t)cfg.planes * tk_flow_zmap_words(ztiles, nb) * 4 > kLdsFlowMax) ztiles = 0;
+    if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or the 32x32x32 form): plain loads
+    flow_cfg_form(&cfg, wide, flow_lds, R, ztiles, nb);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -1558,7 +1609,14 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
       flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, planes, rt, prows_max));
-      flow_cfg_form(&flow_cfg, pwide, pflds, prows_max);
+      size_t ztiles = 0;
+      for (size_t i = 0; i < count; ++i)
+        if (plans[i].flow_ok && plans[i].pr.zskip && !pwide) ztiles = pper;
+      if (ztiles && pflds + (size_t)planes * tk_flow_zmap_words(ztiles, pnb_max) * 4 > kLdsFlowMax) ztiles = 0;
+      if (!ztiles)
+        for (size_t i = 0; i < count; ++i)
+          if (plans[i].flow_ok) plans[i].pr.zskip = 0;
+      flow_cfg_form(&flow_cfg, pwide, pflds, prows_max, ztiles, pnb_max);
     }
   } else if (variant != DECODE_KSPLIT) {
     const unsigned per = variant == DECODE_FLOW ? fper : tpw;
@@ -1574,6 +1632,15 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       for (unsigned j = 0; j < gi; ++j) wg_prob.push_back((int)i);
       groups_total += gi;
     }
+  }
+  // zero-chunk maps in a flow-form group: room for the words of one workgroup's chunks behind the rows
+  size_t group_ztiles = 0;
+  if (variant == DECODE_FLOW) {
+    for (size_t i = 0; i < count; ++i)
+      if (plans[i].pr.zskip && !wide) group_ztiles = fper;
+    if (group_ztiles && flds + (size_t)planes * tk_flow_zmap_words(group_ztiles, nb_max) * 4 > kLdsFlowMax) group_ztiles = 0;
+    if (!group_ztiles)
+      for (size_t i = 0; i < count; ++i) plans[i].pr.zskip = 0;
   }
   tk_group *g = new (std::nothrow) tk_group();
   if (!g) return tk_fail(TK_ERR_BACKEND, "tk_group_create: host allocation failed");
@@ -1672,7 +1739,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     }
     g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, planes, rt, rows_max));
   }
-  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds, rows_max);
+  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds, rows_max, group_ztiles, nb_max);
   ctx->refs.fetch_add(1);
   *out = g;
   return TK_OK;

@@ -86,6 +86,30 @@ extern "C" size_t tk_packed_len(size_t n, size_t k, int format) {
   return total;
 }
 
+// compute_zero_bitmaps (crates/tritium-format/src/tq2.rs:134-181): one bit per 256-trit block and row,
+// set when the block's 64 code bytes are all 0x55. Word `r * ceil(nb/32) + b/32`, bit `b % 32`.
+extern "C" int tk_compute_zero_bitmaps(const uint8_t *packed, size_t packed_len, size_t n, size_t k, size_t row_bytes,
+                                       uint32_t *words, size_t words_len) {
+  const size_t nb = k / kBlock + (k % kBlock != 0), wpr = nb / 32 + (nb % 32 != 0);
+  if (nb == 0) return TK_OK;  // nothing to describe, whatever n says (tq2.rs:146-148)
+  size_t min_row, need, want;
+  if (__builtin_mul_overflow(nb, (size_t)66, &min_row) || row_bytes < min_row)
+    return tk_fail(TK_ERR_INVALID_INPUT, "zero bitmap: row of %zu bytes is shorter than the %zu blocks of k=%zu", row_bytes, nb, k);
+  if (__builtin_mul_overflow(n, row_bytes, &need) || packed_len < need)
+    return tk_fail(TK_ERR_INVALID_INPUT, "zero bitmap: %zu bytes do not hold %zu rows of %zu", packed_len, n, row_bytes);
+  if (__builtin_mul_overflow(n, wpr, &want) || words_len != want) return tk_fail_mismatch(want, words_len);
+  if ((!packed && need) || (!words && want)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_compute_zero_bitmaps: null pointer");
+  std::memset(words, 0, want * sizeof(uint32_t));
+  for (size_t r = 0; r < n; ++r)
+    for (size_t b = 0; b < nb; ++b) {
+      const uint8_t *qs = packed + r * row_bytes + b * 66;
+      bool zero = true;
+      for (size_t i = 0; i < 64 && zero; ++i) zero = qs[i] == 0x55;
+      if (zero) words[r * wpr + b / 32] |= 1u << (b % 32);
+    }
+  return TK_OK;
+}
+
 extern "C" int tk_pack_rows(const int8_t *trits, size_t trits_len, size_t n, size_t k, int format, uint8_t *out,
                             size_t out_len) {
   const size_t bb = block_bytes(format);

@@ -39,6 +39,11 @@ struct TkProblem {
   // of every operand row over each K block [nb][R]
   const float *bscale[TK_MAX_PLANES];
   const int32_t *blocksum;
+  // Zero-chunk skip (flow kernel): per plane, one bit per 1-KiB chunk (tile * nb + K block), set when all
+  // 16 rows of the tile hold only zero trits in that block, or null; a chunk whose bit is set is loaded
+  // from the resident all-zero chunk behind the plane's last chunk instead (same bytes, no memory traffic).
+  const uint32_t *zmap[TK_MAX_PLANES];
+  int zskip;                 // any plane has a map
   void *out;                 // [M,N]
   const void *residual;      // [M,N] in the output's element type, added to every output (one f32 add), or null
   int n, k, nb, R, M;
@@ -99,6 +104,10 @@ extern "C++" {
 hipError_t tk_launch_relayout_tq2(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb,
                                   int *invalid_row, float *block_scales);
 hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *codes, size_t n, size_t nb);
+// chunk map of a re-laid-out plane: bit c of map set iff chunk c is all 0x55; *count receives the set bits
+hipError_t tk_launch_zero_chunk_map(hipStream_t s, const uint8_t *codes, size_t chunks, uint32_t *map, unsigned *count);
+// LDS bytes the flow kernel needs for the maps of one workgroup: planes * this many words
+size_t tk_flow_zmap_words(size_t tiles_per_wg, size_t nb);
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
                                   int8_t *trits);
 // uniform_m > 0 says that entry j of the table starts at token j * uniform_m (all tensors equally long).

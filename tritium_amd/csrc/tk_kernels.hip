@@ -646,19 +646,39 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
     last_off[tw] = min(run_last, plane_last) * 1024u + (unsigned)lane * 16u;
   }
 
+  // Zero-chunk skip: the map words of the chunks this workgroup can ask for sit in LDS behind the
+  // operand rows (staged below); a request for a chunk whose bit is set goes to the all-zero chunk
+  // that follows the plane's last chunk -- the same bytes from the cache instead of from memory, so
+  // neither the arithmetic nor the number of loads per position changes.
+  const bool zskip = pr.zskip != 0;
+  const uint32_t *lds_z = (const uint32_t *)(smem + (size_t)nb * 256 * R);
+  const unsigned zero_off = (unsigned)n_tiles * (unsigned)nb * 1024u + (unsigned)lane * 16u;
+  const unsigned wg_first = (unsigned)(blockIdx.x - pr.group_begin) * (unsigned)(NW * TW * S);
+  const unsigned zc0 = min(wg_first, (unsigned)n_tiles - 1u) * (unsigned)nb;
+  const unsigned zc1 = min(wg_first + (unsigned)(NW * TW * S), (unsigned)n_tiles) * (unsigned)nb;  // exclusive
+  const unsigned zw0 = zc0 >> 5, zwords = zskip ? ((max(zc1, zc0 + 1u) - 1u) >> 5) - zw0 + 1u : 0u;
   uint4 ring[DR][TW][P];
-  auto request = [&](int slot, bool real, bool tile_start) {
+  auto request = [&](int slot, bool real, bool tile_start, bool use_map) {
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       roff[tw] += tile_start ? skip : 0u;
       const unsigned off = min(roff[tw], last_off[tw]);
 #pragma unroll
-      for (int p = 0; p < P; ++p) ring[slot][tw][p] = gload16(codes[p] + (size_t)off);
+      for (int p = 0; p < P; ++p) {
+        unsigned o = off;
+        if (use_map && zskip) {
+          const unsigned chunk = (unsigned)__builtin_amdgcn_readfirstlane((int)(off >> 10));
+          const unsigned wi = (chunk >> 5) - zw0;
+          const uint32_t word = wi < zwords ? lds_z[(unsigned)p * zwords + wi] : 0u;
+          if ((word >> (chunk & 31u)) & 1u) o = zero_off;
+        }
+        ring[slot][tw][p] = gload16(codes[p] + (size_t)o);
+      }
       roff[tw] += real ? 1024u : 0u;
     }
   };
 #pragma unroll
-  for (int d = 0; d < D; ++d) request(d, d < nb, d == 0);
+  for (int d = 0; d < D; ++d) request(d, d < nb, d == 0, false);  // the map is not staged yet
 
   // stage every operand row of the problem in LDS
   {
@@ -666,6 +686,13 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
     uint4 *lds4w = (uint4 *)smem;
     const int cnt = nb * 16 * R;
     for (int idx = threadIdx.x; idx < cnt; idx += (int)blockDim.x) lds4w[idx] = gload16(ap4 + idx);
+    if (zskip) {
+      uint32_t *lz = (uint32_t *)(smem + (size_t)nb * 256 * R);
+      for (unsigned idx = threadIdx.x; idx < (unsigned)P * zwords; idx += blockDim.x) {
+        const unsigned p = idx / zwords, w = idx - p * zwords;
+        lz[idx] = pr.zmap[p] ? gload(pr.zmap[p] + zw0 + w) : 0u;
+      }
+    }
   }
   RowConst rc[RT];
   unsigned any_flag = 0;
@@ -708,7 +735,7 @@ __global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, co
         {  // request the position D ahead (slot (d + D) % DR, consumed at the previous position)
           int kb2 = kb + D;
           if (kb2 >= nbpad) kb2 -= nbpad;
-          request((d + D) % DR, kb2 < nb, kb2 == 0);
+          request((d + D) % DR, kb2 < nb, kb2 == 0, true);
         }
         if (kb < nb) {
 #pragma unroll
@@ -2737,6 +2764,20 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_i8_kernel(TkPrep single, const 
   if (threadIdx.x == 0) pp.rowsum[row] = sum;
 }
 
+// One wave per 1-KiB chunk of a re-laid-out plane: the chunk is zero when all of its bytes are 0x55
+// (rows past n were filled with that, so they do not stand in the way).
+__global__ __launch_bounds__(TK_WG) void tk_zero_chunk_map_kernel(const uint8_t *__restrict__ codes, size_t chunks,
+                                                                  uint32_t *__restrict__ map, unsigned *__restrict__ count) {
+  const size_t chunk = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (chunk >= chunks) return;
+  const uint4 v = gload16(codes + chunk * TK_CHUNK_BYTES + (size_t)(threadIdx.x & 63) * 16);
+  const bool zero = v.x == 0x55555555u && v.y == 0x55555555u && v.z == 0x55555555u && v.w == 0x55555555u;
+  if (__all(zero) && (threadIdx.x & 63) == 0) {
+    atomicOr(map + (chunk >> 5), 1u << (chunk & 31));
+    atomicAdd(count, 1u);
+  }
+}
+
 __global__ void tk_copy_kernel_dev(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
   size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
@@ -2763,6 +2804,16 @@ hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *co
   hipLaunchKernelGGL(tk_relayout_tq1_kernel, dim3(grid_for(pieces, 256)), dim3(256), 0, s, raw, codes, n, nb, pieces);
   return hipGetLastError();
 }
+
+hipError_t tk_launch_zero_chunk_map(hipStream_t s, const uint8_t *codes, size_t chunks, uint32_t *map, unsigned *count) {
+  if (!chunks) return hipSuccess;
+  hipLaunchKernelGGL(tk_zero_chunk_map_kernel, dim3(grid_for(chunks, 4)), dim3(TK_WG), 0, s, codes, chunks, map, count);
+  return hipGetLastError();
+}
+
+// words of one plane's map a flow workgroup of `tiles_per_wg` tiles can touch (its chunk range may start
+// and end inside a word)
+size_t tk_flow_zmap_words(size_t tiles_per_wg, size_t nb) { return (tiles_per_wg * nb + 31) / 32 + 1; }
 
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb, int8_t *trits) {
   if (!(n * k)) return hipSuccess;
