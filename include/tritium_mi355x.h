@@ -436,6 +436,11 @@ int tk_set_flow_mfma(tk_ctx *ctx, int rows);
  * leave fewer than four workgroups per CU), 2 or 4 to force. A tuning and test knob: both forms give
  * identical bits. */
 int tk_set_gemm_tiles(tk_ctx *ctx, int tiles);
+/* K slices of the prefill kernel in single launches: 0 = chosen per launch (a launch with fewer
+ * workgroups than CUs is cut into about one workgroup per CU, at least two K blocks per slice), 1 =
+ * never split, 2..64 = that many slices where K allows. Integer partial sums, added by the last
+ * workgroup to arrive: identical bits. A tuning and test knob. */
+int tk_set_gemm_ksplit(tk_ctx *ctx, int slices);
 /* The K-split decode kernel has the finer grain (a single narrow layer), the streaming and flow
  * kernels walk whole output tiles per wave (launches that fill the chip): the latter are taken when
  * a launch needs at least this many workgroups; default = the device's CU count. No counterpart

@@ -161,3 +161,59 @@ def test_gemm_tiles_knob_rejects_other_values(backend):
     for bad in (1, 3, 8, -2):
         with pytest.raises(T.InvalidInput):
             backend.set_gemm_tiles(bad)
+
+
+@pytest.mark.parametrize("slices", [2, 3, 5, 0])
+@pytest.mark.parametrize("m,n,k,planes,tiles", [(64, 200, 2816, 3, 0), (40, 1040, 4352, 1, 2), (40, 1040, 4352, 1, 4),
+                                                  (100, 50, 1300, 2, 0), (130, 131, 1024, 1, 0)])
+def test_prefill_kernel_k_split(backend, oracle, slices, m, n, k, planes, tiles):
+    """Single launches of the prefill kernel with K cut into slices (tk_gemm32_kernel<P,NT,false,true>): int32
+    partial sums meet in a workspace and the last workgroup to arrive finishes the tile. Bits equal the
+    unsplit kernel's and the CPU composition's; a second call reuses the arrival counters (they must be
+    back at zero); ragged slice counts (11, 17, 6, 4 K blocks over 2, 3, 5 slices) included."""
+    print("case k-split", slices, m, n, k, planes, tiles, flush=True)
+    backend.set_gemm_tiles(tiles)
+    rng = np.random.default_rng(slices * 1000 + m + n + k)
+    ws, scs, packed = _planes(rng, n, k, planes)
+    layer = backend.linear(packed, scs, n, k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[1, 3] = np.nan
+    dact = backend.to_device(act, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k).reshape(m, n)
+    fin = ~np.isnan(want)
+    backend.set_gemm_ksplit(1)
+    d0 = backend.empty(m * n, "f32")
+    backend.linear_a8(layer, dact, m, d0)
+    backend.set_gemm_ksplit(slices)
+    try:
+        for dtype in ("f32", "bf16"):
+            d1 = backend.empty(m * n, dtype)
+            for _ in range(2):
+                backend.linear_a8(layer, dact, m, d1)
+                got = d1.to_host().reshape(m, n)
+                if dtype == "f32":
+                    assert same_bits(got[fin], want[fin]) and same_bits(got[fin], d0.to_host().reshape(m, n)[fin])
+                    assert (np.isnan(got) == ~fin).all()
+                else:
+                    assert (got[fin] == f32_to_bf16_bits(want).reshape(m, n)[fin]).all()
+            d1.free()
+        if planes == 1:  # raw accumulators
+            q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+            dq, dacc = backend.to_device(q, "i8"), backend.empty(m * n, "i32")
+            backend.linear_i8(layer, dq, None, m, dacc)
+            assert (dacc.to_host().reshape(m, n) == oracle.int8_accumulators(packed[0], FMT_TQ2_0, q, m, n, k)).all()
+            dq.free()
+            dacc.free()
+        # the float contract through the same split
+        mf = min(m, 30)
+        df = backend.empty(mf * n, "f32")
+        backend.linear_float(layer, dact, mf, df)
+        wantf = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act[:mf], mf, n, k)
+        finf = ~np.isnan(wantf)
+        assert accepts(df.to_host().reshape(mf, n)[finf], wantf[finf], rel=1e-4, floor=1.0).all()
+        df.free()
+    finally:
+        backend.set_gemm_ksplit(0)
+    for a in (dact, d0):
+        a.free()
+    layer.free()

@@ -524,6 +524,10 @@ class Mi355xBackend:
         """0 automatic, 2 or 4 output tiles per wave of the one-plane prefill kernel."""
         _check(self._lib.tk_set_gemm_tiles(self._ctx, tiles))
 
+    def set_gemm_ksplit(self, slices):
+        """0 automatic, 1 off, 2..64 K slices of the prefill kernel in single launches."""
+        _check(self._lib.tk_set_gemm_ksplit(self._ctx, slices))
+
     def set_zero_skip(self, mode):
         """Later uploads: 0 keep a zero-chunk map by the 0.5% threshold, 1 never, 2 always."""
         _check(self._lib.tk_set_zero_skip(self._ctx, mode))

@@ -77,10 +77,11 @@ struct tk_ctx {
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
   int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
+  int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
   unsigned *d_count = nullptr;  // a device counter for the uploads
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
-  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum;
+  DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum, kpart, kcount;
   int *d_invalid = nullptr;
   // The context itself plus every weight buffer and group created on it: tk_destroy gives up the
   // context's own reference, the stream and this record live until the last of them is released, so
@@ -256,7 +257,7 @@ extern "C" void tk_destroy(tk_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     DevBuf *bufs[] = {&ctx->ap, &ctx->rowsum, &ctx->fscale, &ctx->aux, &ctx->exps,
                       &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp,
-                      &ctx->ynorm, &ctx->blocksum};
+                      &ctx->ynorm, &ctx->blocksum, &ctx->kpart, &ctx->kcount};
     for (DevBuf *b : bufs) {
       if (b->p) (void)hipFree(b->p);
       b->p = nullptr;
@@ -317,6 +318,14 @@ extern "C" int tk_set_gemm_tiles(tk_ctx *ctx, int tiles) {
     return tk_fail(TK_ERR_INVALID_INPUT, "gemm_tiles=%d - use 0 (automatic), 2 or 4", tiles);
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->gemm_tiles = tiles;
+  return TK_OK;
+}
+
+extern "C" int tk_set_gemm_ksplit(tk_ctx *ctx, int slices) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_ksplit: null context");
+  if (slices < 0 || slices > 64) return tk_fail(TK_ERR_INVALID_INPUT, "gemm_ksplit=%d - use 0 (automatic), 1 (off) or 2..64", slices);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->gemm_ksplit = slices;
   return TK_OK;
 }
 
@@ -945,6 +954,34 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else if (pl.skinny) {
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
   } else {
+    // A single launch with few workgroups is a latency chain over K per workgroup: cut K into slices.
+    // The partial sums cost 4 bytes per accumulator and slice, so few slices: measured, call incl.
+    // quantization, 64 tokens x 3 planes: 17408 -> 5120 (40 workgroups) 108 us unsplit, 72 / 56 / 54 / 72
+    // with 2 / 4 / 6 / 8 slices; 5120 -> 5120 39 -> 30 us at 4; 5120 -> 1024 (8 workgroups) 39 -> 28 at 4;
+    // 5120 -> 17408 (136 workgroups) is best left alone (42 us; 53 with 2 slices). Rule: split when the
+    // launch has at most a third of the CUs in workgroups, into about three quarters of the CUs, 2..6
+    // slices of at least two K blocks.
+    const unsigned wgs = 8u * (unsigned)pr.sub_m * (unsigned)pr.sub_n;
+    int ksn = 1;
+    if (!static_ws && pr.planes <= 3 && nb >= 4) {
+      if (ctx->gemm_ksplit >= 2) ksn = ctx->gemm_ksplit;
+      else if (ctx->gemm_ksplit == 0 && wgs * 3 <= (unsigned)ctx->info.compute_units) {
+        ksn = (int)((3u * (unsigned)ctx->info.compute_units / 4u) / wgs);
+        ksn = ksn < 2 ? 2 : (ksn > 6 ? 6 : ksn);
+      }
+      if ((size_t)ksn > nb / 2) ksn = (int)(nb / 2);  // every slice holds at least two K blocks (the kernel relies on it)
+    }
+    if (ksn > 1) {
+      const size_t tiles = (size_t)pr.grid_m * (size_t)pr.grid_n;
+      const size_t regs = (size_t)32 * (size_t)pr.planes * (pr.planes == 1 ? (pl.cfg.gemm_nt == 2 ? 1 : 2) : 1);  // 2 * NP * 16
+      const bool fresh = tiles * 4 > ctx->kcount.cap;
+      TKCHK(ensure(ctx, ctx->kpart, tiles * (size_t)ksn * regs * 256 * 4));
+      TKCHK(ensure(ctx, ctx->kcount, tiles * 4));
+      if (fresh) HIPCHK(hipMemsetAsync(ctx->kcount.p, 0, ctx->kcount.cap, ctx->stream));  // the kernel leaves it zero
+      pr.ksplit = ksn;
+      pr.kpart = (int32_t *)ctx->kpart.p;
+      pr.kcount = (int *)ctx->kcount.p;
+    }
     HIPCHK(tk_launch_gemm(ctx->stream, &pr, nullptr, nullptr, pl.cfg));
   }
   return TK_OK;

@@ -54,6 +54,13 @@ struct TkProblem {
   int kc;                    // K blocks staged in LDS per pass (decode kernels)
   int group_begin;           // streaming / flow kernels: first workgroup index of this problem
   int run_tiles;             // flow kernel: consecutive tiles per run (S)
+  // prefill kernel, K split (single launches with too few workgroups to fill the chip): every output tile
+  // is computed by `ksplit` workgroups, each over a slice of the K blocks; their int32 partial sums meet in
+  // kpart, and the workgroup that arrives last (kcount) adds them up -- integer adds, so the bits are those
+  // of the unsplit kernel -- and runs the epilogue. 0 or 1 = no split.
+  int ksplit;
+  int32_t *kpart;            // [tile][slice][accumulator register][thread]
+  int *kcount;               // [tile], zero between launches
   int grid_m, grid_n;        // GEMM: row blocks and column blocks
   int xr, sub_m, sub_n;      // GEMM: XCDs along M, and the tile sub-grid one XCD owns
 };

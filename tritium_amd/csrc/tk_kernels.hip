@@ -1565,10 +1565,11 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
 #define TK_GEMM32_OCC(P) ((P) >= 3 ? 2 : 3)
 #endif
 
-template <int P, int NT, bool TABLE>
+template <int P, int NT, bool TABLE, bool KSPLIT = false>
 __global__ __launch_bounds__(TK_GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(TK_GEMM32_OCC(P), TK_GEMM32_OCC(P)))) void
 tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, const int *__restrict__ wg_prob) {
   static_assert(NT % 2 == 0, "tiles are processed in pairs");
+  static_assert(!(TABLE && KSPLIT), "the K split is for single launches");
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
   const TkHot hot = make_hot(pr);
   const uint8_t *codes[P];
@@ -1586,12 +1587,19 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // three A blocks of 16 KiB + row constants
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, h = (lane >> 4) & 1, kappa = lane >> 5;
-  const int nb = pr.nb, R = pr.R;
+  const int nb_full = pr.nb, R = pr.R;
   // XCD x = id % 8 owns a compact sub-grid of sub_m x sub_n tiles. Inside it the slots walk bands of
   // TK_GEMM_BAND row tiles: down the band first, then along the columns, so the ~100 workgroups an
   // XCD holds at a time are a band x 12 patch (8 A row blocks + 12 weight column blocks to keep in
   // its L2) instead of a full column strip (32 + 3).
-  const int xcd = wg & 7, slot = wg >> 3;
+  // K split: the slices of a tile are consecutive slots of one XCD (they meet in its L2).
+  const int ksn = KSPLIT ? pr.ksplit : 1;
+  const int xcd = wg & 7, slot_k = wg >> 3;
+  const int slot = KSPLIT ? slot_k / ksn : slot_k, ks = KSPLIT ? slot_k - slot * ksn : 0;
+  // slice ks takes the K blocks [ks * nb / ksn, (ks + 1) * nb / ksn): at least two each (the host keeps
+  // ksn <= nb / 2), so the pipeline's first two stages are loaded unconditionally
+  const int kb_begin = KSPLIT ? ks * nb_full / ksn : 0;
+  const int nb = KSPLIT ? (ks + 1) * nb_full / ksn - kb_begin : nb_full;
   const int sub_m = pr.sub_m, sub_n = pr.sub_n;
   const int band_sz = TK_GEMM_BAND * sub_n;
   const int band = slot / band_sz, in_band = slot - band * band_sz;
@@ -1609,7 +1617,8 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
 #pragma unroll
   for (int y = 0; y < NP; ++y) {
     const int p = y / HP, nt = (y % HP) * 2 + h;
-    wptr[y] = codes[p] + ((size_t)min(tile0 + nt, n_tiles - 1) * (size_t)nb * 64 + (size_t)(kappa * 16 + r16)) * 16;
+    wptr[y] = codes[p] + ((size_t)min(tile0 + nt, n_tiles - 1) * (size_t)nb_full * 64 + (size_t)(kappa * 16 + r16)) * 16 +
+              (size_t)kb_begin * TK_CHUNK_BYTES;
   }
 
   const unsigned a_lane = (unsigned)min(row0 + lane, R - 1) * 16u;
@@ -1618,7 +1627,7 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
 #pragma unroll
     for (int u = 0; u < SEGS; ++u) {
       const int seg = wave_u * SEGS + u;
-      const uint8_t *seg_base = (const uint8_t *)ap + ((size_t)kb * 16 + seg) * (size_t)rs * 16;  // wave-uniform
+      const uint8_t *seg_base = (const uint8_t *)ap + ((size_t)(kb_begin + kb) * 16 + seg) * (size_t)rs * 16;  // wave-uniform
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(seg_base + a_lane),
                                        (__attribute__((address_space(3))) void *)(smem + ((size_t)slot3 * A4 + (size_t)seg * ROWS) * 16),
                                        16, 0, 0);
@@ -1698,11 +1707,11 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
   };
 #pragma unroll
   for (int q = 0; q < NS - 1; ++q)
-    if (q < nb) {
+    if (KSPLIT || q < nb) {
       load_w(wset[q], q);
       dma_block(q, q);
     }
-  wait_blocks(min(NS - 2, nb - 1));  // block 0 has landed
+  wait_blocks(KSPLIT ? NS - 2 : min(NS - 2, nb - 1));  // block 0 has landed
 #pragma unroll
   for (int q = 0; q < NS; ++q) tie_w(wset[q]);
   __builtin_amdgcn_s_barrier();
@@ -1751,6 +1760,46 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
 
   unsigned tid_e = threadIdx.x;
   asm volatile("" : "+v"(tid_e));
+  if constexpr (KSPLIT) {
+    // Partial sums out, one coalesced KiB per register; the last workgroup of the tile to arrive adds
+    // the others' to its own and goes on to the epilogue. Integer adds: the order does not matter.
+    constexpr int NREG = 2 * NP * 16;
+    const int tile_id = bm * pr.grid_n + bn;
+    int32_t *mine = pr.kpart + ((size_t)tile_id * ksn + ks) * (size_t)(NREG * TK_GEMM_THREADS) + tid_e;
+#pragma unroll
+    for (int rt2 = 0; rt2 < 2; ++rt2)
+#pragma unroll
+      for (int y = 0; y < NP; ++y)
+#pragma unroll
+        for (int c = 0; c < 16; ++c)
+          __hip_atomic_store(mine + ((rt2 * NP + y) * 16 + c) * TK_GEMM_THREADS, acc[rt2][y][c], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    // The partial sums and the counter are accessed with device-scope (cache-coherent) stores, loads and
+    // atomics of their own, so no fence has to write back or invalidate a whole L2 (a device-scope
+    // fence per workgroup costs several times the kernel). Order: all of this workgroup's stores are
+    // acknowledged (vmcnt 0, every thread, then the barrier) before thread 0 counts the arrival; the
+    // last workgroup reads the others' sums only after it has seen every arrival.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int *arrived = (int *)smem;  // the A slots are free after the main loop's last barrier
+    if (tid_e == 0) *arrived = __hip_atomic_fetch_add(pr.kcount + tile_id, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*arrived != ksn - 1) return;
+    for (int k2 = 0; k2 < ksn; ++k2) {
+      if (k2 == ks) continue;
+      int32_t *theirs = pr.kpart + ((size_t)tile_id * ksn + k2) * (size_t)(NREG * TK_GEMM_THREADS) + tid_e;
+#pragma unroll
+      for (int rt2 = 0; rt2 < 2; ++rt2)
+#pragma unroll
+        for (int y = 0; y < NP; ++y)
+#pragma unroll
+          for (int c = 0; c < 16; ++c)
+            acc[rt2][y][c] += __hip_atomic_load(theirs + ((rt2 * NP + y) * 16 + c) * TK_GEMM_THREADS, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (tid_e == 0) __hip_atomic_store(pr.kcount + tile_id, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero again for the next launch
+    __syncthreads();  // `arrived` was read by everyone before the epilogue reuses the LDS
+  }
   tk_gemm32_epilogue<P, NT>(pr, hot, scales, acc, smem, (int)tid_e, bm, bn);
 }
 
@@ -3113,8 +3162,18 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
                           const TkLaunchCfg &cfg) {
   TkProblem dummy = {};
   const TkProblem &sg = single ? *single : dummy;
-  const unsigned wgs = table ? cfg.grid : 8u * (unsigned)sg.sub_m * (unsigned)sg.sub_n;
+  const bool ksplit = !table && sg.ksplit > 1;
+  const unsigned wgs = table ? cfg.grid : 8u * (unsigned)sg.sub_m * (unsigned)sg.sub_n * (ksplit ? (unsigned)sg.ksplit : 1u);
   if (!wgs) return hipSuccess;
+  if (ksplit) {
+    if (cfg.planes == 1 && cfg.gemm_nt == 2) return gemm_launch_one(tk_gemm32_kernel<1, 2, false, true>, s, sg, table, wg_prob, cfg, wgs);
+    switch (cfg.planes) {
+      case 1: return gemm_launch_one(tk_gemm32_kernel<1, 4, false, true>, s, sg, table, wg_prob, cfg, wgs);
+      case 2: return gemm_launch_one(tk_gemm32_kernel<2, 2, false, true>, s, sg, table, wg_prob, cfg, wgs);
+      case 3: return gemm_launch_one(tk_gemm32_kernel<3, 2, false, true>, s, sg, table, wg_prob, cfg, wgs);
+      default: return hipErrorInvalidValue;  // four planes take the 16x16x64 kernel, which has no K split
+    }
+  }
   dim3 grid(wgs), block(TK_GEMM_THREADS);
 #define TK_GEMM_CASE(PP, NTT)                                                                                 \
   if (table) hipLaunchKernelGGL((tk_gemm_kernel<PP, NTT, true>), grid, block, cfg.lds_bytes, s, sg, table, wg_prob); \
