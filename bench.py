@@ -472,6 +472,55 @@ def bench_zero_skip(T, be, rng, iters=60):
     return res
 
 
+def bench_base3(T, be, rng, iters=60):
+    """A/B of the two weight streams of the decode kernel: 2-bit codes (64 bytes per 256 trits of a row) against
+    the base-3 stream (52 bytes, TQ1_0-coded bytes decoded in the kernel), same layers, same activations,
+    128 layer copies per launch, decode kernel alone. configs[0]'s layer uploaded in TQ1_0 (one plane,
+    K=2560, N=6912) and the headline layer (two planes, K=2048, N=8192). GB/s are the 2-bit algorithmic
+    bytes over time for both, so the ratio is the speed-up of the base-3 stream; outputs must carry the
+    same bits."""
+    res = {"workload": f"{COPIES} layer copies per launch, decode kernel alone; GB/s on the 2-bit algorithmic bytes for both streams"}
+    shapes = (("config1_layer_tq1_0", 6912, 2560, 1, T.TernaryFormat.Tq1_0, ((1, "f32", 0), (1, "bf16", 1), (4, "bf16", 1), (16, "bf16", 1))),
+              ("headline_layer", N2, K2, 2, T.TernaryFormat.Tq2_0, ((1, "bf16", 0), (2, "bf16", 0), (4, "bf16", 0), (8, "bf16", 0), (16, "bf16", 1))))
+    for name, n, k, planes, fmt, cases in shapes:
+        host = []
+        for _ in range(2):
+            trits = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7)[:planes]]
+            host.append(([T.pack_rows(w, n, k, fmt) for w in trits], [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in range(planes)]))
+        layers = {}
+        for mode in (0, 2):
+            be.set_base3_stream(mode)
+            layers[mode] = [be.linear(host[i % 2][0], host[i % 2][1], n, k, fmt) for i in range(COPIES)]
+        be.set_base3_stream(0)
+        res[name] = {"base3_bytes_per_plane": layers[2][0].planes[0].base3_bytes(), "two_bit_bytes_per_plane": ((n + 15) // 16) * ((k + 255) // 256) * 1024}
+        for m, dt, gmode in cases:
+            mk = lambda: rng.standard_normal((m, k)).astype(np.float32)
+            acts = [be.to_device(mk() if dt == "f32" else f32_to_bf16_bits(mk()), dt) for _ in range(COPIES)]
+            outs = [be.empty(m * n, "f32") for _ in range(COPIES)]
+            by = COPIES * algorithmic_bytes(m, n, k, planes, 4 if dt == "f32" else 2, 4, a8=(gmode == 1))
+            row, ref = {}, None
+            for mode, tag in ((0, "two_bit"), (2, "base3")):
+                g = be.group([(layers[mode][i], acts[i], m, outs[i]) for i in range(COPIES)], gmode, dt, "f32")
+                g.launch()
+                be.sync()
+                got = outs[COPIES - 1].to_host().copy()
+                if ref is not None and not (got.view(np.uint32) == ref.view(np.uint32)).all():
+                    sys.exit(f"bench.py: base-3 leg: bits differ between the two streams ({name}, batch {m})")
+                ref = got
+                ms = time_calls(be, lambda i: g.launch_parts(False, True), iters)
+                row[tag] = {"kernel_us_per_launch": round(ms * 1e3, 1), "GB/s": round(by / ms / 1e6, 1)}
+                g.destroy()
+            row["base3_over_two_bit"] = round(row["two_bit"]["kernel_us_per_launch"] / row["base3"]["kernel_us_per_launch"], 3)
+            res[name][f"batch{m}_{dt}_{'a8' if gmode else 'float'}"] = row
+            for x in acts + outs:
+                x.free()
+        for mode in (0, 2):
+            for l in layers[mode]:
+                l.free()
+    res["bits"] = "identical between the two streams (checked on the last layer copy of every launch)"
+    return res
+
+
 def bench_salt(T, be, rng, iters=30):
     """Block-scale additive planes (SALT): the headline shape K=2048 x 2 planes with per-256-block f16
     scales, one tall layer of N = 262,144 output channels per launch (2 x 134 MB of codes; two
@@ -642,7 +691,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,salt,vjp",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,base3,salt,vjp",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -699,6 +748,7 @@ def main():
                 "stack": ("projection_stack", lambda: bench_stack(T, be, rng)),
                 "config5": ("config5_three_planes", lambda: bench_config5(T, be, rng)),
                 "zero_skip": ("zero_chunk_skip", lambda: bench_zero_skip(T, be, rng)),
+                "base3": ("base3_stream_vs_two_bit", lambda: bench_base3(T, be, rng)),
                 "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng)),
                 "vjp": ("projected_vjp", lambda: bench_vjp(T, be, rng))}
         out["extra"] = {}

@@ -207,6 +207,17 @@ int tk_weights_format(const tk_weights *w);
  * 1 = never keep a map, 2 = always. tk_weights_zero_chunks reports what an upload found. */
 int tk_set_zero_skip(tk_ctx *ctx, int mode);
 int tk_weights_zero_chunks(const tk_weights *w, size_t *zero, size_t *total, int *map_kept);
+/* Base-3 weight stream: the decode GEMV of the reference that reads TQ1_0's five-trits-per-byte codes and
+ * unpacks them in the kernel (crates/tritium-cuda/kernels/tq2_0_add.cu:744-774,796-913). Here: a second
+ * device copy of a plane in which every byte is a TQ1_0-coded group of five trits (52 bytes per 256
+ * trits where the 2-bit layout holds 64), regrouped for the int8 matrix instruction, kept BESIDE the 2-bit
+ * codes (memory: +81%). Decode launches whose operand rows stay in LDS (at most 32 rows: up to 32 int8
+ * tokens or 8 float tokens; at most three planes) then stream the base-3 copy and decode it in the
+ * kernel; every other launch reads the 2-bit codes. Same integers, identical bits.
+ * tk_set_base3_stream acts on later uploads: 0 = no base-3 copy (default), 1 = uploads in TQ1_0 keep
+ * one, 2 = every upload does. tk_weights_base3_bytes: size of a buffer's base-3 copy, 0 if it has none. */
+int tk_set_base3_stream(tk_ctx *ctx, int mode);
+size_t tk_weights_base3_bytes(const tk_weights *w);
 /* Debug/parity aid: decode the device-resident planes back to [n,k] trits. */
 int tk_weights_download_trits(tk_ctx *ctx, const tk_weights *w, int8_t *trits, size_t trits_len);
 

@@ -64,6 +64,8 @@ SIGNATURES = {
     "tk_weights_k": (sz, [vp]),
     "tk_weights_format": (C.c_int, [vp]),
     "tk_set_zero_skip": (C.c_int, [vp, C.c_int]),
+    "tk_set_base3_stream": (C.c_int, [vp, C.c_int]),
+    "tk_weights_base3_bytes": (sz, [vp]),
     "tk_weights_zero_chunks": (C.c_int, [vp, C.POINTER(sz), C.POINTER(sz), C.POINTER(C.c_int)]),
     "tk_weights_download_trits": (C.c_int, [vp, vp, vp, sz]),
     "tk_mpgemm": (C.c_int, [vp, vp, sz, vp, vp, sz, sz, sz, sz, C.c_int, vp, sz]),

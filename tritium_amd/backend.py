@@ -196,6 +196,10 @@ class Mi355xBuffer(DeviceBuffer):
         _check(L.load().tk_weights_zero_chunks(self._h, C.byref(z), C.byref(t), C.byref(kept)))
         return z.value, t.value, bool(kept.value)
 
+    def base3_bytes(self):
+        """Bytes of this buffer's base-3 stream (0 when the upload kept none)."""
+        return L.load().tk_weights_base3_bytes(self._h)
+
     def download_trits(self):
         out = np.empty(self.n * self.k, np.int8)
         _check(L.load().tk_weights_download_trits(self._backend._ctx, self._h, out.ctypes.data, out.size))
@@ -531,6 +535,10 @@ class Mi355xBackend:
     def set_zero_skip(self, mode):
         """Later uploads: 0 keep a zero-chunk map by the 0.5% threshold, 1 never, 2 always."""
         _check(self._lib.tk_set_zero_skip(self._ctx, mode))
+
+    def set_base3_stream(self, mode):
+        """Later uploads: 0 no base-3 copy, 1 TQ1_0 uploads keep one beside the 2-bit codes, 2 every upload."""
+        _check(self._lib.tk_set_base3_stream(self._ctx, mode))
 
     def set_stream_min_groups(self, groups):
         _check(self._lib.tk_set_stream_min_groups(self._ctx, groups))

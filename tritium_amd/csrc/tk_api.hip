@@ -79,6 +79,7 @@ struct tk_ctx {
   int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
+  int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
   unsigned *d_count = nullptr;  // a device counter for the uploads
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum, kpart, kcount;
@@ -99,6 +100,7 @@ static void ctx_release(tk_ctx *ctx) {
 struct tk_weights {
   tk_ctx *ctx;
   uint8_t *codes;           // n_tiles * nb chunks of 1 KiB, then one chunk of all-zero trits (0x55)
+  uint8_t *codes3;          // the same chunks as a base-3 stream of 832 bytes each (tk_internal.h), or null
   uint32_t *zero_map;       // one bit per chunk, set = all-zero trits; null when too few chunks are zero
   size_t zero_chunks;       // how many chunks are zero (counted at upload whether or not the map is kept)
   float *block_scales;  // [(tile, K block), 16 rows] f32, only for uploads that keep the block scales
@@ -337,6 +339,14 @@ extern "C" int tk_set_zero_skip(tk_ctx *ctx, int mode) {
   return TK_OK;
 }
 
+extern "C" int tk_set_base3_stream(tk_ctx *ctx, int mode) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_base3_stream: null context");
+  if (mode < 0 || mode > 2) return tk_fail(TK_ERR_INVALID_INPUT, "base3_stream=%d - use 0 (off), 1 (TQ1_0 uploads) or 2 (every upload)", mode);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->base3 = mode;
+  return TK_OK;
+}
+
 extern "C" int tk_set_flow_ring(tk_ctx *ctx, int positions) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_ring: null context");
   if (positions != 0 && (positions < 2 || positions > 5))
@@ -403,15 +413,18 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
   const size_t n_tiles = (n + 15) / 16;
   const size_t n_chunks = n_tiles * nb, code_bytes = n_chunks * TK_CHUNK_BYTES;
   const size_t map_words = (n_chunks + 31) / 32;
-  void *codes = nullptr, *raw = nullptr, *bscales = nullptr, *zmap = nullptr;
+  void *codes = nullptr, *raw = nullptr, *bscales = nullptr, *zmap = nullptr, *codes3 = nullptr;
+  const bool want3 = n_chunks && !keep_block_scales && (ctx->base3 == 2 || (ctx->base3 == 1 && format == TK_FORMAT_TQ1_0));
   TKCHK(dev_malloc(code_bytes + TK_CHUNK_BYTES, &codes));  // + the resident all-zero chunk
   int rc = dev_malloc(packed_len, &raw);
+  if (!rc && want3) rc = dev_malloc(n_chunks * TK_B3_CHUNK_BYTES, &codes3);
   if (!rc && keep_block_scales) rc = dev_malloc(n_tiles * nb * 16 * sizeof(float), &bscales);
   if (!rc && ctx->zero_skip != 1 && n_chunks) rc = dev_malloc(map_words * 4, &zmap);
   if (rc) {
     (void)hipFree(codes);
     if (raw) (void)hipFree(raw);
     if (bscales) (void)hipFree(bscales);
+    if (codes3) (void)hipFree(codes3);
     return rc;
   }
   int invalid = INT32_MAX;
@@ -428,6 +441,7 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
     else
       e = tk_launch_relayout_tq1(ctx->stream, (const uint8_t *)raw, (uint8_t *)codes, n, nb);
   }
+  if (e == hipSuccess && codes3) e = tk_launch_encode_base3(ctx->stream, (const uint8_t *)codes, (uint8_t *)codes3, n_chunks);
   if (e == hipSuccess && zmap)
     e = tk_launch_zero_chunk_map(ctx->stream, (const uint8_t *)codes, n_chunks, (uint32_t *)zmap, ctx->d_count);
   if (e == hipSuccess && zmap)
@@ -446,6 +460,7 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
     (void)hipFree(codes);
     if (bscales) (void)hipFree(bscales);
     if (zmap) (void)hipFree(zmap);
+    if (codes3) (void)hipFree(codes3);
     return tk_fail(TK_ERR_BACKEND, "upload_weights: %s", hipGetErrorString(e));
   }
   tk_weights *w = new (std::nothrow) tk_weights();
@@ -453,12 +468,14 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
     (void)hipFree(codes);
     if (bscales) (void)hipFree(bscales);
     if (zmap) (void)hipFree(zmap);
+    if (codes3) (void)hipFree(codes3);
     return tk_fail(TK_ERR_BACKEND, "tk_upload_weights: host allocation failed");
   }
   w->zero_map = (uint32_t *)zmap;
   w->zero_chunks = zero_chunks;
   w->ctx = ctx;
   w->codes = (uint8_t *)codes;
+  w->codes3 = (uint8_t *)codes3;
   w->block_scales = (float *)bscales;
   w->n = n;
   w->k = k;
@@ -536,6 +553,7 @@ extern "C" void tk_free_weights(tk_weights *w) {
     (void)hipFree(w->codes);
     if (w->block_scales) (void)hipFree(w->block_scales);
     if (w->zero_map) (void)hipFree(w->zero_map);
+    if (w->codes3) (void)hipFree(w->codes3);
     delete w;
   }
   ctx_release(ctx);
@@ -547,6 +565,9 @@ extern "C" int tk_weights_zero_chunks(const tk_weights *w, size_t *zero, size_t 
   if (total) *total = w->n_tiles * w->nb;
   if (map_kept) *map_kept = w->zero_map ? 1 : 0;
   return TK_OK;
+}
+extern "C" size_t tk_weights_base3_bytes(const tk_weights *w) {
+  return w && w->codes3 ? w->n_tiles * w->nb * (size_t)TK_B3_CHUNK_BYTES : 0;
 }
 extern "C" size_t tk_weights_n(const tk_weights *w) { return w ? w->n : 0; }
 extern "C" size_t tk_weights_k(const tk_weights *w) { return w ? w->k : 0; }
@@ -634,15 +655,27 @@ static bool flow_wide(const tk_ctx *ctx, int planes, int rt, size_t nb, size_t r
   if (ctx->flow_mfma == 32) return true;
   return rt == 2 && rows > 24 && flow_wide_lds(rt, nb) <= 64 * 1024;
 }
-static int flow_runs_per_wave(bool wide, int planes, int rt, size_t rows) {
+static int flow_runs_per_wave(bool wide, bool b3, int planes, int rt, size_t rows) {
+  if (b3) return tk_flow3_runs_per_wave(planes);
   return wide ? tk_flow32_runs_per_wave() : tk_flow_runs_per_wave(planes, rt, (int)rows);
+}
+// The base-3 form of the flow kernel: every plane of the problem carries a base-3 stream, at most three
+// planes and 32 operand rows, and the rows fit in LDS behind the decode table.
+static bool flow_base3(const TkProblem &pr, int planes, int rt, size_t rows_lds) {
+  if (planes > 3 || rt > 2 || TK_B3_TABLE_BYTES + rows_lds > kLdsFlowMax) return false;
+  for (int p = 0; p < planes; ++p)
+    if (!pr.codes3[p]) return false;
+  return true;
 }
 // zmap_tiles > 0: some plane of the launch carries a zero-chunk map; a workgroup of that many tiles stages
 // the words of its chunks behind the operand rows (16x16x64 form only; the other kernels ignore the maps)
-static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds, size_t rows, size_t zmap_tiles = 0,
+// (b3: flow_lds includes the decode table; ring and runs per wave are the base-3 kernel's own)
+static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds, size_t rows, size_t zmap_tiles = 0,
                           size_t zmap_nb = 0) {
   cfg->wide_mfma = wide ? 1 : 0;
-  cfg->tw = flow_runs_per_wave(wide, cfg->planes, cfg->rt, rows);
+  cfg->base3 = b3 ? 1 : 0;
+  if (b3) cfg->ring = 4;
+  cfg->tw = flow_runs_per_wave(wide, b3, cfg->planes, cfg->rt, rows);
   cfg->lds_bytes = flow_lds + (wide ? kFlowWideExtraLds : 0);
   if (!wide && zmap_tiles) cfg->lds_bytes += (size_t)cfg->planes * tk_flow_zmap_words(zmap_tiles, zmap_nb) * 4;
   if (wide && cfg->ring > 4) cfg->ring = 4;
@@ -657,10 +690,10 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, size_t flow_lds, size_t r
 // operand rows (8-16 KiB staged) are 5-8% faster with runs of ONE tile (64 KiB per workgroup), 16
 // rows stay at 2.
 static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
-                          size_t nb, bool wide, size_t rows) {
+                          size_t nb, bool wide, bool b3, size_t rows) {
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
-  const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, planes, rt, rows);
-  const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * TK_CHUNK_BYTES;
+  const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows);
+  const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * (b3 ? TK_B3_CHUNK_BYTES : TK_CHUNK_BYTES);
   size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 ? 2 : 4);
   if (target < 64 * 1024) target = 64 * 1024;
   size_t s = 1;
@@ -750,6 +783,7 @@ static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_
   const size_t R = mode == TK_MODE_DIGITS ? 4 * m : m;
   for (int p = 0; p < layer->n_planes; ++p) {
     pr.codes[p] = layer->planes[p]->codes;
+    pr.codes3[p] = layer->planes[p]->codes3;
     pr.scales[p] = layer->scales[p];
     pr.zmap[p] = layer->planes[p]->zero_map;
     if (pr.zmap[p]) pr.zskip = 1;
@@ -863,14 +897,16 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   const size_t nb = pl.pr.nb, R = pl.pr.R;
   int variant = DECODE_KSPLIT, run_tiles = 1;
   unsigned flow_groups = 0;
-  bool wide = false;
+  bool wide = false, b3 = false;
   size_t flow_lds = pl.flow_lds;
   if (pl.skinny) {
-    wide = pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R);
+    b3 = pl.flow_ok && flow_base3(pl.pr, pl.cfg.planes, pl.cfg.rt, flow_lds);
+    wide = !b3 && pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R);
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
-    const int fw = flow_waves(flow_lds);
-    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, R);
-    const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
+    if (b3) flow_lds += TK_B3_TABLE_BYTES;
+    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds);
+    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R);
+    const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
     variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
@@ -935,15 +971,16 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
-    cfg.waves = flow_waves(flow_lds);
-    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R));
-    size_t ztiles = pr.zskip && !wide ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0;
+    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds);
+    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R));
+    size_t ztiles = pr.zskip && !wide && !b3 ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0;
     if (ztiles && flow_lds + (size_t)cfg.planes * tk_flow_zmap_words(ztiles, nb) * 4 > kLdsFlowMax) ztiles = 0;
-    if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or the 32x32x32 form): plain loads
-    flow_cfg_form(&cfg, wide, flow_lds, R, ztiles, nb);
+    if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or another form of the kernel): plain loads
+    flow_cfg_form(&cfg, wide, b3, flow_lds, R, ztiles, nb);
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
-    HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
+    if (b3) HIPCHK(tk_launch_flow3(ctx->stream, &pr, nullptr, nullptr, cfg));
+    else HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
   } else if (pl.skinny && variant == DECODE_STREAM) {
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = pl.stream_groups;
@@ -1552,16 +1589,19 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     if ((size_t)plans[i].pr.nb > nb_max) nb_max = plans[i].pr.nb;
     if ((size_t)plans[i].pr.R > rows_max) rows_max = plans[i].pr.R;
   }
-  const bool wide = flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
+  bool b3 = flow_ok;
+  for (size_t i = 0; i < count && b3; ++i) b3 = flow_base3(plans[i].pr, planes, rt, flds);
+  const bool wide = !b3 && flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
   if (wide) flds = flow_wide_lds(rt, nb_max);
-  const int fw = flow_waves(flds);
-  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, rows_max);
+  if (b3) flds += TK_B3_TABLE_BYTES;
+  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds);
+  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, b3, rows_max);
   {
     std::vector<unsigned> member_tiles(count);
     for (size_t i = 0; i < count; ++i) member_tiles[i] = (unsigned)plans[i].pr.n_tiles;
-    run_tiles = trim_run_tiles(ctx, run_tiles, (size_t)fw * (size_t)flow_runs_per_wave(wide, planes, rt, rows_max), member_tiles);
+    run_tiles = trim_run_tiles(ctx, run_tiles, (size_t)fw * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows_max), member_tiles);
   }
-  const unsigned fper = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, planes, rt, rows_max) * (unsigned)run_tiles;
+  const unsigned fper = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, planes, rt, rows_max) * (unsigned)run_tiles;
   unsigned fgroups = 0;
   for (size_t i = 0; i < count; ++i) {
     sgroups += ((unsigned)plans[i].pr.n_tiles + tpw - 1) / tpw;
@@ -1610,14 +1650,14 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds);
-    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, prows_max) : 1;
+    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max) : 1;
     {
       std::vector<unsigned> member_tiles;
       for (size_t i = 0; i < count; ++i)
         if (plans[i].flow_ok) member_tiles.push_back((unsigned)plans[i].pr.n_tiles);
-      prun = trim_run_tiles(ctx, prun, (size_t)pfw * (size_t)flow_runs_per_wave(pwide, planes, rt, prows_max), member_tiles);
+      prun = trim_run_tiles(ctx, prun, (size_t)pfw * (size_t)flow_runs_per_wave(pwide, false, planes, rt, prows_max), member_tiles);
     }
-    const unsigned pper = (unsigned)pfw * (unsigned)flow_runs_per_wave(pwide, planes, rt, prows_max) * (unsigned)prun;
+    const unsigned pper = (unsigned)pfw * (unsigned)flow_runs_per_wave(pwide, false, planes, rt, prows_max) * (unsigned)prun;
     unsigned flow_total = 0;
     for (size_t i = 0; i < count; ++i) {
       if (plans[i].flow_ok) {
@@ -1645,7 +1685,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.lds_bytes = pflds;
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
-      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, planes, rt, prows_max));
+      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, false, planes, rt, prows_max));
       size_t ztiles = 0;
       for (size_t i = 0; i < count; ++i)
         if (plans[i].flow_ok && plans[i].pr.zskip && !pwide) ztiles = pper;
@@ -1653,7 +1693,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       if (!ztiles)
         for (size_t i = 0; i < count; ++i)
           if (plans[i].flow_ok) plans[i].pr.zskip = 0;
-      flow_cfg_form(&flow_cfg, pwide, pflds, prows_max, ztiles, pnb_max);
+      flow_cfg_form(&flow_cfg, pwide, false, pflds, prows_max, ztiles, pnb_max);
     }
   } else if (variant != DECODE_KSPLIT) {
     const unsigned per = variant == DECODE_FLOW ? fper : tpw;
@@ -1674,7 +1714,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   size_t group_ztiles = 0;
   if (variant == DECODE_FLOW) {
     for (size_t i = 0; i < count; ++i)
-      if (plans[i].pr.zskip && !wide) group_ztiles = fper;
+      if (plans[i].pr.zskip && !wide && !b3) group_ztiles = fper;
     if (group_ztiles && flds + (size_t)planes * tk_flow_zmap_words(group_ztiles, nb_max) * 4 > kLdsFlowMax) group_ztiles = 0;
     if (!group_ztiles)
       for (size_t i = 0; i < count; ++i) plans[i].pr.zskip = 0;
@@ -1774,9 +1814,9 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       nbs[i] = plans[i].pr.nb;
       wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
     }
-    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, planes, rt, rows_max));
+    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max));
   }
-  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, flds, rows_max, group_ztiles, nb_max);
+  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max);
   ctx->refs.fetch_add(1);
   *out = g;
   return TK_OK;
@@ -1797,6 +1837,8 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
                           g->flow_cfg));
   if (do_main && g->variant == DECODE_GEMM)
     HIPCHK(tk_launch_gemm(ctx->stream, nullptr, probs, wg_prob, g->cfg));
+  else if (do_main && g->variant == DECODE_FLOW && g->cfg.base3)
+    HIPCHK(tk_launch_flow3(ctx->stream, nullptr, probs, wg_prob, g->cfg));
   else if (do_main && g->variant == DECODE_FLOW)
     HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, wg_prob, g->cfg));
   else if (do_main && g->variant == DECODE_STREAM)

@@ -17,6 +17,20 @@
 #define TK_TILE_ROWS 16
 #define TK_CHUNK_BYTES 1024
 
+// ---- base-3 weight stream ("T16B3"), an optional second copy of a plane ----------------------
+// The same tiles and K blocks, 832 bytes per chunk instead of 1024: lane l = g*16 + r keeps its 64
+// trits (the ones its 16 bytes of the T16 chunk hold) in 13 bytes of five base-3 digits each, encoded
+// as TQ1_0 encodes a byte (v = d0*81 + d1*27 + d2*9 + d3*3 + d4 over codes trit+1, byte =
+// ceil(v*256/243); digit n decodes as ((uint8)(byte*3^n) * 3) >> 8: crates/tritium-format/src/tq1.rs:18-30,
+// crates/tritium-cuda/kernels/tq2_0_add.cu:744-774). Bytes 0..11 of lane l sit at l*12 (three dwords),
+// byte 12 at 768 + l. With c[j][s][b] the code of the T16 chunk's dword j, byte b, 2-bit slot s:
+//   byte t < 12: digit 0 = c[t/4][3][t%4], digits 1..4 = c[t/3][t%3][0..3]
+//   byte 12:     digit 0 = 0,              digits 1..4 = c[3][3][0..3]
+// so that digits 1..4 of a byte are one MFMA operand dword (read from a 256-entry table) and digit 0
+// of the four bytes of a dword is another (two multiplies by 3 on the even and the odd bytes).
+#define TK_B3_CHUNK_BYTES 832
+#define TK_B3_TABLE_BYTES 65536  // 256 entries x 64 lanes x 4 bytes: every lane reads its own bank
+
 // ---- activation operand layout ("Ap") -----------------------------------------------------
 // int8 rows (R of them), laid out so that one 16-byte read is one MFMA A operand matching the
 // B operand obtained from dword j of a weight lane:
@@ -27,6 +41,7 @@ enum { TK_MODE_INT8 = 0, TK_MODE_DIGITS = 1 };
 
 struct TkProblem {
   const uint8_t *codes[TK_MAX_PLANES];
+  const uint8_t *codes3[TK_MAX_PLANES];  // the plane's base-3 stream, or null (only the base-3 flow kernel reads it)
   const float *scales[TK_MAX_PLANES];
   const int8_t *ap;          // operand rows, row stride R
   const int32_t *rowsum;     // [R]
@@ -102,6 +117,7 @@ struct TkLaunchCfg {
   int wide_mfma; // flow kernel: 32x32x32 form (17..64 operand rows, row constants in LDS)
   int gemm_nt;  // prefill kernel, one plane: tiles per wave (0 = the default 4, or 2)
   int tw;       // flow kernel, 16x16x64 form: runs per wave (tk_flow_runs_per_wave)
+  int base3;    // flow kernel: stream the planes' base-3 copies (tk_launch_flow3)
 };
 
 #ifdef __cplusplus
@@ -131,6 +147,15 @@ hipError_t tk_launch_stream(hipStream_t s, const TkProblem *single, const TkProb
 int tk_flow_runs_per_wave(int planes, int rt, int rows);
 hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
+// base-3 stream (tk_base3.hip): re-encode a T16 plane, and the flow kernel that streams the result.
+// The kernel takes 1..3 planes and one or two row tiles (<= 32 operand rows), always with a ring of four
+// positions and tk_flow3_runs_per_wave(planes) runs per wave; its LDS holds the decode table
+// (TK_B3_TABLE_BYTES) in front of the operand rows.
+hipError_t tk_launch_encode_base3(hipStream_t s, const uint8_t *codes, uint8_t *codes3, size_t chunks);
+int tk_flow3_runs_per_wave(int planes);
+int tk_flow3_waves(int rt);  // waves per workgroup
+hipError_t tk_launch_flow3(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                           const TkLaunchCfg &cfg);
 int tk_gemm_tiles_per_wg(int planes);
 int tk_gemm_lds_bytes(void);
 int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows, int tw);
