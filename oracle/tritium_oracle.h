@@ -196,6 +196,66 @@ int to_cpu_mpgemm_fast(const uint8_t *packed, size_t packed_len, int format, con
                        const float *scales, size_t m, size_t n, size_t k, float *out, int threads,
                        int *threads_used, int *kernel_used);
 
+/* ======================================================================================
+ * SALT containers and SALT V2 (salt_oracle.c)
+ * ====================================================================================== */
+/* FormatError variants of crates/tritium-format/src/lib.rs the SALT readers and writers return, and the
+ * SaltV2CodecError / SaltV2CpuError variants of salt_v2.rs and crates/tritium-cpu/src/salt_v2.rs. */
+enum {
+  TO_SALT_BAD_MAGIC = 20,
+  TO_SALT_UNSUPPORTED_VERSION = 21,
+  TO_SALT_WRONG_LEN = 22,           /* WrongBlockLen */
+  TO_SALT_INVALID_PLANE_TAG = 23,
+  TO_SALT_SPARSE_BASE_PLANE = 24,
+  TO_SALT_OUT_OF_RANGE = 25,        /* DecodedOutOfRange */
+  TO_SALT_NONCANONICAL_INDICES = 26,
+  TO_SALT_ROW_TOO_LONG = 27,
+  TO_SALT_NONZERO_PADDING = 28,
+  TO_SALT_INVALID_DENSITY = 29,
+  TO_SALT_TOO_MANY_PLANES = 30,
+  TO_SALT_V2_WRONG_PACKED_LENGTH = 40,
+  TO_SALT_V2_INVALID_D2_CODE = 41,
+  TO_SALT_V2_INVALID_B3_CODE = 42,
+  TO_SALT_V2_NONCANONICAL_TRIT_PADDING = 43,
+  TO_SALT_V2_S34_NOT_MULTIPLE_OF_FOUR = 44,
+  TO_SALT_V2_S34_ZERO_COUNT = 45,
+  TO_SALT_V2_NONCANONICAL_BIT_PADDING = 46,
+  TO_SALT_V2_NONFINITE_ACTIVATION = 47,
+  TO_SALT_V2_NONFINITE_OUTPUT = 48
+};
+/* crates/tritium-format/src/salt_v2.rs:22-32 (tags as crates/tritium-cuda/kernels/salt_v2.cu:31-52 numbers them) */
+enum { TO_SALT_V2_D2 = 0, TO_SALT_V2_B3 = 1, TO_SALT_V2_S34 = 2 };
+
+/* ---- crates/tritium-format/src/sparse.rs ---- */
+size_t to_sparse_plane_packed_len(size_t k, size_t nnz);                                             /* :33-34,444-475 */
+int to_sparse_from_tq2_0(const uint8_t *packed, size_t packed_len, size_t k, uint16_t *scales, uint32_t *idx,
+                         int8_t *sign, size_t *nnz);                                                 /* :235-285 */
+int to_sparse_to_tq2_0(size_t k, const uint16_t *scales, size_t n_scales, const uint32_t *idx, const int8_t *sign,
+                       size_t nnz, uint8_t *out, size_t out_len);                                    /* :293-340 */
+int to_pack_sparse_plane(size_t k, const uint16_t *scales, size_t n_scales, const uint32_t *idx, const int8_t *sign,
+                         size_t nnz, uint8_t *out, size_t out_len);                                  /* :444-475 */
+int to_unpack_sparse_plane(const uint8_t *bytes, size_t len, size_t *k, uint16_t *scales, size_t scales_cap,
+                           uint32_t *idx, int8_t *sign, size_t cap, size_t *nnz);                    /* :92-157,479-481 */
+/* ---- crates/tritium-format/src/salt.rs ---- */
+int to_pack_salt_row(size_t k, const uint8_t *const *planes, size_t t, uint8_t *out, size_t out_cap, size_t *written); /* :229-241 */
+int to_pack_progressive_salt_row(size_t k, const uint8_t *const *planes, size_t t, float max_sparse_density,
+                                 uint8_t *out, size_t out_cap, size_t *written);                     /* :253-316 */
+int to_packed_salt_row_len(const uint8_t *bytes, size_t len, size_t *row_len);                       /* :352-434,596-598 */
+int to_unpack_salt_row_prefix(const uint8_t *bytes, size_t len, size_t max_planes, size_t *k, size_t *planes,
+                              uint8_t *dense_out, size_t dense_cap);                                 /* :484-515,669-700 */
+/* ---- crates/tritium-format/src/salt_v2.rs ---- */
+int to_salt_v2_payload_bytes(int codec, size_t trits, size_t *bytes);                                /* :160-258 */
+int to_salt_v2_pack(int codec, const int8_t *trits, size_t n, uint8_t *out, size_t out_len);          /* :268-281,326-349,420-452 */
+int to_salt_v2_unpack(int codec, const uint8_t *packed, size_t packed_len, size_t n, int8_t *trits);  /* :289-322,358-392,454-520 */
+/* ---- crates/tritium-cpu/src/salt_v2.rs:316-423 (batched as crates/tritium-cuda/kernels/salt_v2.cu:114-216) ---- */
+int to_salt_v2_forward(int codec, size_t scale_group, const uint8_t *payload, size_t payload_len,
+                       const uint16_t *scales, size_t scale_count, const uint8_t *plane_counts, size_t tiles,
+                       size_t n, size_t k, const float *act, size_t m, float *out);
+/* ---- crates/tritium-cpu/src/salt_v2.rs:283-300,516-546 ---- */
+int to_salt_v2_coefficient(int codec, size_t scale_group, const uint8_t *payload, size_t payload_len,
+                           const uint16_t *scales, size_t scale_count, const uint8_t *plane_counts, size_t tiles,
+                           size_t n, size_t k, size_t index, float *value);
+
 #ifdef __cplusplus
 }
 #endif
