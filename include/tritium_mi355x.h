@@ -381,6 +381,70 @@ int tk_linear_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int 
 int tk_linear_salt_seq(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int act_dtype, size_t m,
                        void *out, int out_dtype);
 
+/* ---- SALT containers: the row sidecar "TSLT" (version 1: dense planes back to back; version 2,
+ *      progressive: each plane framed by a tag and a length, residual planes may be sparse) and the sparse
+ *      residual plane "TSSP" (crates/tritium-format/src/salt.rs:1-19,229-316,352-434,484-515,596-700;
+ *      crates/tritium-format/src/sparse.rs:27-41,92-157,293-309). Host functions; every check of the
+ *      reference's readers, in their order, failures are TK_ERR_INVALID_INPUT naming the reference's error.
+ *      A sparse plane expands to exactly the dense TQ2_0 row it was made from, so the device path below is
+ *      bit-identical whichever way a residual was stored. ---- */
+/* packed_salt_row_len: length of the first encoded row in `bytes` (rows are stored back to back) */
+int tk_salt_row_len(const uint8_t *bytes, size_t len, size_t *row_len);
+/* header fields of the first row: k, plane count, version (any of the three may be NULL) */
+int tk_salt_row_info(const uint8_t *bytes, size_t len, size_t *k, size_t *planes, int *version);
+/* unpack_salt_row_prefix: `bytes` is exactly one row; all planes are validated, the first
+ * min(planes, max_planes) are written as dense TQ2_0 rows of ceil(k/256)*66 bytes, back to back. */
+int tk_salt_row_unpack(const uint8_t *bytes, size_t len, size_t max_planes, uint8_t *planes_out,
+                       size_t planes_out_len, size_t *k, size_t *n_planes);
+/* unpack_sparse_plane + sparse_to_tq2_0: one encoded sparse plane -> its dense TQ2_0 row */
+int tk_sparse_plane_to_tq2_0(const uint8_t *bytes, size_t len, uint8_t *row_out, size_t row_out_len, size_t *k);
+/* A SALT tensor: n encoded rows back to back (as a bundle stores them) -> up to TK_MAX_PLANES block-scale
+ * planes on the device (the loader of crates/tritium-nn/src/layers/packed_salt.rs:612-678). Rows may differ
+ * in plane count: plane p of a row with fewer planes is all-zero trits with scale 0 (adds +0.0, as a missing
+ * plane adds nothing). max_planes keeps a prefix of every row (the lower-memory tiers of the progressive
+ * format). planes_out receives *n_planes buffers (from tk_upload_weights_scaled; free each with
+ * tk_free_weights) to put into a tk_salt_desc. A row with more than TK_MAX_PLANES kept planes ->
+ * TK_ERR_UNSUPPORTED_FORMAT; a row whose k differs -> TK_ERR_SHAPE_MISMATCH. */
+int tk_upload_salt_rows(tk_ctx *ctx, const uint8_t *bytes, size_t len, size_t n, size_t k, size_t max_planes,
+                        tk_weights **planes_out, int *n_planes);
+
+/* ---- SALT V2: zero-point-free additive ternary matrices over 256-coefficient allocation tiles with one
+ *      to three planes each, f16 scales per group of 128 (or 64) coefficients, three physical codecs
+ *      (crates/tritium-format/src/salt_v2.rs:22-32; crates/tritium-format/src/salt_v2_package.rs:38-47). ---- */
+enum { TK_SALT_V2_D2 = 0, TK_SALT_V2_B3 = 1, TK_SALT_V2_S34 = 2 }; /* as crates/tritium-cuda/kernels/salt_v2.cu:31-52 */
+/* SaltV2Codec::ledger: physical bytes of `trits` logical trits (salt_v2.rs:160-258) */
+int tk_salt_v2_payload_bytes(int codec, size_t trits, size_t *bytes);
+/* pack_d2 / pack_b3 / pack_s34 and their canonical decoders (salt_v2.rs:268-520): padding slots are zero
+ * trits, padding bits zero; reserved codes, B3 bytes >= 243, S34 groups without exactly one zero, wrong
+ * lengths are rejected. */
+int tk_salt_v2_pack(int codec, const int8_t *trits, size_t n, uint8_t *out, size_t out_len);
+int tk_salt_v2_unpack(int codec, const uint8_t *packed, size_t packed_len, size_t n, int8_t *trits);
+/* A resident SALT V2 matrix [n,k], in the runtime form the reference's device code takes
+ * (crates/tritium-cuda/kernels/salt_v2.cu:114-131; built by crates/tritium-cuda/src/cuda/backend/
+ * salt_v2_reader_upload.rs:40-252): `payload` = the codec bytes of every plane, tile after tile, planes of a
+ * tile in order (a tile whose planes start at running plane index b has plane j at b*bytes(256) +
+ * j*bytes(tile length)); `scales` = one f16 per (plane, scale group) in the same order; plane_counts[tile]
+ * in 1..3 (the reference packs the same counts two bits per tile with a rank directory; the adapter hands
+ * them over unpacked). Tiles cover the row-major coefficients, tiles == ceil(n*k/256). scale_group is 128 or
+ * 64. Host pointers; every plane is decoded once here, so a non-canonical payload is rejected at upload. */
+typedef struct tk_salt_v2 tk_salt_v2;
+int tk_salt_v2_upload(tk_ctx *ctx, int codec, size_t scale_group, const uint8_t *payload, size_t payload_len,
+                      const uint16_t *scales_f16, size_t scale_count, const uint8_t *plane_counts, size_t tiles,
+                      size_t n, size_t k, tk_salt_v2 **out);
+void tk_salt_v2_free(tk_salt_v2 *t);
+/* salt_v2_forward_exact: out[m,n] = act[m,k] x W^T in the reference's pinned scalar order -- per output,
+ * segments (tile x scale group) ascending, planes ascending, per plane one f32 accumulator over the columns
+ * (add / subtract / skip), ONE multiply by the f16 scale, one add into the output (crates/tritium-cpu/src/
+ * salt_v2.rs:10-23,316-423; salt_v2.cu:133-214) -- so the bits are the CPU reference's. The device computes
+ * the (segment, plane) terms in parallel and adds them in that order. act and out are device f32. A
+ * non-finite activation or result -> TK_ERR_INVALID_INPUT and `out` is left untouched
+ * (crates/tritium-cuda/src/cuda/tests.rs:246-280). Synchronizes. */
+int tk_salt_v2_forward(tk_ctx *ctx, const tk_salt_v2 *t, const float *act, size_t m, float *out);
+/* salt_v2_gather_rows: out[i, :] = row rows[i] of W, each coefficient the f32 sum over its tile's planes,
+ * ascending, of +-scale (salt_v2.cu:218-304; crates/tritium-cpu/src/salt_v2.rs:283-300,516-546). rows is a
+ * host array (may repeat; order kept); out device f32 [count,k]. A row index >= n -> TK_ERR_INVALID_INPUT. */
+int tk_salt_v2_gather_rows(tk_ctx *ctx, const tk_salt_v2 *t, const uint32_t *rows, size_t count, float *out);
+
 /* mpgemm_projected_vjp on device-resident operands (same arithmetic and bits as
  * tk_mpgemm_projected_vjp; precedent for device-resident gradients:
  * crates/tritium-cuda/src/cuda/backend.rs:8755-8830, which stages exactly these buffers). scales [n],

@@ -100,6 +100,18 @@ SIGNATURES = {
     "tk_gguf_load_ternary": (C.c_int, [vp, vp, sz, C.c_char_p, vp, sz, vp, sz]),
     "tk_upload_weights_gguf": (C.c_int, [vp, vp, vp, sz, C.c_char_p, C.POINTER(vp), vp, sz]),
     "tk_upload_weights_scaled": (C.c_int, [vp, vp, sz, sz, sz, C.POINTER(vp)]),
+    "tk_salt_row_len": (C.c_int, [vp, sz, C.POINTER(sz)]),
+    "tk_salt_row_info": (C.c_int, [vp, sz, C.POINTER(sz), C.POINTER(sz), C.POINTER(C.c_int)]),
+    "tk_salt_row_unpack": (C.c_int, [vp, sz, sz, vp, sz, C.POINTER(sz), C.POINTER(sz)]),
+    "tk_sparse_plane_to_tq2_0": (C.c_int, [vp, sz, vp, sz, C.POINTER(sz)]),
+    "tk_upload_salt_rows": (C.c_int, [vp, vp, sz, sz, sz, sz, C.POINTER(vp), C.POINTER(C.c_int)]),
+    "tk_salt_v2_payload_bytes": (C.c_int, [C.c_int, sz, C.POINTER(sz)]),
+    "tk_salt_v2_pack": (C.c_int, [C.c_int, vp, sz, vp, sz]),
+    "tk_salt_v2_unpack": (C.c_int, [C.c_int, vp, sz, sz, vp]),
+    "tk_salt_v2_upload": (C.c_int, [vp, C.c_int, sz, vp, sz, vp, sz, vp, sz, sz, sz, C.POINTER(vp)]),
+    "tk_salt_v2_free": (None, [vp]),
+    "tk_salt_v2_forward": (C.c_int, [vp, vp, vp, sz, vp]),
+    "tk_salt_v2_gather_rows": (C.c_int, [vp, vp, vp, sz, vp]),
     "tk_linear_salt": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_salt_seq": (C.c_int, [vp, C.POINTER(SaltDesc), vp, C.c_int, sz, vp, C.c_int]),
     "tk_linear_a8": (C.c_int, [vp, C.POINTER(LinearDesc), vp, C.c_int, sz, vp, C.c_int]),

@@ -169,6 +169,33 @@ class DeviceArray:
             self.ptr = None
 
 
+class SaltV2Tensor:
+    """A SALT V2 matrix resident on the device (tk_salt_v2)."""
+
+    def __init__(self, backend, handle, n, k):
+        self._backend, self._h, self.n, self.k = backend, handle, n, k
+
+    def forward(self, act, m, out):
+        """out[m,n] = act[m,k] x W^T in the reference's pinned order (device f32 arrays); raises InvalidInput
+        and leaves out untouched when an activation or a result is not finite."""
+        _check(L.load().tk_salt_v2_forward(self._backend._ctx, self._h, act.ptr, m, out.ptr))
+
+    def gather_rows(self, rows, out):
+        r = np.ascontiguousarray(rows, np.uint32).reshape(-1)
+        _check(L.load().tk_salt_v2_gather_rows(self._backend._ctx, self._h, r.ctypes.data, r.size, out.ptr))
+
+    def free(self):
+        if self._h:
+            L.load().tk_salt_v2_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
 class Mi355xBuffer(DeviceBuffer):
     """Packed ternary weights resident on the device; frees its memory when dropped."""
 
@@ -346,6 +373,24 @@ class Mi355xBackend:
         h = C.c_void_p()
         _check(self._lib.tk_upload_weights_scaled(self._ctx, b.ctypes.data, b.size, shape.n, shape.k, C.byref(h)))
         return Mi355xBuffer(self, h)
+
+    def upload_salt_rows(self, data, n, k, max_planes=1 << 30):
+        """A SALT tensor -- n encoded rows ("TSLT" version 1 or 2, sparse residuals allowed) back to back -- as
+        block-scale planes for linear_salt; max_planes keeps a prefix of every row."""
+        b = np.ascontiguousarray(data, dtype=np.uint8).reshape(-1)
+        hs, count = (C.c_void_p * L.TK_MAX_PLANES)(), C.c_int(0)
+        _check(self._lib.tk_upload_salt_rows(self._ctx, b.ctypes.data, b.size, n, k, max_planes, hs, C.byref(count)))
+        return [Mi355xBuffer(self, C.c_void_p(hs[i])) for i in range(count.value)]
+
+    def salt_v2_upload(self, codec, scale_group, payload, scales_f16, plane_counts, n, k):
+        """A SALT V2 matrix [n,k] from its runtime parts: codec payload, f16 scale bits, per-tile plane counts."""
+        pay = np.ascontiguousarray(payload, np.uint8).reshape(-1)
+        sc = np.ascontiguousarray(scales_f16, np.uint16).reshape(-1)
+        pc = np.ascontiguousarray(plane_counts, np.uint8).reshape(-1)
+        h = C.c_void_p()
+        _check(self._lib.tk_salt_v2_upload(self._ctx, int(codec), scale_group, pay.ctypes.data, pay.size, sc.ctypes.data, sc.size,
+                                           pc.ctypes.data, pc.size, n, k, C.byref(h)))
+        return SaltV2Tensor(self, h, n, k)
 
     def linear_salt(self, planes, act, m, out, seq=False):
         """Block-scale additive planes on float activations: planes = buffers from
@@ -563,6 +608,64 @@ class Mi355xBackend:
 
 def packed_len(n, k, format):
     return L.load().tk_packed_len(n, k, int(format))
+
+
+def salt_row_len(data):
+    """Length of the first encoded SALT row in data (packed_salt_row_len)."""
+    b = np.ascontiguousarray(data, np.uint8).reshape(-1)
+    n = C.c_size_t(0)
+    _check(L.load().tk_salt_row_len(b.ctypes.data, b.size, C.byref(n)))
+    return n.value
+
+
+def salt_row_unpack(data, max_planes=1 << 30):
+    """One encoded SALT row -> (k, [dense TQ2_0 plane rows]); sparse residuals are expanded."""
+    b = np.ascontiguousarray(data, np.uint8).reshape(-1)
+    k, planes, version = C.c_size_t(0), C.c_size_t(0), C.c_int(0)
+    _check(L.load().tk_salt_row_info(b.ctypes.data, b.size, C.byref(k), C.byref(planes), C.byref(version)))
+    pb = (k.value + 255) // 256 * 66
+    keep = min(planes.value, max_planes)
+    out = np.zeros(max(keep * pb, 1), np.uint8)
+    kk, got = C.c_size_t(0), C.c_size_t(0)
+    _check(L.load().tk_salt_row_unpack(b.ctypes.data, b.size, max_planes, out.ctypes.data, keep * pb, C.byref(kk), C.byref(got)))
+    return kk.value, [out[i * pb:(i + 1) * pb].copy() for i in range(got.value)]
+
+
+def sparse_plane_to_tq2_0(data):
+    """One encoded sparse residual plane ("TSSP") -> (k, the dense TQ2_0 row it stands for)."""
+    b = np.ascontiguousarray(data, np.uint8).reshape(-1)
+    if b.size < 10:
+        k_hint = 0
+    else:
+        k_hint = int.from_bytes(bytes(b[6:10]), "little")
+    out = np.zeros(max((k_hint + 255) // 256 * 66, 1), np.uint8)
+    k = C.c_size_t(0)
+    _check(L.load().tk_sparse_plane_to_tq2_0(b.ctypes.data, b.size, out.ctypes.data, (k_hint + 255) // 256 * 66, C.byref(k)))
+    return k.value, out[: (k.value + 255) // 256 * 66]
+
+
+SALT_V2_D2, SALT_V2_B3, SALT_V2_S34 = 0, 1, 2
+
+
+def salt_v2_payload_bytes(codec, trits):
+    n = C.c_size_t(0)
+    _check(L.load().tk_salt_v2_payload_bytes(int(codec), trits, C.byref(n)))
+    return n.value
+
+
+def salt_v2_pack(codec, trits):
+    t = np.ascontiguousarray(trits, np.int8).reshape(-1)
+    out = np.zeros(max(salt_v2_payload_bytes(codec, t.size), 1), np.uint8)
+    need = salt_v2_payload_bytes(codec, t.size)
+    _check(L.load().tk_salt_v2_pack(int(codec), t.ctypes.data, t.size, out.ctypes.data, need))
+    return out[:need]
+
+
+def salt_v2_unpack(codec, packed, n):
+    b = np.ascontiguousarray(packed, np.uint8).reshape(-1)
+    out = np.zeros(max(n, 1), np.int8)
+    _check(L.load().tk_salt_v2_unpack(int(codec), b.ctypes.data, b.size, n, out.ctypes.data))
+    return out[:n]
 
 
 def pack_rows(trits, n, k, format=TernaryFormat.Tq2_0):

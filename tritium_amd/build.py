@@ -10,7 +10,7 @@ import tempfile
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtritium_mi355x.so")
-SOURCES = ["tk_kernels.hip", "tk_base3.hip", "tk_vjp.hip", "tk_api.hip", "tk_format.cpp", "tk_gguf.cpp"]
+SOURCES = ["tk_kernels.hip", "tk_base3.hip", "tk_salt_v2.hip", "tk_vjp.hip", "tk_api.hip", "tk_format.cpp", "tk_salt.cpp", "tk_gguf.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # packed-FP32 instructions are kept out of every kernel of this library

@@ -1202,6 +1202,210 @@ extern "C" int tk_linear_salt_seq(tk_ctx *ctx, const tk_salt_desc *layer, const 
   return run_salt(ctx, layer, act, act_dtype, m, out, out_dtype, true);
 }
 
+// A SALT tensor (n encoded rows back to back) -> block-scale planes. The rows are walked with the reader's own
+// length function, unpacked (sparse residuals expanded) into one row-major TQ2_0 tensor per plane, and
+// each plane uploaded with its block scales kept.
+extern "C" int tk_upload_salt_rows(tk_ctx *ctx, const uint8_t *bytes, size_t len, size_t n, size_t k, size_t max_planes,
+                                   tk_weights **planes_out, int *n_planes) {
+  if (!ctx || !planes_out || !n_planes || (!bytes && len)) return tk_fail(TK_ERR_INVALID_INPUT, "tk_upload_salt_rows: null pointer");
+  *n_planes = 0;
+  const size_t row_bytes = num_blocks(k) * 66;
+  size_t plane_len;
+  if (__builtin_mul_overflow(n, row_bytes, &plane_len)) return tk_fail(TK_ERR_INVALID_INPUT, "packed weight byte count overflows");
+  // the rows must fit the bytes given before anything is sized from n: a row is at least its header
+  if (n > len / 10 + 1 && n) return tk_fail_mismatch(n * 10, len);
+  std::vector<std::vector<uint8_t>> planes;
+  std::vector<uint8_t> row_planes;
+  size_t off = 0;
+  try {
+    for (size_t r = 0; r < n; ++r) {
+      size_t rl = 0, rk = 0, rp = 0;
+      TKCHK(tk_salt_row_len(bytes + off, len - off, &rl));
+      TKCHK(tk_salt_row_info(bytes + off, rl, &rk, &rp, nullptr));
+      if (rk != k) return tk_fail_mismatch(k, rk);
+      const size_t keep = rp < max_planes ? rp : max_planes;
+      if (keep > (size_t)TK_MAX_PLANES)
+        return tk_fail(TK_ERR_UNSUPPORTED_FORMAT, "SALT row %zu keeps %zu planes; the kernels take at most %d", r, keep, TK_MAX_PLANES);
+      row_planes.resize(keep * row_bytes);
+      size_t got_k = 0, got_p = 0;
+      TKCHK(tk_salt_row_unpack(bytes + off, rl, max_planes, row_planes.data(), row_planes.size(), &got_k, &got_p));
+      while (planes.size() < got_p) {
+        // a plane no earlier row had: all-zero trits with scale 0 for those rows
+        std::vector<uint8_t> fresh(plane_len);
+        for (size_t b = 0; b < plane_len; b += 66) {
+          memset(fresh.data() + b, 0x55, 64);
+          fresh[b + 64] = fresh[b + 65] = 0;
+        }
+        planes.push_back(std::move(fresh));
+      }
+      for (size_t p = 0; p < got_p; ++p) memcpy(planes[p].data() + r * row_bytes, row_planes.data() + p * row_bytes, row_bytes);
+      off += rl;
+    }
+  } catch (const std::exception &) {
+    return tk_fail(TK_ERR_BACKEND, "tk_upload_salt_rows: host allocation failed");
+  }
+  if (off != len) return tk_fail(TK_ERR_INVALID_INPUT, "%zu bytes follow the last of the %zu SALT rows", len - off, n);
+  for (size_t p = 0; p < planes.size(); ++p) {
+    int rc = tk_upload_weights_scaled(ctx, planes[p].data(), plane_len, n, k, &planes_out[p]);
+    if (rc) {
+      for (size_t q = 0; q < p; ++q) {
+        tk_free_weights(planes_out[q]);
+        planes_out[q] = nullptr;
+      }
+      return rc;
+    }
+  }
+  *n_planes = (int)planes.size();
+  return TK_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// SALT V2
+// ------------------------------------------------------------------------------------------
+struct tk_salt_v2 {
+  tk_ctx *ctx;
+  void *payload, *scales, *tile_begin;
+  TkSaltV2 dev;
+};
+
+extern "C" int tk_salt_v2_upload(tk_ctx *ctx, int codec, size_t scale_group, const uint8_t *payload, size_t payload_len,
+                                 const uint16_t *scales_f16, size_t scale_count, const uint8_t *plane_counts, size_t tiles,
+                                 size_t n, size_t k, tk_salt_v2 **out) {
+  if (!ctx || !out) return tk_fail(TK_ERR_INVALID_INPUT, "tk_salt_v2_upload: null pointer");
+  *out = nullptr;
+  if (codec != TK_SALT_V2_D2 && codec != TK_SALT_V2_B3 && codec != TK_SALT_V2_S34)
+    return tk_fail(TK_ERR_UNSUPPORTED_FORMAT, "SALT V2 codec %d", codec);
+  if (scale_group != 128 && scale_group != 64)
+    return tk_fail(TK_ERR_UNSUPPORTED_FORMAT, "SALT V2 scale group of %zu coefficients - the format defines 128 and 64", scale_group);
+  size_t total;
+  if (__builtin_mul_overflow(n, k, &total) || n > (size_t)UINT32_MAX || k > (size_t)UINT32_MAX)
+    return tk_fail(TK_ERR_INVALID_INPUT, "SALT V2 shape n=%zu k=%zu exceeds the kernels' index range", n, k);
+  if (tiles != (total + 255) / 256) return tk_fail_mismatch((total + 255) / 256, tiles);
+  if ((!payload && payload_len) || (!scales_f16 && scale_count) || (!plane_counts && tiles))
+    return tk_fail(TK_ERR_INVALID_INPUT, "tk_salt_v2_upload: null pointer");
+  if (tk_salt_v2_lds_bytes(k, scale_group) > kLdsFlowMax)
+    return tk_fail(TK_ERR_INVALID_INPUT, "SALT V2 rows of %zu columns exceed what the forward kernel stages", k);
+  // running plane index per tile; every plane decoded once (a non-canonical payload is rejected here), and
+  // the payload and the scales must be exactly as long as the tiles say
+  std::vector<uint32_t> begin;
+  std::vector<int8_t> scratch(256);
+  try {
+    begin.resize(tiles + 1);
+  } catch (const std::exception &) {
+    return tk_fail(TK_ERR_BACKEND, "tk_salt_v2_upload: host allocation failed");
+  }
+  size_t full_bytes = 0, planes = 0, pay = 0, sc = 0;
+  TKCHK(tk_salt_v2_payload_bytes(codec, 256, &full_bytes));
+  const size_t full_groups = 256 / scale_group;
+  for (size_t t = 0; t < tiles; ++t) {
+    const size_t ln = total - t * 256 < 256 ? total - t * 256 : 256;
+    if (plane_counts[t] < 1 || plane_counts[t] > 3)
+      return tk_fail(TK_ERR_INVALID_INPUT, "SALT V2 tile %zu has %u planes - one to three", t, (unsigned)plane_counts[t]);
+    if (planes > (size_t)UINT32_MAX - 3) return tk_fail(TK_ERR_INVALID_INPUT, "SALT V2 plane count exceeds the index range");
+    begin[t] = (uint32_t)planes;
+    size_t cur_bytes = 0;
+    TKCHK(tk_salt_v2_payload_bytes(codec, ln, &cur_bytes));
+    const size_t cur_groups = (ln + scale_group - 1) / scale_group;
+    for (unsigned j = 0; j < plane_counts[t]; ++j) {
+      const size_t base = planes * full_bytes + (size_t)j * cur_bytes;
+      if (base + cur_bytes > payload_len) return tk_fail_mismatch(base + cur_bytes, payload_len);
+      TKCHK(tk_salt_v2_unpack(codec, payload + base, cur_bytes, ln, scratch.data()));
+      pay = base + cur_bytes;
+      sc = planes * full_groups + (size_t)j * cur_groups + cur_groups;
+    }
+    planes += plane_counts[t];
+  }
+  begin[tiles] = (uint32_t)planes;
+  if (pay != payload_len) return tk_fail_mismatch(pay, payload_len);
+  if (sc != scale_count) return tk_fail_mismatch(sc, scale_count);
+
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  tk_salt_v2 *w = new (std::nothrow) tk_salt_v2();
+  if (!w) return tk_fail(TK_ERR_BACKEND, "tk_salt_v2_upload: host allocation failed");
+  w->ctx = ctx;
+  w->payload = w->scales = w->tile_begin = nullptr;
+  int rc = dev_malloc(payload_len, &w->payload);
+  if (!rc) rc = dev_malloc(scale_count * 2, &w->scales);
+  if (!rc) rc = dev_malloc((tiles + 1) * 4, &w->tile_begin);
+  hipError_t e = hipSuccess;
+  if (!rc && payload_len) e = hipMemcpyAsync(w->payload, payload, payload_len, hipMemcpyHostToDevice, ctx->stream);
+  if (!rc && e == hipSuccess && scale_count) e = hipMemcpyAsync(w->scales, scales_f16, scale_count * 2, hipMemcpyHostToDevice, ctx->stream);
+  if (!rc && e == hipSuccess) e = hipMemcpyAsync(w->tile_begin, begin.data(), (tiles + 1) * 4, hipMemcpyHostToDevice, ctx->stream);
+  if (!rc && e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (rc || e != hipSuccess) {
+    if (w->payload) (void)hipFree(w->payload);
+    if (w->scales) (void)hipFree(w->scales);
+    if (w->tile_begin) (void)hipFree(w->tile_begin);
+    delete w;
+    return rc ? rc : tk_fail(TK_ERR_BACKEND, "tk_salt_v2_upload: %s", hipGetErrorString(e));
+  }
+  w->dev.payload = (const uint8_t *)w->payload;
+  w->dev.scales = (const uint16_t *)w->scales;
+  w->dev.tile_begin = (const uint32_t *)w->tile_begin;
+  w->dev.n = (unsigned)n;
+  w->dev.k = (unsigned)k;
+  w->dev.codec = (unsigned)codec;
+  w->dev.group = (unsigned)scale_group;
+  w->dev.tiles = (unsigned)tiles;
+  w->dev.total = total;
+  ctx->refs.fetch_add(1);
+  *out = w;
+  return TK_OK;
+}
+
+extern "C" void tk_salt_v2_free(tk_salt_v2 *t) {
+  if (!t) return;
+  tk_ctx *ctx = t->ctx;
+  {
+    std::lock_guard<std::mutex> lk(ctx->mu);
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(t->payload);
+    (void)hipFree(t->scales);
+    (void)hipFree(t->tile_begin);
+    delete t;
+  }
+  ctx_release(ctx);
+}
+
+extern "C" int tk_salt_v2_forward(tk_ctx *ctx, const tk_salt_v2 *t, const float *act, size_t m, float *out) {
+  if (!ctx || !t) return tk_fail(TK_ERR_INVALID_INPUT, "tk_salt_v2_forward: null pointer");
+  if (t->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tensor belongs to another context");
+  if (m == 0 || t->dev.n == 0) return TK_OK;
+  if (!act || !out) return tk_fail(TK_ERR_INVALID_INPUT, "null activation or output pointer");
+  if (m > (size_t)65535 * TK_SALT_V2_TOKENS) return tk_fail(TK_ERR_INVALID_INPUT, "m=%zu - at most %d tokens per call", m, 65535 * TK_SALT_V2_TOKENS);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  const size_t bytes = m * (size_t)t->dev.n * sizeof(float);
+  TKCHK(ensure(ctx, ctx->tmp, bytes));
+  unsigned flag = 0;
+  HIPCHK(hipMemsetAsync(ctx->d_count, 0, sizeof(unsigned), ctx->stream));
+  HIPCHK(tk_launch_salt_v2_forward(ctx->stream, t->dev, act, m, (float *)ctx->tmp.p, ctx->d_count));
+  HIPCHK(hipMemcpyAsync(&flag, ctx->d_count, sizeof flag, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  if (flag) return tk_fail(TK_ERR_INVALID_INPUT, "SALT V2 forward: a non-finite activation or result; the output was not written");
+  HIPCHK(hipMemcpyAsync(out, ctx->tmp.p, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+
+extern "C" int tk_salt_v2_gather_rows(tk_ctx *ctx, const tk_salt_v2 *t, const uint32_t *rows, size_t count, float *out) {
+  if (!ctx || !t) return tk_fail(TK_ERR_INVALID_INPUT, "tk_salt_v2_gather_rows: null pointer");
+  if (t->ctx != ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tensor belongs to another context");
+  if (count == 0 || t->dev.k == 0) return TK_OK;
+  if (!rows || !out) return tk_fail(TK_ERR_INVALID_INPUT, "null row list or output pointer");
+  for (size_t i = 0; i < count; ++i)
+    if (rows[i] >= t->dev.n) return tk_fail(TK_ERR_INVALID_INPUT, "row %u of a matrix of %u rows", rows[i], t->dev.n);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  HIPCHK(hipSetDevice(ctx->device));
+  TKCHK(ensure(ctx, ctx->tmp, count * 4));
+  HIPCHK(hipMemcpyAsync(ctx->tmp.p, rows, count * 4, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(tk_launch_salt_v2_gather(ctx->stream, t->dev, (const uint32_t *)ctx->tmp.p, count, out));
+  HIPCHK(hipStreamSynchronize(ctx->stream));
+  return TK_OK;
+}
+
 extern "C" int tk_linear_i8(tk_ctx *ctx, const tk_linear_desc *layer, const int8_t *q, const float *act_scale,
                             size_t m, void *out, int out_dtype) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "null context");

@@ -172,6 +172,23 @@ hipError_t tk_launch_projected_vjp(hipStream_t s, const uint8_t *codes, size_t n
                                    const float *scales, const float *act, const float *grad_output, float *grad_act,
                                    float *grad_w, float *grad_bias);
 hipError_t tk_launch_copy(hipStream_t s, void *dst, const void *src, size_t bytes);
+
+// SALT V2 (tk_salt_v2.hip). The resident tensor: codec payload, f16 scales, and per tile the running plane
+// index of its first plane (tile_begin[tiles + 1]; the plane count of a tile is the difference).
+struct TkSaltV2 {
+  const uint8_t *payload;
+  const uint16_t *scales;
+  const uint32_t *tile_begin;
+  unsigned n, k, codec, group;       // group = coefficients per scale: 128 or 64
+  unsigned tiles;
+  unsigned long long total;          // n * k
+};
+// tokens one workgroup carries through a weight row, and the LDS a launch needs for rows of k columns
+#define TK_SALT_V2_TOKENS 8
+size_t tk_salt_v2_lds_bytes(size_t k, size_t group);
+// tmp receives the [m,n] results; *flag is raised when an activation or a result is not finite
+hipError_t tk_launch_salt_v2_forward(hipStream_t s, const TkSaltV2 &t, const float *act, size_t m, float *tmp, unsigned *flag);
+hipError_t tk_launch_salt_v2_gather(hipStream_t s, const TkSaltV2 &t, const uint32_t *rows, size_t count, float *out);
 #ifdef __cplusplus
 }
 #endif
