@@ -61,3 +61,23 @@ def test_branch_targets_start_from_the_state_at_the_jump():
 def test_other_kernels_are_not_scanned():
     text = "_Z14tk_flow_kernelILi1EEvv:\n\tglobal_load_dwordx4 v[1:4], v[8:9], off\n\tv_mov_b32_e32 v0, v1\n.Lfunc_end1:\n"
     assert check_isa.check_text(text) == {}
+
+
+def test_register_budgets():
+    """A kernel over its budget, one that spills, and one missing from the assembly are all reported."""
+    meta = """
+amdhsa.kernels:
+  - .name:           _Z5alphaILi1EEvv
+    .vgpr_count:     128
+    .vgpr_spill_count: 0
+  - .name:           _Z4betaILi2EEvv
+    .vgpr_count:     169
+    .vgpr_spill_count: 0
+  - .name:           _Z5gammaILi3EEvv
+    .vgpr_count:     100
+    .vgpr_spill_count: 4
+"""
+    budgets = (("alphaILi1E", 128), ("betaILi2E", 168), ("gammaILi3E", 128), ("deltaILi4E", 64))
+    bad = check_isa.check_budgets(meta, budgets)
+    assert ("_Z4betaILi2EEvv", 169, 168) in bad and ("_Z5gammaILi3EEvv", 10100, 128) in bad and ("deltaILi4E", None, 64) in bad
+    assert not any("alpha" in b[0] for b in bad) and len(bad) == 3

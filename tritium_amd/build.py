@@ -65,6 +65,11 @@ def build_library(verbose=True):
             bad = check_isa.check_text(f.read())
         if bad:
             raise RuntimeError("generated code reads registers of loads still in flight:\n" + check_isa.report(bad))
+        with open(asm_file.name) as f:
+            over = check_isa.check_budgets(f.read())
+        if over:
+            raise RuntimeError("kernels over their register budget (kernel, registers [+10000 = spills], budget):\n" +
+                               "\n".join(str(x) for x in over))
     finally:
         os.unlink(asm_file.name)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]

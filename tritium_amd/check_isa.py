@@ -111,6 +111,49 @@ def check_text(text, only=("tk_gemm",)):
     return found
 
 
+# Register budgets of the bandwidth kernels: (template arguments of the kernel, vector registers at most).
+# A CU runs floor(512 / registers) waves per SIMD, in steps of 8 registers: 128 -> 4, 168 -> 3, 256 -> 2. The
+# decode kernels' rate follows the bytes their waves keep in flight, so a change that pushes one of these
+# forms over its step (a few registers are enough) costs a third or a quarter of the rate without any test
+# noticing. The build fails instead.
+REGISTER_BUDGETS = (
+    ("tk_flow_kernelILi1ELi1ELi1ELi4ELb1E", 128),   # one plane, one run per wave: a single operand row
+    ("tk_flow_kernelILi1ELi1ELi2ELi4ELb1E", 128),   # one plane, two runs per wave: 2..16 rows
+    ("tk_flow_kernelILi2ELi1ELi1ELi4ELb1E", 128),   # two planes, up to 8 rows
+    ("tk_flow_kernelILi2ELi1ELi2ELi4ELb1E", 168),   # two planes, 9..16 rows
+    ("tk_flow32_kernelILi2ELi1ELi4ELb1E", 168),     # two planes, 25..32 rows
+    ("tk_flow_kernelILi2ELi4ELi2ELi2ELb1E", 256),   # two planes, 33..64 rows
+    ("tk_gemm32_kernelILi1ELi2ELb0ELb0E", 168),     # prefill, one plane (three waves per SIMD by design)
+    ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
+    ("tk_gemm32_kernelILi3ELi2ELb0ELb0E", 256),     # prefill, three planes (two waves per SIMD)
+)
+
+
+def check_budgets(text, budgets=REGISTER_BUDGETS):
+    """[(kernel, registers used, budget)] for every budgeted kernel over its budget, or that spills, or that
+    the assembly does not contain (a renamed kernel must not drop out of the check silently)."""
+    used, spills, name = {}, {}, None
+    for line in text.splitlines():
+        m = re.match(r"\s+\.name:\s+(\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.match(r"\s+\.vgpr_count:\s+(\d+)", line)
+        if m and name:
+            used[name] = int(m.group(1))
+        m = re.match(r"\s+\.vgpr_spill_count:\s+(\d+)", line)
+        if m and name:
+            spills[name] = int(m.group(1))
+    bad = []
+    for key, budget in budgets:
+        names = [n for n in used if key in n]
+        if not names:
+            bad.append((key, None, budget))
+        for n in names:
+            if used[n] > budget or spills.get(n, 0):
+                bad.append((n, used[n] + (10000 if spills.get(n, 0) else 0), budget))
+    return bad
+
+
 def report(found):
     out = []
     for name, hz in found.items():

@@ -246,8 +246,13 @@ __global__ __launch_bounds__(TK_WG) void tk_stream_kernel(TkProblem single, cons
 // ------------------------------------------------------------------------------------------
 
 
+// Waves per SIMD the register allocation must leave room for: two follow from the workgroup size (up to
+// eight waves); the form with two planes and two runs per wave on a ring of four sits at the edge of
+// three (168 registers) -- left alone it takes 169, which costs a third of the waves in flight and 8% of
+// the rate at 9..16 operand rows.
+#define TK_FLOW_MIN_WAVES(P, RT, TW, DR) (((P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
 template <int P, int RT, int TW, int DR, bool TABLE>
-__global__ __launch_bounds__(512) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                       const int *__restrict__ wg_prob) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : *single_problem();
