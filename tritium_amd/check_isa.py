@@ -134,13 +134,13 @@ def check_budgets(text, budgets=REGISTER_BUDGETS):
     the assembly does not contain (a renamed kernel must not drop out of the check silently)."""
     used, spills, name = {}, {}, None
     for line in text.splitlines():
-        m = re.match(r"\s+\.name:\s+(\S+)", line)
+        m = re.match(r"[\s-]+\.name:\s+(\S+)", line)
         if m:
             name = m.group(1)
-        m = re.match(r"\s+\.vgpr_count:\s+(\d+)", line)
+        m = re.match(r"[\s-]+\.vgpr_count:\s+(\d+)", line)
         if m and name:
             used[name] = int(m.group(1))
-        m = re.match(r"\s+\.vgpr_spill_count:\s+(\d+)", line)
+        m = re.match(r"[\s-]+\.vgpr_spill_count:\s+(\d+)", line)
         if m and name:
             spills[name] = int(m.group(1))
     bad = []
