@@ -511,6 +511,10 @@ int tk_set_flow_mfma(tk_ctx *ctx, int rows);
  * leave fewer than four workgroups per CU), 2 or 4 to force. A tuning and test knob: both forms give
  * identical bits. */
 int tk_set_gemm_tiles(tk_ctx *ctx, int tiles);
+/* The 64 x 128 form of the one-plane prefill kernel has its four waves side by side (64 rows x 32 outputs
+ * each). on != 0 arranges them two by two (32 rows x 64 outputs each: half the LDS reads, twice the weight
+ * loads; measured 3-6% slower, identical bits). A measurement knob. */
+int tk_set_gemm_two_by_two(tk_ctx *ctx, int on);
 /* K slices of the prefill kernel in single launches: 0 = chosen per launch (a launch with fewer
  * workgroups than CUs is cut into about one workgroup per CU, at least two K blocks per slice), 1 =
  * never split, 2..64 = that many slices where K allows. Integer partial sums, added by the last

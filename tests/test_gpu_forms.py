@@ -18,11 +18,20 @@ def automatic_dispatch(backend):
     backend.set_decode_kernel(0)
     backend.set_flow_mfma(0)
     backend.set_gemm_tiles(0)
+    backend.set_gemm_two_by_two(False)
     yield
     backend.set_decode_kernel(0)
     backend.set_flow_mfma(0)
     backend.set_gemm_tiles(0)
+    backend.set_gemm_two_by_two(False)
     backend.set_stream_min_groups(backend.info.compute_units)
+
+
+def _set_tiles(backend, tiles):
+    """2 = the 64 x 128 form of the one-plane prefill kernel with its four waves side by side (the default
+    arrangement), 22 = the same form with the waves two by two, 4 = the 64 x 256 form, 0 = automatic."""
+    backend.set_gemm_tiles(2 if tiles == 22 else tiles)
+    backend.set_gemm_two_by_two(tiles == 22)
 
 
 def _planes(rng, n, k, planes):
@@ -32,13 +41,13 @@ def _planes(rng, n, k, planes):
     return ws, scs, packed
 
 
-@pytest.mark.parametrize("tiles", [2, 4])
+@pytest.mark.parametrize("tiles", [2, 22, 4])
 @pytest.mark.parametrize("m,n,k", [(65, 8, 256), (130, 257, 512), (200, 129, 300), (128, 1040, 2560), (300, 2100, 768)])
 def test_one_plane_prefill_kernel_both_tile_counts(backend, oracle, tiles, m, n, k):
-    """tk_gemm32_kernel<1,2,false> and <1,4,false>: ragged tile counts (partial workgroups, partial
-    pairs), several row blocks, every output type."""
+    """tk_gemm32_kernel<1,4,false,false,2> (two by two), <1,2,false> and <1,4,false>: ragged tile counts
+    (partial workgroups, partial pairs), several row blocks, every output type."""
     print("case gemm-tiles", tiles, m, n, k, flush=True)
-    backend.set_gemm_tiles(tiles)
+    _set_tiles(backend, tiles)
     rng = np.random.default_rng(tiles * 1000 + m + n + k)
     ws, scs, packed = _planes(rng, n, k, 1)
     layer = backend.linear(packed, scs, n, k)
@@ -69,14 +78,14 @@ def test_one_plane_prefill_kernel_both_tile_counts(backend, oracle, tiles, m, n,
     layer.free()
 
 
-@pytest.mark.parametrize("planes,tiles", [(1, 2), (1, 4), (2, 0), (3, 0)])
+@pytest.mark.parametrize("planes,tiles", [(1, 2), (1, 22), (1, 4), (2, 0), (3, 0)])
 def test_grouped_prefill_kernel_every_plane_count(backend, oracle, planes, tiles):
     """A grouped decode launch whose operand rows exceed LDS runs the prefill kernel from a problem
     table: tk_gemm32_kernel<1,2,true>, <1,4,true>, <2,2,true>, <3,2,true>. Members of different widths
     (ragged tile counts), two sharing an activation; one member short enough for the flow kernel's
     share of the group. Bits equal the single launches and the CPU composition."""
     print("case grouped-prefill", planes, tiles, flush=True)
-    backend.set_gemm_tiles(tiles)
+    _set_tiles(backend, tiles)
     rng = np.random.default_rng(planes * 10 + tiles)
     m, k_long, k_short = 40, 4500, 768  # 40 rows x 18 K blocks = 184 KiB of operand rows: beyond LDS
     acts = {"a": rng.standard_normal((m, k_long)).astype(np.float32),
@@ -164,7 +173,7 @@ def test_gemm_tiles_knob_rejects_other_values(backend):
 
 
 @pytest.mark.parametrize("slices", [2, 3, 5, 0])
-@pytest.mark.parametrize("m,n,k,planes,tiles", [(64, 200, 2816, 3, 0), (40, 1040, 4352, 1, 2), (40, 1040, 4352, 1, 4),
+@pytest.mark.parametrize("m,n,k,planes,tiles", [(64, 200, 2816, 3, 0), (40, 1040, 4352, 1, 2), (40, 1040, 4352, 1, 22), (40, 1040, 4352, 1, 4),
                                                   (100, 50, 1300, 2, 0), (130, 131, 1024, 1, 0)])
 def test_prefill_kernel_k_split(backend, oracle, slices, m, n, k, planes, tiles):
     """Single launches of the prefill kernel with K cut into slices (tk_gemm32_kernel<P,NT,false,true>): int32
@@ -172,7 +181,7 @@ def test_prefill_kernel_k_split(backend, oracle, slices, m, n, k, planes, tiles)
     unsplit kernel's and the CPU composition's; a second call reuses the arrival counters (they must be
     back at zero); ragged slice counts (11, 17, 6, 4 K blocks over 2, 3, 5 slices) included."""
     print("case k-split", slices, m, n, k, planes, tiles, flush=True)
-    backend.set_gemm_tiles(tiles)
+    _set_tiles(backend, tiles)
     rng = np.random.default_rng(slices * 1000 + m + n + k)
     ws, scs, packed = _planes(rng, n, k, planes)
     layer = backend.linear(packed, scs, n, k)

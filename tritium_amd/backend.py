@@ -573,6 +573,10 @@ class Mi355xBackend:
         """0 automatic, 2 or 4 output tiles per wave of the one-plane prefill kernel."""
         _check(self._lib.tk_set_gemm_tiles(self._ctx, tiles))
 
+    def set_gemm_two_by_two(self, on):
+        """One-plane prefill kernel, 64 x 128 form: waves two by two instead of four side by side (same bits)."""
+        _check(self._lib.tk_set_gemm_two_by_two(self._ctx, 1 if on else 0))
+
     def set_gemm_ksplit(self, slices):
         """0 automatic, 1 off, 2..64 K slices of the prefill kernel in single launches."""
         _check(self._lib.tk_set_gemm_ksplit(self._ctx, slices))

@@ -77,6 +77,7 @@ struct tk_ctx {
   int flow_ring = 0;       // 0 = automatic
   int flow_mfma = 0;       // 0 = automatic, 16 / 32 = force the 16x16x64 / 32x32x32 form of the flow kernel
   int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
+  int gemm_two_by_two = 0;  // one-plane prefill kernel, 64 x 128 form: 0 = four waves side by side, 1 = two by two
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
   int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
@@ -320,6 +321,13 @@ extern "C" int tk_set_gemm_tiles(tk_ctx *ctx, int tiles) {
     return tk_fail(TK_ERR_INVALID_INPUT, "gemm_tiles=%d - use 0 (automatic), 2 or 4", tiles);
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->gemm_tiles = tiles;
+  return TK_OK;
+}
+
+extern "C" int tk_set_gemm_two_by_two(tk_ctx *ctx, int on) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_two_by_two: null context");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->gemm_two_by_two = on ? 1 : 0;
   return TK_OK;
 }
 
@@ -1019,6 +1027,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
       pr.kpart = (int32_t *)ctx->kpart.p;
       pr.kcount = (int *)ctx->kcount.p;
     }
+    pl.cfg.gemm_two_by_two = ctx->gemm_two_by_two;
     HIPCHK(tk_launch_gemm(ctx->stream, &pr, nullptr, nullptr, pl.cfg));
   }
   return TK_OK;
@@ -2009,6 +2018,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   g->cfg.lds_bytes = variant == DECODE_FLOW ? flds : (variant == DECODE_STREAM ? slds : lds);
   if (variant == DECODE_GEMM) g->cfg.lds_bytes = (size_t)tk_gemm_lds_bytes();
   g->cfg.gemm_nt = variant == DECODE_GEMM ? group_gemm_nt : 0;
+  g->cfg.gemm_two_by_two = ctx->gemm_two_by_two;
   g->cfg.grid = variant == DECODE_KSPLIT ? tiles : groups_total;
   g->cfg.waves = fw;
   {

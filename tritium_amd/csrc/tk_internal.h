@@ -115,7 +115,8 @@ struct TkLaunchCfg {
   int waves;    // flow kernel: waves per workgroup (4, or 8 when the operand rows need > 64 KiB of LDS)
   int ring;     // flow kernel: positions in the prefetch ring (2..5)
   int wide_mfma; // flow kernel: 32x32x32 form (17..64 operand rows, row constants in LDS)
-  int gemm_nt;  // prefill kernel, one plane: tiles per wave (0 = the default 4, or 2)
+  int gemm_nt;  // prefill kernel, one plane: 0 = 64 x 256 outputs per workgroup (4 tiles per wave), 2 = 64 x 128
+  int gemm_two_by_two;  // ... the 64 x 128 form with its waves two by two (32 rows x 4 tiles each) instead of side by side
   int tw;       // flow kernel, 16x16x64 form: runs per wave (tk_flow_runs_per_wave)
   int base3;    // flow kernel: stream the planes' base-3 copies (tk_launch_flow3)
 };

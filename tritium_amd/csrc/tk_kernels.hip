@@ -1202,9 +1202,9 @@ __device__ __forceinline__ void tk_gemm_epilogue(const TkProblem &pr, const TkHo
 // ------------------------------------------------------------------------------------------
 
 
-template <int P, int NT>
+template <int P, int NT, int WR>
 __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
-                                                   v16i (&acc)[2][NT * P / 2], uint8_t *smem, int tid, int bm, int bn);
+                                                   v16i (&acc)[2 / WR][NT * P / 2], uint8_t *smem, int tid, int bm, int bn);
 
 #ifndef TK_GEMM32_STAGES
 #define TK_GEMM32_STAGES 3
@@ -1216,10 +1216,22 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
 #define TK_GEMM32_OCC(P) ((P) >= 3 ? 2 : 3)
 #endif
 
-template <int P, int NT, bool TABLE, bool KSPLIT = false>
+// WR = 1: the four waves of a workgroup sit side by side, each over all 64 rows and its own NT tiles.
+// WR = 2: two by two -- a wave takes 32 of the rows and NT tiles of one half of the columns. Per k step a
+// wave then reads one 32-row A piece from LDS instead of two for the same number of matrix instructions
+// (with one plane and two tiles per wave side by side -- one pair: two reads, two instructions per step --
+// the four waves of a workgroup ask LDS for 128 bytes per clock at full matrix rate), and every weight
+// chunk is loaded by two waves instead of one. Measured on the 64 x 128 form of the one-plane kernel,
+// int8 rows in, bf16 out: 2048 x 2560 -> 6912 53.0 us side by side, 54.9 two by two; 512 tokens 20.2 /
+// 21.1; 2048 x 6912 -> 2560 53.3 / 56.6. The LDS reads are not what holds that form back; the doubled
+// weight loads cost more than the halved reads save. Side by side stays the default; two by two is
+// kept behind a knob (identical bits).
+template <int P, int NT, bool TABLE, bool KSPLIT = false, int WR = 1>
 __global__ __launch_bounds__(TK_GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(TK_GEMM32_OCC(P), TK_GEMM32_OCC(P)))) void
 tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, const int *__restrict__ wg_prob) {
   static_assert(NT % 2 == 0, "tiles are processed in pairs");
+  static_assert(WR == 1 || WR == 2, "one or two row groups");
+  constexpr int WC = TK_GEMM_WAVES / WR, RT2W = 2 / WR;  // column groups; 32-row tiles per wave
   static_assert(!(TABLE && KSPLIT), "the K split is for single launches");
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : single;
   const TkHot hot = make_hot(pr);
@@ -1260,7 +1272,8 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
   const int bn = (xcd / pr.xr) * sub_n + ln;
   if (lm >= sub_m || ln >= sub_n || bm >= pr.grid_m || bn >= pr.grid_n) return;
   const int row0 = bm * ROWS;
-  const int tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+  const int wr = wave / WC, wc = wave % WC;
+  const int tile0 = (bn * WC + wc) * NT;
 
   // per pair: this lane's address of load l = 0 in K block 0 (load 1 is 512 bytes further, block kb
   // kb KiB further); tiles past the end re-read the last tile (results dropped)
@@ -1299,9 +1312,9 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
                                        (__attribute__((address_space(3))) void *)(smem + CST + wave_u * 256), 4, 0, 0);
   }
 
-  v16i acc[2][NP];
+  v16i acc[RT2W][NP];
 #pragma unroll
-  for (int rt2 = 0; rt2 < 2; ++rt2)
+  for (int rt2 = 0; rt2 < RT2W; ++rt2)
 #pragma unroll
     for (int y = 0; y < NP; ++y)
 #pragma unroll
@@ -1311,15 +1324,15 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
   // that the destination registers of such a load are in flight until the wait: were it to split
   // their live range (a copy out and back under register pressure) it would read stale data. The
   // build checks the generated code for exactly that (tritium_amd/check_isa.py) and fails on it.
-  auto lds_read = [&](v4i (&a)[2], unsigned addr, int off) {
+  auto lds_read = [&](v4i (&a)[RT2W], unsigned addr, int off) {
 #pragma unroll
-    for (int rt2 = 0; rt2 < 2; ++rt2)
+    for (int rt2 = 0; rt2 < RT2W; ++rt2)
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[rt2]) : "v"(addr), "n"(off + rt2 * 512));
   };
-  auto lds_wait = [&](v4i (&a)[2]) {
+  auto lds_wait = [&](v4i (&a)[RT2W]) {
     asm volatile("s_waitcnt lgkmcnt(0)");
 #pragma unroll
-    for (int rt2 = 0; rt2 < 2; ++rt2) asm volatile("" : "+v"(a[rt2]));
+    for (int rt2 = 0; rt2 < RT2W; ++rt2) asm volatile("" : "+v"(a[rt2]));
   };
   auto load_w = [&](v4i (&w)[NP][2], int kb) {
 #pragma unroll
@@ -1367,14 +1380,15 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
   for (int q = 0; q < NS; ++q) tie_w(wset[q]);
   __builtin_amdgcn_s_barrier();
 
-  const unsigned lds_lane = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t *)smem + (unsigned)(kappa * ROWS + (lane & 31)) * 16u;
+  const unsigned lds_lane = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t *)smem +
+                            (unsigned)(kappa * ROWS + wr * RT2W * 32 + (lane & 31)) * 16u;
   auto block = [&](auto cur_c, int kb) {
     constexpr int cur = decltype(cur_c)::value, nxt = (cur + NS - 1) % NS, n1 = (cur + 1) % NS;
     if (kb + NS - 1 < nb) {
       load_w(wset[nxt], kb + NS - 1);
       dma_block(kb + NS - 1, nxt);
     }
-    v4i a[2];
+    v4i a[RT2W];
 #pragma unroll
     for (int l = 0; l < 2; ++l)
 #pragma unroll
@@ -1385,7 +1399,7 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
         for (int y = 0; y < NP; ++y) {
           const v4i b = expand_codes((uint32_t)wset[cur][y][l][j]);
 #pragma unroll
-          for (int rt2 = 0; rt2 < 2; ++rt2)
+          for (int rt2 = 0; rt2 < RT2W; ++rt2)
             acc[rt2][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[rt2], b, acc[rt2][y], 0, 0, 0);
         }
       }
@@ -1414,11 +1428,11 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
   if constexpr (KSPLIT) {
     // Partial sums out, one coalesced KiB per register; the last workgroup of the tile to arrive adds
     // the others' to its own and goes on to the epilogue. Integer adds: the order does not matter.
-    constexpr int NREG = 2 * NP * 16;
+    constexpr int NREG = RT2W * NP * 16;
     const int tile_id = bm * pr.grid_n + bn;
     int32_t *mine = pr.kpart + ((size_t)tile_id * ksn + ks) * (size_t)(NREG * TK_GEMM_THREADS) + tid_e;
 #pragma unroll
-    for (int rt2 = 0; rt2 < 2; ++rt2)
+    for (int rt2 = 0; rt2 < RT2W; ++rt2)
 #pragma unroll
       for (int y = 0; y < NP; ++y)
 #pragma unroll
@@ -1440,7 +1454,7 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
       if (k2 == ks) continue;
       int32_t *theirs = pr.kpart + ((size_t)tile_id * ksn + k2) * (size_t)(NREG * TK_GEMM_THREADS) + tid_e;
 #pragma unroll
-      for (int rt2 = 0; rt2 < 2; ++rt2)
+      for (int rt2 = 0; rt2 < RT2W; ++rt2)
 #pragma unroll
         for (int y = 0; y < NP; ++y)
 #pragma unroll
@@ -1451,15 +1465,17 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
     if (tid_e == 0) __hip_atomic_store(pr.kcount + tile_id, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero again for the next launch
     __syncthreads();  // `arrived` was read by everyone before the epilogue reuses the LDS
   }
-  tk_gemm32_epilogue<P, NT>(pr, hot, scales, acc, smem, (int)tid_e, bm, bn);
+  tk_gemm32_epilogue<P, NT, WR>(pr, hot, scales, acc, smem, (int)tid_e, bm, bn);
 }
 
-template <int P, int NT>
+template <int P, int NT, int WR>
 __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const TkHot &hot, const float *const (&scales)[P],
-                                                   v16i (&acc)[2][NT * P / 2], uint8_t *smem, int tid, int bm, int bn) {
+                                                   v16i (&acc)[2 / WR][NT * P / 2], uint8_t *smem, int tid, int bm, int bn) {
   constexpr int ROWS = 64, A4 = 16 * ROWS, CST = TK_GEMM32_STAGES * A4 * 16, HP = NT / 2;
+  constexpr int WC = TK_GEMM_WAVES / WR, RT2W = 2 / WR;
   const int wave = tid >> 6, lane = tid & 63, r16 = lane & 15, h = (lane >> 4) & 1, kappa = lane >> 5;
-  const int R = hot.R, row0 = bm * ROWS, tile0 = (bn * TK_GEMM_WAVES + wave) * NT;
+  const int wr = wave / WC, wc = wave % WC;
+  const int R = hot.R, row0 = bm * ROWS, tile0 = (bn * WC + wc) * NT;
   const int n_tiles = (hot.n + 15) >> 4;
   const int *cst_rs = (const int *)(smem + CST);
   const float *cst_as = (const float *)(smem + CST + 256);
@@ -1511,7 +1527,7 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
   // (a call with a fused residual add takes the direct stores: the residual is read where the value is formed)
   const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0 && !hot.residual;
   if (staged) {
-    constexpr int WG_COLS = TK_GEMM_WAVES * NT * 16;
+    constexpr int WG_COLS = WC * NT * 16;
     const bool int8_mode = hot.mode == TK_MODE_INT8 || hot.out_dtype == TK_I32;
     const int halves = esz == 4 ? 2 : 1;       // 4-byte outputs take the 64 rows in two halves
     const int orows_half = int8_mode ? (64 / halves) : (16 / halves);
@@ -1524,16 +1540,16 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
     for (int hh = 0; hh < halves; ++hh) {
       if (hh > 0) __syncthreads();
 #pragma unroll
-      for (int rt2 = 0; rt2 < 2; ++rt2) {
-        if (halves == 2 && rt2 != hh) continue;
+      for (int rt2 = 0; rt2 < RT2W; ++rt2) {
+        if (halves == 2 && wr * RT2W + rt2 != hh) continue;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int rl = rt2 * 32 + 8 * q + 4 * kappa;             // first of this lane's 4 rows, tile-local
+          const int rl = (wr * RT2W + rt2) * 32 + 8 * q + 4 * kappa;  // first of this lane's 4 rows, tile-local
           const int sl = rl - (halves == 2 ? hh * 32 : 0);         // ... staging-local
           const RowConst rc = row_const(rl);
 #pragma unroll
           for (int z = 0; z < HP; ++z) {
-            const int cl = (wave * NT + 2 * z + h) * 16 + r16;
+            const int cl = (wc * NT + 2 * z + h) * 16 + r16;
             v4i av[P];
             quad(rt2, q, z, av);
             if (hot.out_dtype == TK_I32) {
@@ -1567,10 +1583,10 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
     }
   } else {
 #pragma unroll
-    for (int rt2 = 0; rt2 < 2; ++rt2)
+    for (int rt2 = 0; rt2 < RT2W; ++rt2)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int rl = rt2 * 32 + 8 * q + 4 * kappa;
+        const int rl = (wr * RT2W + rt2) * 32 + 8 * q + 4 * kappa;
         const RowConst rc = row_const(rl);
 #pragma unroll
         for (int z = 0; z < HP; ++z) {
@@ -1586,9 +1602,9 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
     for (int z = 0; z < HP; ++z) {
       const int t = tile0 + 2 * z + h, n = t * 16 + r16;
       if (t >= pr.n_tiles || n >= pr.n) continue;
-      for (int rt2 = 0; rt2 < 2; ++rt2)
+      for (int rt2 = 0; rt2 < RT2W; ++rt2)
         for (int q = 0; q < 4; ++q) {
-          const int rowbase = row0 + rt2 * 32 + 8 * q + 4 * kappa;
+          const int rowbase = row0 + (wr * RT2W + rt2) * 32 + 8 * q + 4 * kappa;
           const unsigned fl = row_flags(pr, rowbase);
           if (fl) exact_rows(pr, n, rowbase, fl);
         }
@@ -2817,7 +2833,10 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
   const unsigned wgs = table ? cfg.grid : 8u * (unsigned)sg.sub_m * (unsigned)sg.sub_n * (ksplit ? (unsigned)sg.ksplit : 1u);
   if (!wgs) return hipSuccess;
   if (ksplit) {
-    if (cfg.planes == 1 && cfg.gemm_nt == 2) return gemm_launch_one(tk_gemm32_kernel<1, 2, false, true>, s, sg, table, wg_prob, cfg, wgs);
+    if (cfg.planes == 1 && cfg.gemm_nt == 2) {
+      if (!cfg.gemm_two_by_two) return gemm_launch_one(tk_gemm32_kernel<1, 2, false, true>, s, sg, table, wg_prob, cfg, wgs);
+      return gemm_launch_one(tk_gemm32_kernel<1, 4, false, true, 2>, s, sg, table, wg_prob, cfg, wgs);
+    }
     switch (cfg.planes) {
       case 1: return gemm_launch_one(tk_gemm32_kernel<1, 4, false, true>, s, sg, table, wg_prob, cfg, wgs);
       case 2: return gemm_launch_one(tk_gemm32_kernel<2, 2, false, true>, s, sg, table, wg_prob, cfg, wgs);
@@ -2833,9 +2852,13 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
 #define TK_GEMM32_CASE(PP, NTT)                                                                              \
   if (table) return gemm_launch_one(tk_gemm32_kernel<PP, NTT, true>, s, sg, table, wg_prob, cfg, wgs);        \
   return gemm_launch_one(tk_gemm32_kernel<PP, NTT, false>, s, sg, table, wg_prob, cfg, wgs);
-  if (cfg.planes == 1 && cfg.gemm_nt == 2) {
-    if (table) return gemm_launch_one(tk_gemm32_kernel<1, 2, true>, s, sg, table, wg_prob, cfg, wgs);
-    return gemm_launch_one(tk_gemm32_kernel<1, 2, false>, s, sg, table, wg_prob, cfg, wgs);
+  if (cfg.planes == 1 && cfg.gemm_nt == 2) {  // 64 x 128 outputs per workgroup: four waves side by side, or two by two
+    if (!cfg.gemm_two_by_two) {
+      if (table) return gemm_launch_one(tk_gemm32_kernel<1, 2, true>, s, sg, table, wg_prob, cfg, wgs);
+      return gemm_launch_one(tk_gemm32_kernel<1, 2, false>, s, sg, table, wg_prob, cfg, wgs);
+    }
+    if (table) return gemm_launch_one(tk_gemm32_kernel<1, 4, true, false, 2>, s, sg, table, wg_prob, cfg, wgs);
+    return gemm_launch_one(tk_gemm32_kernel<1, 4, false, false, 2>, s, sg, table, wg_prob, cfg, wgs);
   }
   switch (cfg.planes) {
     case 1: TK_GEMM32_CASE(1, 4)
