@@ -515,6 +515,10 @@ int tk_set_gemm_tiles(tk_ctx *ctx, int tiles);
  * each). on != 0 arranges them two by two (32 rows x 64 outputs each: half the LDS reads, twice the weight
  * loads; measured 3-6% slower, identical bits). A measurement knob. */
 int tk_set_gemm_two_by_two(tk_ctx *ctx, int on);
+/* Activation prep (quantization / digit split): launches of up to `rows` tokens give every token a whole
+ * workgroup instead of one wave (few tokens: the launch lasts as long as one token's chain of instructions).
+ * Default 384 (the digit split of the float contract: 8/3 of it). Process-wide; identical bits either way. A tuning and test knob. */
+int tk_set_prep_team_rows(tk_ctx *ctx, int rows);
 /* K slices of the prefill kernel in single launches: 0 = chosen per launch (a launch with fewer
  * workgroups than CUs is cut into about one workgroup per CU, at least two K blocks per slice), 1 =
  * never split, 2..64 = that many slices where K allows. Integer partial sums, added by the last

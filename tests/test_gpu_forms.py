@@ -226,3 +226,66 @@ def test_prefill_kernel_k_split(backend, oracle, slices, m, n, k, planes, tiles)
     for a in (dact, d0):
         a.free()
     layer.free()
+
+
+@pytest.mark.parametrize("mode", [1, 0])
+@pytest.mark.parametrize("k,m,copies", [(256, 1, 40), (2048, 4, 10), (2560, 2, 20), (6912, 3, 12), (17408, 1, 3), (6912, 40, 1),
+                                          (2000, 2, 20)])
+def test_activation_prep_forms_agree(backend, oracle, mode, k, m, copies):
+    """The quantization / digit-split launch has three forms: a wave per token, a workgroup per token (both in
+    a straight-line variant for rows of whole K blocks, up to 8 pieces held per thread), and the general
+    workgroup-per-token kernels. Forced either way through the knob, a grouped launch of `copies` members must
+    give the same bits, and the int8 contract the oracle's (rows with NaN, Inf, all zeros and a single
+    non-zero element included; K=2000 is not whole blocks: the general kernels)."""
+    print("case prep-forms", mode, k, m, copies, flush=True)
+    if mode == 0 and m * 4 > 64:
+        pytest.skip("float groups take at most 16 tokens")
+    rng = np.random.default_rng(k + m * 7 + copies + mode)
+    n = 48
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    acts = []
+    for c in range(copies):
+        a = (rng.standard_normal((m, k)) * 10.0 ** rng.integers(-3, 3)).astype(np.float32)
+        if c == 1:
+            a[0] = 0.0
+        if c == 2:
+            a[0] = 0.0
+            a[0, k // 2] = -3.25
+        if c == 3:
+            a[m - 1, 5] = np.nan
+        if c == 4:
+            a[0, k - 1] = np.inf
+        acts.append(a)
+    results = []
+    for team_rows in (0, 1 << 20):
+        backend.set_prep_team_rows(team_rows)
+        for dt in ("f32", "bf16"):
+            host = [f32_to_bf16_bits(a) if dt == "bf16" else a for a in acts]
+            seen = [bf16_bits_to_f32(h).reshape(m, k) if dt == "bf16" else h for h in host]
+            dev = [backend.to_device(h, dt) for h in host]
+            outs = [backend.empty(m * n, "f32") for _ in range(copies)]
+            grp = backend.group([(layer, dev[c], m, outs[c]) for c in range(copies)], mode, dt, "f32")
+            grp.launch()
+            got = [o.to_host().reshape(m, n) for o in outs]
+            results.append(got)
+            if mode == 1:
+                for c in range(copies):
+                    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, seen[c], m, n, k).reshape(m, n)
+                    fin = ~np.isnan(want)
+                    assert (np.isnan(got[c]) == ~fin).all() and same_bits(got[c][fin], want[fin])
+            else:
+                for c in range(copies):
+                    want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, seen[c], m, n, k).reshape(m, n)
+                    fin = ~np.isnan(want)
+                    assert (np.isnan(got[c]) == ~fin).all() and accepts(got[c][fin], want[fin], rel=1e-4, floor=1.0).all()
+            grp.destroy()
+            for x in dev + outs:
+                x.free()
+    backend.set_prep_team_rows(384)
+    for dt_i in range(2):  # same element type, the two settings
+        for c in range(copies):
+            a, b = results[dt_i][c], results[2 + dt_i][c]
+            fin = ~np.isnan(a)
+            assert (np.isnan(b) == ~fin).all() and same_bits(a[fin], b[fin])
+    layer.free()

@@ -577,6 +577,10 @@ class Mi355xBackend:
         """One-plane prefill kernel, 64 x 128 form: waves two by two instead of four side by side (same bits)."""
         _check(self._lib.tk_set_gemm_two_by_two(self._ctx, 1 if on else 0))
 
+    def set_prep_team_rows(self, rows):
+        """Activation prep: launches of up to `rows` tokens give a token the whole workgroup (default 384)."""
+        _check(self._lib.tk_set_prep_team_rows(self._ctx, rows))
+
     def set_gemm_ksplit(self, slices):
         """0 automatic, 1 off, 2..64 K slices of the prefill kernel in single launches."""
         _check(self._lib.tk_set_gemm_ksplit(self._ctx, slices))

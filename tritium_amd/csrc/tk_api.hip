@@ -331,6 +331,14 @@ extern "C" int tk_set_gemm_two_by_two(tk_ctx *ctx, int on) {
   return TK_OK;
 }
 
+extern "C" int tk_set_prep_team_rows(tk_ctx *ctx, int rows) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_prep_team_rows: null context");
+  if (rows < 0) return tk_fail(TK_ERR_INVALID_INPUT, "prep_team_rows=%d - use 0 or more", rows);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  tk_prep_set_team_rows(rows);
+  return TK_OK;
+}
+
 extern "C" int tk_set_gemm_ksplit(tk_ctx *ctx, int slices) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_ksplit: null context");
   if (slices < 0 || slices > 64) return tk_fail(TK_ERR_INVALID_INPUT, "gemm_ksplit=%d - use 0 (automatic), 1 (off) or 2..64", slices);
@@ -1686,6 +1694,7 @@ struct tk_group {
   int nprobs = 0, nprep = 0, prep_kind = 0;
   int prep_uniform_m = 0;    // > 0: prep entry j starts at token j * prep_uniform_m
   int prep_wave_pieces = 0;  // > 0: every entry fits the one-wave-per-token prep kernels; the largest piece count
+  int prep_fast = 0;         // tk_prep_fast of every entry when they agree
   unsigned prep_rows = 0;
   int variant = 1;
   size_t wg_prob_off = 0;
@@ -2008,10 +2017,13 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     size_t pieces = 0;
     bool ok = true;
     for (const TkPrep &pp : preps) {
-      ok = ok && pp.nb * 16 <= 256 && !pp.norm_kind && !pp.blocksum;
+      ok = ok && !pp.norm_kind && !pp.blocksum;  // (which form, if any, takes that many pieces: the launcher's rule)
       if (pp.nb * 16 > pieces) pieces = pp.nb * 16;
     }
     if (ok) g->prep_wave_pieces = (int)pieces;
+    g->prep_fast = preps.empty() ? 0 : tk_prep_fast(preps[0]);
+    for (const TkPrep &pp : preps)
+      if (tk_prep_fast(pp) != g->prep_fast) g->prep_fast = 0;
   }
   g->cfg.planes = planes;
   g->cfg.rt = rt;
@@ -2044,7 +2056,7 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
   if (do_prep)
     HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows,
-                          g->prep_wave_pieces));
+                          g->prep_wave_pieces, g->prep_fast));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
   if (do_main && g->has_flow_part)
     HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),

@@ -2241,9 +2241,29 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_kernel(TkPrep single, co
 // The token a wave works on, and its tensor. Single tensor, workgroup count a multiple of 16: eight
 // consecutive rows share every 128-byte line of the operand layout, and workgroups go to the 8 XCDs
 // in turn, so the two workgroups that cover rows 8j..8j+7 are taken from the same XCD.
+// (team: the threads working on one token -- a wave, or the whole workgroup)
 __device__ __forceinline__ const TkPrep &find_prep_wave(const TkPrep &single, const TkPrep *table, int nprep,
-                                                        int uniform_m, int wave, int &row, int &gt) {
+                                                        int uniform_m, int wave, int &row, int &gt, int team = 64) {
   const unsigned blk = blockIdx.x;
+  if (team != 64) {
+    gt = (int)blk;
+    if (!table) {
+      row = gt;
+      return single;
+    }
+    if (uniform_m > 0) {
+      const int t = min(gt / uniform_m, nprep - 1);
+      row = gt - t * uniform_m;
+      return table[t];
+    }
+    int lo = 0, hi = nprep - 1;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (table[mid].row_begin <= gt) lo = mid; else hi = mid - 1;
+    }
+    row = gt - table[lo].row_begin;
+    return table[lo];
+  }
   if (!table) {
     if ((gridDim.x & 15u) == 0) {
       const unsigned xcd = blk & 7u, slot = blk >> 3;
@@ -2274,16 +2294,43 @@ __device__ __forceinline__ int wave_sum(int v) {
   return v;
 }
 
-template <int HELD>
+// FAST != 0: the launch's rows are whole K blocks (k a multiple of 256), 16-byte aligned, of one element type
+// (1 = f32, 2 = bf16) and only the operand rows are wanted: no bound, alignment or type is tested per
+// element, which is most of what the general form executes (a wave works through its token alone, one
+// dependent instruction after the other: the instruction count is the launch's time).
+template <int FAST>
+__device__ __forceinline__ void load_piece_fast(const void *act, size_t base, size_t e0, float (&v)[16]) {
+#pragma unroll
+  for (int sl = 0; sl < 4; ++sl) {
+    if constexpr (FAST == 2) {
+      typedef unsigned v2u __attribute__((ext_vector_type(2)));
+      const v2u u = *(const TK_GLOBAL v2u *)((const uint16_t *)act + base + e0 + sl * 32);
+      v[sl * 4 + 0] = __uint_as_float(u.x << 16);
+      v[sl * 4 + 1] = __uint_as_float(u.x & 0xFFFF0000u);
+      v[sl * 4 + 2] = __uint_as_float(u.y << 16);
+      v[sl * 4 + 3] = __uint_as_float(u.y & 0xFFFF0000u);
+    } else {
+      const v4u u = *(const TK_GLOBAL v4u *)((const float *)act + base + e0 + sl * 32);
+      v[sl * 4 + 0] = __uint_as_float(u.x);
+      v[sl * 4 + 1] = __uint_as_float(u.y);
+      v[sl * 4 + 2] = __uint_as_float(u.z);
+      v[sl * 4 + 3] = __uint_as_float(u.w);
+    }
+  }
+}
+
+template <int HELD, int FAST = 0, int TEAM = 64>
 __device__ __forceinline__ void wave_absmax_held(const void *act, int dtype, size_t base, size_t k, size_t npieces, bool vec,
-                                                 int lane, float (&held)[HELD][16], float &gamma, int &nonfinite) {
+                                                 int lane, float (&held)[HELD][16], float &gamma, int &nonfinite,
+                                                 float *shf = nullptr, int *shi = nullptr) {
   float g = 0.0f;
   int nf = 0;
 #pragma unroll
   for (int it = 0; it < HELD; ++it) {
-    const size_t pc = (size_t)lane + (size_t)it * 64;
+    const size_t pc = (size_t)lane + (size_t)it * TEAM;
     if (pc < npieces) {
-      load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, held[it]);
+      if constexpr (FAST != 0) load_piece_fast<FAST>(act, base, piece_elem0(pc >> 4, (int)(pc & 15)), held[it]);
+      else load_piece(act, dtype, base, piece_elem0(pc >> 4, (int)(pc & 15)), k, vec, held[it]);
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
         const float a = fabsf(held[it][x]);  // elements past k were loaded as 0
@@ -2292,21 +2339,30 @@ __device__ __forceinline__ void wave_absmax_held(const void *act, int dtype, siz
       }
     }
   }
-  for (int o = 32; o > 0; o >>= 1) {
-    g = fmaxf(g, __shfl_xor(g, o));
-    nf |= __shfl_xor(nf, o);
+  if constexpr (TEAM == 64) {
+    for (int o = 32; o > 0; o >>= 1) {
+      g = fmaxf(g, __shfl_xor(g, o));
+      nf |= __shfl_xor(nf, o);
+    }
+  } else {
+    block_max_any(g, nf, shf, shi);
   }
   gamma = g;
   nonfinite = nf != 0;
 }
 
-template <int HELD>
+// TEAM = 64: a wave per token, four tokens per workgroup, no barrier. TEAM = 256: the workgroup per token (the
+// maximum and the sums cross its waves through LDS): a quarter of the instructions per thread, for launches
+// of few tokens, whose time is one token's chain.
+template <int HELD, int FAST = 0, int TEAM = 64>
 __global__ __launch_bounds__(TK_WG) void tk_prep_a8_wave_kernel(TkPrep single, const TkPrep *__restrict__ table, int nprep,
                                                                 int uniform_m, unsigned rows) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __shared__ float shf[4];
+  __shared__ int shi[4];
+  const int wave = threadIdx.x >> 6, lane = TEAM == 64 ? (threadIdx.x & 63) : threadIdx.x;
   int rowi, gt;
-  const TkPrep &pp = find_prep_wave(single, table, nprep, uniform_m, wave, rowi, gt);
-  if ((unsigned)gt >= rows) return;  // no barrier anywhere below
+  const TkPrep &pp = find_prep_wave(single, table, nprep, uniform_m, wave, rowi, gt, TEAM);
+  if ((unsigned)gt >= rows) return;  // (a whole team leaves together: the barriers below stay uniform)
   const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = row * k;
   const void *act = pp.act;
@@ -2317,13 +2373,39 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_wave_kernel(TkPrep single, c
   float held[HELD][16];
   float gamma;
   int nonfinite;
-  wave_absmax_held<HELD>(act, dtype, base, k, npieces, vec, lane, held, gamma, nonfinite);
+  wave_absmax_held<HELD, FAST, TEAM>(act, dtype, base, k, npieces, vec, lane, held, gamma, nonfinite, shf, shi);
   const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
   const bool live = gamma != 0.0f && !nonfinite;
   int sum = 0;
+  if constexpr (FAST != 0) {
+    // a multiply by 0 stands in for the tests of `live` (a row without a finite maximum quantizes to zeros)
+    const float sl_ = live ? s : 0.0f;
+#pragma unroll
+    for (int it = 0; it < HELD; ++it) {
+      const size_t pc = (size_t)lane + (size_t)it * TEAM;
+      if (pc >= npieces) continue;
+      v4u piece;
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          float x = held[it][sl * 4 + b];
+          if (!live) x = 0.0f;  // (a NaN or Inf times zero would not be zero)
+          float r = rintf(__fmul_rn(x, sl_));  // one multiply, ties to even
+          r = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+          const int q = (int)r;
+          sum += q;
+          packed |= ((uint32_t)q & 0xFFu) << (8 * b);
+        }
+        piece[sl] = packed;
+      }
+      *(TK_GLOBAL v4u *)(ap + piece_offset(pc >> 4, (int)(pc & 15), R, row)) = piece;
+    }
+  } else
 #pragma unroll
   for (int it = 0; it < HELD; ++it) {
-    const size_t pc = (size_t)lane + (size_t)it * 64;
+    const size_t pc = (size_t)lane + (size_t)it * TEAM;
     if (pc >= npieces) continue;
     const size_t kb = pc >> 4;
     const int q16 = (int)(pc & 15);
@@ -2356,7 +2438,8 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_wave_kernel(TkPrep single, c
     }
     if (ap) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, row)) = piece;
   }
-  sum = wave_sum(sum);
+  if constexpr (TEAM == 64) sum = wave_sum(sum);
+  else sum = block_sum(sum, shi);
   if (lane == 0) {
     if (pp.rowsum) pp.rowsum[row] = sum;
     pp.act_scale[row] = gamma == 0.0f ? 0.0f : __fdiv_rn(gamma, 127.0f);
@@ -2365,12 +2448,14 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_wave_kernel(TkPrep single, c
   }
 }
 
-template <int HELD>
+template <int HELD, int FAST = 0, int TEAM = 64>
 __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                                     int nprep, int uniform_m, unsigned rows) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __shared__ float shf[4];
+  __shared__ int shi[32];
+  const int wave = threadIdx.x >> 6, lane = TEAM == 64 ? (threadIdx.x & 63) : threadIdx.x;
   int rowi, gt;
-  const TkPrep &pp = find_prep_wave(single, table, nprep, uniform_m, wave, rowi, gt);
+  const TkPrep &pp = find_prep_wave(single, table, nprep, uniform_m, wave, rowi, gt, TEAM);
   if ((unsigned)gt >= rows) return;
   const size_t tok = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
   const size_t base = tok * k;
@@ -2382,7 +2467,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
   float held[HELD][16];
   float gamma;
   int nonfinite;
-  wave_absmax_held<HELD>(act, dtype, base, k, npieces, vec, lane, held, gamma, nonfinite);
+  wave_absmax_held<HELD, FAST, TEAM>(act, dtype, base, k, npieces, vec, lane, held, gamma, nonfinite, shf, shi);
   int E = 0;
   if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
   const int shift = 30 - E;
@@ -2390,7 +2475,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
   int sums[4] = {0, 0, 0, 0}, n_poor = 0;
 #pragma unroll
   for (int it = 0; it < HELD; ++it) {
-    const size_t pc = (size_t)lane + (size_t)it * 64;
+    const size_t pc = (size_t)lane + (size_t)it * TEAM;
     if (pc >= npieces) continue;
     const size_t kb = pc >> 4;
     const int q16 = (int)(pc & 15);
@@ -2403,7 +2488,11 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         int q = 0;
-        if (live && e + b < k) {
+        if constexpr (FAST != 0) {  // every element is inside the row; a row without a finite maximum splits zeros
+          const float r = ldexpf(live ? held[it][sl * 4 + b] : 0.0f, shift);
+          q = __float2int_rn(r);  // |q| <= 2^30
+          n_poor += digit_poor(r, q) ? 1 : 0;
+        } else if (live && e + b < k) {
           const float r = ldexpf(held[it][sl * 4 + b], shift);
           q = __float2int_rn(r);  // |q| <= 2^30
           n_poor += digit_poor(r, q) ? 1 : 0;
@@ -2422,19 +2511,31 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
 #pragma unroll
     for (int dg = 0; dg < 4; ++dg) *(TK_GLOBAL v4u *)(ap + piece_offset(kb, q16, R, tok * 4 + dg)) = piece[dg];
   }
+  if constexpr (TEAM == 64) {
 #pragma unroll
-  for (int dg = 0; dg < 4; ++dg) sums[dg] = wave_sum(sums[dg]);
-  n_poor = wave_sum(n_poor);
+    for (int dg = 0; dg < 4; ++dg) sums[dg] = wave_sum(sums[dg]);
+    n_poor = wave_sum(n_poor);
+  } else {
+    int five[5] = {sums[0], sums[1], sums[2], sums[3], n_poor};
+    block_sums<5>(five, shi);
+#pragma unroll
+    for (int dg = 0; dg < 4; ++dg) sums[dg] = five[dg];
+    n_poor = five[4];
+  }
   bool narrow = false;
-  if (n_poor > 0) {  // wave-uniform
+  if (n_poor > 0) {  // uniform over the team
     int bands[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int it = 0; it < HELD; ++it) {
-      const size_t pc = (size_t)lane + (size_t)it * 64;
+      const size_t pc = (size_t)lane + (size_t)it * TEAM;
       if (pc < npieces) count_bands(held[it], shift, bands);
     }
+    if constexpr (TEAM == 64) {
 #pragma unroll
-    for (int b = 0; b < 8; ++b) bands[b] = wave_sum(bands[b]);
+      for (int b = 0; b < 8; ++b) bands[b] = wave_sum(bands[b]);
+    } else {
+      block_sums<8>(bands, shi);
+    }
     narrow = digits_narrow(n_poor, bands);
   }
   if (lane < 4) pp.rowsum[tok * 4 + lane] = lane == 0 ? sums[0] : lane == 1 ? sums[1] : lane == 2 ? sums[2] : sums[3];
@@ -2537,28 +2638,64 @@ hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n,
   return hipGetLastError();
 }
 
+// Launches of up to this many tokens (quantization; the digit split, which does more per element, up to 8/3 of
+// it) give a token the whole workgroup (tk_launch_prep). Measured, wave per token / workgroup per token:
+// quantization K=2048 256 tokens 4.1 / 3.7 us, 512 tokens 4.2 / 4.5; K=6912 120 tokens 7.1 / 4.6, 960 tokens
+// 8.8 / 9.7; digit split K=2048 512 tokens 5.9 / 5.7, 1024 tokens 8.1 / 7.0, 2048 tokens 10.7 / 11.7.
+static int g_prep_team_rows = 384;
+void tk_prep_set_team_rows(int rows) { g_prep_team_rows = rows < 0 ? 0 : rows; }
+int tk_prep_fast(const TkPrep &pp) {
+  const bool ok = pp.k % 256 == 0 && (((size_t)pp.act) & 15) == 0 && pp.ap && !pp.q_rowmajor && !pp.norm_kind && !pp.blocksum;
+  if (!ok) return 0;
+  return pp.act_dtype == TK_F32 ? 1 : (pp.act_dtype == TK_BF16 ? 2 : 0);
+}
+
 hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
-                          unsigned rows, int table_wave_pieces) {
+                          unsigned rows, int table_wave_pieces, int table_fast) {
   if (!rows) return hipSuccess;
   TkPrep dummy = {};
   const TkPrep &sg = single ? *single : dummy;
-  // one wave per token where every row has at most 256 pieces and needs neither a norm nor per-block sums
-  size_t wave_pieces = (size_t)(table_wave_pieces > 0 ? table_wave_pieces : 0);
-  if (single) wave_pieces = (single->nb * 16 <= 256 && !single->norm_kind && !single->blocksum) ? single->nb * 16 : 0;
-  // a handful of tokens is a latency problem: a whole workgroup per token finishes a row sooner
-  if (rows < 32) wave_pieces = 0;
-  if (wave_pieces && (kind == TK_PREP_A8 || kind == TK_PREP_DIGITS)) {
-    const dim3 grid((rows + 3) / 4), block(TK_WG);
-    const int held = wave_pieces <= 64 ? 1 : (wave_pieces <= 128 ? 2 : 4);
+  // Rows that need neither a norm nor per-block sums, whose pieces the threads working on a token can keep
+  // in registers. Team = the threads of one token: a wave (four tokens per workgroup, no barrier), up to 4
+  // pieces per lane (K <= 4096) or 8 in the straight-line form (whole K blocks, aligned rows of one element
+  // type, operand rows only), whose registers hold little else; or, in the straight-line form, the whole
+  // workgroup (up to 8 pieces per thread: K <= 32768), where few tokens make the launch one token's chain of
+  // instructions (g_prep_team_rows tokens and fewer).
+  const int fast = single ? tk_prep_fast(*single) : table_fast;
+  size_t pieces = (size_t)(table_wave_pieces > 0 ? table_wave_pieces : 0);
+  if (single) pieces = (!single->norm_kind && !single->blocksum) ? single->nb * 16 : 0;
+  const bool plain = pieces && (kind == TK_PREP_A8 || kind == TK_PREP_DIGITS);
+  const bool team_wg = plain && fast && pieces <= 8 * (size_t)TK_WG && (rows <= (unsigned)(kind == TK_PREP_DIGITS ? g_prep_team_rows * 8 / 3 : g_prep_team_rows) || pieces > 512);
+  const bool team_wave = plain && !team_wg && rows >= 32 && pieces <= (fast ? 512u : 256u);
+  if (team_wg || team_wave) {
+    const size_t team = team_wg ? TK_WG : 64;
+    const dim3 grid(team_wg ? rows : (rows + 3) / 4), block(TK_WG);
+    const size_t per = (pieces + team - 1) / team;
+    const int held = per <= 1 ? 1 : (per <= 2 ? 2 : (per <= 4 ? 4 : 8));
+#define TK_WAVE_PREP(KERNEL, H, F, T) hipLaunchKernelGGL((KERNEL<H, F, T>), grid, block, 0, s, sg, table, nprep, uniform_m, rows)
+#define TK_WAVE_PREP_H(KERNEL, F, T)                    \
+  switch (held) {                                       \
+    case 1: TK_WAVE_PREP(KERNEL, 1, F, T); break;       \
+    case 2: TK_WAVE_PREP(KERNEL, 2, F, T); break;       \
+    case 4: TK_WAVE_PREP(KERNEL, 4, F, T); break;       \
+    default: TK_WAVE_PREP(KERNEL, 8, F, T); break;      \
+  }
+#define TK_WAVE_PREP_K(KERNEL)                                                         \
+  if (team_wg) {                                                                       \
+    if (fast == 2) { TK_WAVE_PREP_H(KERNEL, 2, 256) } else { TK_WAVE_PREP_H(KERNEL, 1, 256) } \
+  } else if (fast == 2) { TK_WAVE_PREP_H(KERNEL, 2, 64) }                              \
+  else if (fast == 1) { TK_WAVE_PREP_H(KERNEL, 1, 64) }                                \
+  else if (held == 1) TK_WAVE_PREP(KERNEL, 1, 0, 64);                                  \
+  else if (held == 2) TK_WAVE_PREP(KERNEL, 2, 0, 64);                                  \
+  else TK_WAVE_PREP(KERNEL, 4, 0, 64)
     if (kind == TK_PREP_A8) {
-      if (held == 1) hipLaunchKernelGGL(tk_prep_a8_wave_kernel<1>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
-      else if (held == 2) hipLaunchKernelGGL(tk_prep_a8_wave_kernel<2>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
-      else hipLaunchKernelGGL(tk_prep_a8_wave_kernel<4>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+      TK_WAVE_PREP_K(tk_prep_a8_wave_kernel);
     } else {
-      if (held == 1) hipLaunchKernelGGL(tk_prep_digits_wave_kernel<1>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
-      else if (held == 2) hipLaunchKernelGGL(tk_prep_digits_wave_kernel<2>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
-      else hipLaunchKernelGGL(tk_prep_digits_wave_kernel<4>, grid, block, 0, s, sg, table, nprep, uniform_m, rows);
+      TK_WAVE_PREP_K(tk_prep_digits_wave_kernel);
     }
+#undef TK_WAVE_PREP_K
+#undef TK_WAVE_PREP_H
+#undef TK_WAVE_PREP
     return hipGetLastError();
   }
   switch (kind) {
