@@ -1,5 +1,5 @@
 """Zero-block bitmaps (crates/tritium-format/src/tq2.rs:101-181): the oracle's restatement against
-every case the reference's own tests hold (tq2.rs:187-207, 259-377) and an independent numpy statement;
+every case the reference's own tests hold (tq2.rs:187-207, 259-370) and an independent numpy statement;
 then the product's host function against the oracle."""
 import ctypes as C
 
