@@ -43,6 +43,37 @@ def test_overwrite_and_partial_waits():
     assert list(bad.values())[0][0][2] == 21
 
 
+def test_lds_reads_one_step_ahead():
+    # lgkmcnt(2) retires all but the two youngest LDS reads: the pair read first may feed the matrix
+    # instruction, the pair read ahead may not be touched until its own wait
+    ok = run("""
+	ds_read_b128 v[10:13], v2
+	ds_read_b128 v[14:17], v2 offset:512
+	ds_read_b128 v[20:23], v2 offset:4096
+	ds_read_b128 v[24:27], v2 offset:4608
+	s_waitcnt lgkmcnt(2)
+	v_mfma_i32_32x32x32_i8 v[40:55], v[10:13], v[30:33], v[40:55]
+	s_waitcnt lgkmcnt(0)
+	v_mfma_i32_32x32x32_i8 v[40:55], v[20:23], v[30:33], v[40:55]
+""")
+    assert ok == {}
+    bad = run("""
+	ds_read_b128 v[10:13], v2
+	ds_read_b128 v[20:23], v2 offset:4096
+	s_waitcnt lgkmcnt(1)
+	v_mov_b32_e32 v5, v22
+	s_waitcnt lgkmcnt(0)
+""")
+    assert list(bad.values())[0][0][2] == 22
+    # a vmcnt wait does not retire LDS reads
+    bad = run("""
+	ds_read_b128 v[10:13], v2
+	s_waitcnt vmcnt(0)
+	v_mov_b32_e32 v5, v10
+""")
+    assert list(bad.values())[0][0][2] == 10
+
+
 def test_branch_targets_start_from_the_state_at_the_jump():
     # the zero-fill path is entered by a jump taken before the loads were issued
     ok = run("""

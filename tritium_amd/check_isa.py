@@ -17,6 +17,7 @@ import sys
 _VREG_RANGE = re.compile(r"\bv\[(\d+):(\d+)\]")
 _VREG_ONE = re.compile(r"\bv(\d+)\b")
 _VMCNT = re.compile(r"vmcnt\((\d+)\)")
+_LGKMCNT = re.compile(r"lgkmcnt\((\d+)\)")
 
 
 def _vregs(text):
@@ -35,6 +36,7 @@ def check_function(name, lines):
     through keeps the state of the code above it; backward branches (loops) are not re-walked, which
     is enough here because every iteration of the pipelined loops ends in the same wait."""
     pending = []  # issue order: (destination registers, line) of every vector-memory operation
+    lds = []      # the same for LDS and scalar-memory operations (one counter, lgkmcnt); LDS returns in order
     at_label = {}  # label -> loads in flight at the first forward jump to it
     reachable = True
     hazards = []
@@ -44,7 +46,7 @@ def check_function(name, lines):
             if ins.endswith(":"):  # a local label
                 label = ins[:-1]
                 if not reachable:
-                    pending = list(at_label.get(label, []))
+                    pending, lds = (list(x) for x in at_label.get(label, ([], [])))
                 reachable = True
             continue
         if ins.endswith(":"):
@@ -53,7 +55,7 @@ def check_function(name, lines):
             continue
         op = ins.split()[0]
         if op.startswith("s_cbranch") or op == "s_branch":
-            at_label.setdefault(ins.split()[-1], list(pending))
+            at_label.setdefault(ins.split()[-1], (list(pending), list(lds)))
             if op == "s_branch":
                 reachable = False
             continue
@@ -65,8 +67,22 @@ def check_function(name, lines):
             if m:
                 keep = int(m.group(1))
                 pending = pending[len(pending) - keep:] if keep else []
+            m = _LGKMCNT.search(ins)
+            if m:
+                keep = int(m.group(1))
+                lds = lds[len(lds) - keep:] if keep else []
             continue
-        in_flight = set().union(*(p[0] for p in pending)) if pending else set()
+        in_flight = set().union(*(p[0] for p in pending + lds)) if pending or lds else set()
+        if op.startswith(("ds_", "s_load", "s_buffer_load")):
+            # the prefill kernels read their A pieces one k step ahead and wait with lgkmcnt(N > 0)
+            operands = ins[len(op):].split(",")
+            is_read = op.startswith(("ds_read", "ds_load"))
+            dest = _vregs(operands[0]) if is_read else set()
+            used = _vregs(",".join(operands[1:])) if is_read else _vregs(ins)
+            for r in sorted((used | dest) & in_flight):
+                hazards.append((no, ins, r))
+            lds.append((dest, no))
+            continue
         if op.startswith("global_load_lds"):  # LDS-DMA: counted by vmcnt, no destination register
             used = _vregs(ins)
             dest = set()

@@ -15,6 +15,23 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
+// float -> bf16, round to nearest even, NaN quieted with its sign and upper payload kept: gfx950's
+// v_cvt_pk_bf16_f32 (what the vector conversion below compiles to) gives, for every one of the 2^32
+// float bit patterns, the bits of the integer statement
+//   nan ? (u >> 16) | 0x40 : (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+// (compared exhaustively on the device).
+typedef float tk_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 tk_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+  const tk_f32x2 v = {lo, hi};
+  const tk_bf16x2 h = __builtin_convertvector(v, tk_bf16x2);
+  uint32_t bits;
+  __builtin_memcpy(&bits, &h, 4);
+  return bits;
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_hw(float x) { return (uint16_t)f32x2_to_bf16x2(x, x); }
+// The integer statement, for the decode kernels: their register budgets are fitted to it (the
+// instruction form changed the allocation of two of them enough to spill).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float x) {
   uint32_t u = __float_as_uint(x);
   if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);

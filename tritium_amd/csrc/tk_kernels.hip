@@ -1338,8 +1338,11 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
     for (int rt2 = 0; rt2 < RT2W; ++rt2)
       asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[rt2]) : "v"(addr), "n"(off + rt2 * 512));
   };
-  auto lds_wait = [&](v4i (&a)[RT2W]) {
-    asm volatile("s_waitcnt lgkmcnt(0)");
+  // wait until only the RT2W reads of the next k step (`ahead`) or none are still in flight: LDS reads
+  // return in order
+  auto lds_wait = [&](v4i (&a)[RT2W], bool ahead) {
+    if (ahead) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(RT2W));
+    else asm volatile("s_waitcnt lgkmcnt(0)");
 #pragma unroll
     for (int rt2 = 0; rt2 < RT2W; ++rt2) asm volatile("" : "+v"(a[rt2]));
   };
@@ -1397,21 +1400,22 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
       load_w(wset[nxt], kb + NS - 1);
       dma_block(kb + NS - 1, nxt);
     }
-    v4i a[RT2W];
+    // the A pieces of k step s + 1 are read while the matrix instructions of step s run
+    v4i a[2][RT2W];
+    lds_read(a[0], lds_lane, cur * (A4 * 16));
 #pragma unroll
-    for (int l = 0; l < 2; ++l)
+    for (int s = 0; s < 8; ++s) {
+      const int l = s >> 2, j = s & 3;
+      if (s < 7) lds_read(a[(s + 1) & 1], lds_lane, cur * (A4 * 16) + (((s + 1) & 3) * 4 + 2 * ((s + 1) >> 2)) * (ROWS * 16));
+      lds_wait(a[s & 1], s < 7);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        lds_read(a, lds_lane, cur * (A4 * 16) + (j * 4 + 2 * l) * (ROWS * 16));
-        lds_wait(a);
+      for (int y = 0; y < NP; ++y) {
+        const v4i b = expand_codes((uint32_t)wset[cur][y][l][j]);
 #pragma unroll
-        for (int y = 0; y < NP; ++y) {
-          const v4i b = expand_codes((uint32_t)wset[cur][y][l][j]);
-#pragma unroll
-          for (int rt2 = 0; rt2 < RT2W; ++rt2)
-            acc[rt2][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[rt2], b, acc[rt2][y], 0, 0, 0);
-        }
+        for (int rt2 = 0; rt2 < RT2W; ++rt2)
+          acc[rt2][y] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[s & 1][rt2], b, acc[rt2][y], 0, 0, 0);
       }
+    }
     // blocks issued after kb+1 and still allowed in flight: kb+2 .. min(kb+NS-1, nb-1)
     wait_blocks(min(kb + NS - 1, nb - 1) - (kb + 1));
     tie_w(wset[n1]);
@@ -1483,7 +1487,7 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
   constexpr int ROWS = 64, A4 = 16 * ROWS, CST = TK_GEMM32_STAGES * A4 * 16, HP = NT / 2;
   constexpr int WC = TK_GEMM_WAVES / WR, RT2W = 2 / WR;
   const int wave = tid >> 6, lane = tid & 63, r16 = lane & 15, h = (lane >> 4) & 1, kappa = lane >> 5;
-  const int wr = wave / WC, wc = wave % WC;
+  const int wr = WR == 1 ? 0 : wave / WC, wc = WR == 1 ? wave : wave % WC;
   const int R = hot.R, row0 = bm * ROWS, tile0 = (bn * WC + wc) * NT;
   const int n_tiles = (hot.n + 15) >> 4;
   const int *cst_rs = (const int *)(smem + CST);
@@ -1535,7 +1539,69 @@ __device__ __forceinline__ void tk_gemm32_epilogue(const TkProblem &pr, const Tk
   const int esz = hot.out_dtype == TK_BF16 ? 2 : 4;
   // (a call with a fused residual add takes the direct stores: the residual is read where the value is formed)
   const bool staged = (((size_t)hot.n * esz) & 15) == 0 && (((size_t)hot.out) & 15) == 0 && !hot.residual;
-  if (staged) {
+  // The common case -- int8 contract, f32 or bf16 out, no row of the tile flagged -- as straight-line code
+  // with compile-time strides: the general staging below decides contract, output type and flags per
+  // output (about 25 instructions and several branches each, as long as a short K loop).
+  auto lean = [&](auto esz_c, auto as_c) {
+    constexpr int ESZ = decltype(esz_c)::value;
+    constexpr bool HAS_AS = decltype(as_c)::value;
+    constexpr int WG_COLS = WC * NT * 16, HALVES = ESZ == 4 ? 2 : 1, OROWS = 64 / HALVES;
+    constexpr int STRIDE = WG_COLS * ESZ + 16, PIECES_ROW = WG_COLS * ESZ / 16, PER16 = 16 / ESZ;
+    const int col0 = bn * WG_COLS;
+    uint8_t *lane_base = smem + (size_t)(4 * kappa) * STRIDE + ((wc * NT + h) * 16 + r16) * ESZ;
+    const int *lane_rs = cst_rs + 4 * kappa;
+    const float *lane_as = cst_as + 4 * kappa;
+#pragma unroll
+    for (int hh = 0; hh < HALVES; ++hh) {
+      if (hh > 0) __syncthreads();
+#pragma unroll
+      for (int rt2 = 0; rt2 < RT2W; ++rt2) {
+        const int rtile = wr * RT2W + rt2;  // this wave's 32-row tile inside the 64 rows
+        if (HALVES == 2 && rtile != hh) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rl = rtile * 32 + 8 * q, sl = rl - (HALVES == 2 ? hh * 32 : 0);
+          RowConst rc;
+          const v4i rs4 = *(const v4i *)(lane_rs + rl);
+          rc.rs[0] = rs4.x; rc.rs[1] = rs4.y; rc.rs[2] = rs4.z; rc.rs[3] = rs4.w;
+          if (HAS_AS) {
+            const float4 as4 = *(const float4 *)(lane_as + rl);
+            rc.as[0] = as4.x; rc.as[1] = as4.y; rc.as[2] = as4.z; rc.as[3] = as4.w;
+          }
+#pragma unroll
+          for (int z = 0; z < HP; ++z) {
+            v4i av[P];
+            quad(rt2, q, z, av);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float f = int8_value<P>(av, r, sc[z], rc, HAS_AS);
+              uint8_t *dst = lane_base + (size_t)(sl + r) * STRIDE + z * 32 * ESZ;
+              if (ESZ == 2) *(uint16_t *)dst = f32_to_bf16_hw(f); else *(float *)dst = f;
+            }
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int it = 0; it < OROWS * PIECES_ROW / TK_GEMM_THREADS; ++it) {
+        const int pc = it * TK_GEMM_THREADS + tid;
+        const int rl = pc / PIECES_ROW, piece = pc % PIECES_ROW;
+        const int orow = row0 + hh * OROWS + rl, c = col0 + piece * PER16;
+        if (orow < R && c < hot.n)
+          *(TK_GLOBAL v4u *)((uint8_t *)hot.out + ((size_t)orow * hot.n + c) * ESZ) = *(const v4u *)(smem + (size_t)rl * STRIDE + piece * 16);
+      }
+    }
+  };
+  if (staged && hot.mode == TK_MODE_INT8 && hot.out_dtype != TK_I32 && !wg_flag) {
+    const bool has_as = hot.act_scale != nullptr;
+    if (esz == 2) {
+      if (has_as) lean(std::integral_constant<int, 2>{}, std::true_type{});
+      else lean(std::integral_constant<int, 2>{}, std::false_type{});
+    } else {
+      if (has_as) lean(std::integral_constant<int, 4>{}, std::true_type{});
+      else lean(std::integral_constant<int, 4>{}, std::false_type{});
+    }
+  } else if (staged) {
     constexpr int WG_COLS = WC * NT * 16;
     const bool int8_mode = hot.mode == TK_MODE_INT8 || hot.out_dtype == TK_I32;
     const int halves = esz == 4 ? 2 : 1;       // 4-byte outputs take the 64 rows in two halves
