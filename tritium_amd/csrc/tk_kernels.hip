@@ -1394,15 +1394,15 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
 
   const unsigned lds_lane = (unsigned)(size_t)(__attribute__((address_space(3))) uint8_t *)smem +
                             (unsigned)(kappa * ROWS + wr * RT2W * 32 + (lane & 31)) * 16u;
+  v4i a[2][RT2W];
   auto block = [&](auto cur_c, int kb) {
     constexpr int cur = decltype(cur_c)::value, nxt = (cur + NS - 1) % NS, n1 = (cur + 1) % NS;
     if (kb + NS - 1 < nb) {
       load_w(wset[nxt], kb + NS - 1);
       dma_block(kb + NS - 1, nxt);
     }
-    // the A pieces of k step s + 1 are read while the matrix instructions of step s run
-    v4i a[2][RT2W];
-    lds_read(a[0], lds_lane, cur * (A4 * 16));
+    // the A pieces of k step s + 1 are read while the matrix instructions of step s run; those of step 0
+    // were read at the end of the block before (or ahead of the loop)
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int l = s >> 2, j = s & 3;
@@ -1420,7 +1420,9 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
     wait_blocks(min(kb + NS - 1, nb - 1) - (kb + 1));
     tie_w(wset[n1]);
     __builtin_amdgcn_s_barrier();
+    lds_read(a[0], lds_lane, n1 * (A4 * 16));  // after the last block: a read of stale rows, waited for below
   };
+  lds_read(a[0], lds_lane, 0);
   int kb = 0;
   for (; kb + NS <= nb; kb += NS) {  // one exit only: the accumulators keep their registers
     block(std::integral_constant<int, 0>{}, kb);
@@ -1436,6 +1438,7 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
     }
   }
 
+  lds_wait(a[0], false);  // the read issued behind the last block
   unsigned tid_e = threadIdx.x;
   asm volatile("" : "+v"(tid_e));
   if constexpr (KSPLIT) {
