@@ -519,6 +519,11 @@ int tk_set_gemm_two_by_two(tk_ctx *ctx, int on);
  * workgroup instead of one wave (few tokens: the launch lasts as long as one token's chain of instructions).
  * Default 384 (the digit split of the float contract: 8/3 of it). Process-wide; identical bits either way. A tuning and test knob. */
 int tk_set_prep_team_rows(tk_ctx *ctx, int rows);
+/* Row count of the workgroup tile for single launches of one plane under the int8 contract (f32 or bf16
+ * rows of whole 16-byte pieces at a 16-byte aligned address, no residual): 0 = chosen per launch, 64 = the
+ * 64-row kernels, 128 = the 128 x 256 kernel, which shares both operands through LDS. Other launches take
+ * the 64-row kernels whatever this says. A tuning and test knob: identical bits. */
+int tk_set_gemm_rows(tk_ctx *ctx, int rows);
 /* K slices of the prefill kernel in single launches: 0 = chosen per launch (a launch with fewer
  * workgroups than CUs is cut into about one workgroup per CU, at least two K blocks per slice), 1 =
  * never split, 2..64 = that many slices where K allows. Integer partial sums, added by the last

@@ -19,11 +19,13 @@ def automatic_dispatch(backend):
     backend.set_flow_mfma(0)
     backend.set_gemm_tiles(0)
     backend.set_gemm_two_by_two(False)
+    backend.set_gemm_rows(0)
     yield
     backend.set_decode_kernel(0)
     backend.set_flow_mfma(0)
     backend.set_gemm_tiles(0)
     backend.set_gemm_two_by_two(False)
+    backend.set_gemm_rows(0)
     backend.set_stream_min_groups(backend.info.compute_units)
 
 
@@ -74,6 +76,77 @@ def test_one_plane_prefill_kernel_both_tile_counts(backend, oracle, tiles, m, n,
     rc, wantf = oracle.cpu_mpgemm(packed[0], FMT_TQ2_0, act[:mf], scs[0], mf, n, k)
     assert rc == 0 and accepts(got, wantf, rel=1e-4, floor=1.0).all()
     for a in (dact, dout, dob, dq, dacc, dof):
+        a.free()
+    layer.free()
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 8, 256), (130, 264, 512), (129, 136, 300), (128, 1040, 2560), (300, 2104, 768),
+                                   (257, 4104, 256), (640, 520, 1280)])
+def test_prefill_kernel_128_rows(backend, oracle, m, n, k):
+    """tk_gemm128_kernel forced at small sizes: partial row blocks and column blocks, odd and even half-block
+    counts, one to several workgroups per XCD; f32 and bf16 outputs from float rows (with an all-zero token and
+    two tokens that hold NaN / Inf and take the reference-order path) and from int8 rows; against the 64-row
+    kernels and the CPU oracle, bit for bit. Shapes it does not take fall back to the 64-row kernels."""
+    print("case gemm-128", m, n, k, flush=True)
+    rng = np.random.default_rng(128000 + m + n + k)
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[m // 2] = 0.0
+    act[1, k // 3] = np.nan
+    act[m - 1, 0] = np.inf
+    dact = backend.to_device(act, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    nan = np.isnan(want)
+    got = {}
+    for rows in (128, 64):
+        backend.set_gemm_rows(rows)
+        dout = backend.empty(m * n, "f32")
+        backend.linear_a8(layer, dact, m, dout)
+        got[rows] = dout.to_host().reshape(m, n)
+        assert (np.isnan(got[rows]) == nan).all()
+        assert same_bits(got[rows][~nan], want[~nan])
+        dob = backend.empty(m * n, "bf16")
+        backend.linear_a8(layer, dact, m, dob)
+        gb = dob.to_host().reshape(m, n)
+        assert (gb[~nan] == f32_to_bf16_bits(want)[~nan]).all()
+        dout.free()
+        dob.free()
+    # int8 rows in, with and without per-token scales
+    backend.set_gemm_rows(128)
+    q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    asc = rng.uniform(0.01, 0.2, m).astype(np.float32)
+    dq, dsc, do = backend.to_device(q, "i8"), backend.to_device(asc, "f32"), backend.empty(m * n, "f32")
+    acc = oracle.int8_accumulators(packed[0], FMT_TQ2_0, q, m, n, k).astype(np.float32)
+    backend.linear_i8(layer, dq, dsc, m, do)
+    assert same_bits(do.to_host().reshape(m, n), (acc * scs[0][None, :]) * asc[:, None])
+    backend.linear_i8(layer, dq, None, m, do)
+    assert same_bits(do.to_host().reshape(m, n), acc * scs[0][None, :])
+    for a in (dact, dq, dsc, do):
+        a.free()
+    layer.free()
+
+
+def test_prefill_kernel_128_rows_leaves_other_shapes_alone(backend, oracle):
+    """Output rows that are not whole 16-byte pieces, raw accumulators and a fused residual stay with the
+    64-row kernels even when 128 rows are asked for."""
+    backend.set_gemm_rows(128)
+    rng = np.random.default_rng(77)
+    m, n, k = 130, 257, 512
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    dact, dout = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    backend.linear_a8(layer, dact, m, dout)
+    assert same_bits(dout.to_host(), want)
+    q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    dq, dacc = backend.to_device(q, "i8"), backend.empty(m * n, "i32")
+    backend.linear_i8(layer, dq, None, m, dacc)
+    assert (dacc.to_host().reshape(m, n) == oracle.int8_accumulators(packed[0], FMT_TQ2_0, q, m, n, k)).all()
+    with pytest.raises(T.InvalidInput):
+        backend.set_gemm_rows(96)
+    for a in (dact, dout, dq, dacc):
         a.free()
     layer.free()
 

@@ -581,6 +581,10 @@ class Mi355xBackend:
         """Activation prep: launches of up to `rows` tokens give a token the whole workgroup (default 384)."""
         _check(self._lib.tk_set_prep_team_rows(self._ctx, rows))
 
+    def set_gemm_rows(self, rows):
+        """0 = automatic, 64 / 128 = rows of the workgroup tile for one-plane int8-contract prefill launches."""
+        _check(self._lib.tk_set_gemm_rows(self._ctx, rows))
+
     def set_gemm_ksplit(self, slices):
         """0 automatic, 1 off, 2..64 K slices of the prefill kernel in single launches."""
         _check(self._lib.tk_set_gemm_ksplit(self._ctx, slices))

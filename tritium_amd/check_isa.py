@@ -142,6 +142,7 @@ REGISTER_BUDGETS = (
     ("tk_gemm32_kernelILi1ELi2ELb0ELb0E", 168),     # prefill, one plane (three waves per SIMD by design)
     ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
     ("tk_gemm32_kernelILi3ELi2ELb0ELb0E", 256),     # prefill, three planes (two waves per SIMD)
+    ("tk_gemm128_kernel", 128),                     # prefill, 128 x 256 form (four waves per SIMD)
 )
 
 

@@ -79,6 +79,7 @@ struct tk_ctx {
   int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
   int gemm_two_by_two = 0;  // one-plane prefill kernel, 64 x 128 form: 0 = four waves side by side, 1 = two by two
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
+  int gemm_rows = 0;       // one-plane int8-contract prefill, single launches: 0 = tile rows chosen per launch, 64 / 128 = force
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
   int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
   unsigned *d_count = nullptr;  // a device counter for the uploads
@@ -336,6 +337,14 @@ extern "C" int tk_set_prep_team_rows(tk_ctx *ctx, int rows) {
   if (rows < 0) return tk_fail(TK_ERR_INVALID_INPUT, "prep_team_rows=%d - use 0 or more", rows);
   std::lock_guard<std::mutex> lk(ctx->mu);
   tk_prep_set_team_rows(rows);
+  return TK_OK;
+}
+
+extern "C" int tk_set_gemm_rows(tk_ctx *ctx, int rows) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_rows: null context");
+  if (rows != 0 && rows != 64 && rows != 128) return tk_fail(TK_ERR_INVALID_INPUT, "gemm_rows=%d - use 0 (automatic), 64 or 128", rows);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->gemm_rows = rows;
   return TK_OK;
 }
 
@@ -791,6 +800,43 @@ static void plan_gemm(Plan *pl, unsigned fill = 0, int force_nt = 0) {
   }
 }
 
+// The 128 x 256 kernel's grid: row blocks of 128 operand rows, column blocks of 16 tiles, split over the
+// XCDs like plan_gemm's (the operand-row stride plan_gemm chose stays).
+static void plan_gemm128(Plan *pl) {
+  TkProblem &pr = pl->pr;
+  pl->grid_m = (unsigned)(((size_t)pr.R + 127) / 128);
+  pl->grid_n = ((unsigned)pr.n_tiles + 15u) / 16u;
+  pr.grid_m = (int)pl->grid_m;
+  pr.grid_n = (int)pl->grid_n;
+  pr.ksplit = 0;
+  size_t best = (size_t)-1;
+  for (int xr = 1; xr <= 8; xr *= 2) {
+    const int xc = 8 / xr;
+    const int sm = ((int)pl->grid_m + xr - 1) / xr, sn = ((int)pl->grid_n + xc - 1) / xc;
+    const size_t cost = (size_t)128 * sm + (size_t)64 * sn;  // bytes touched per XCD and unit of K
+    const size_t waste = (size_t)8 * sm * sn;
+    const size_t score = cost * 1024 + waste;
+    if (score < best) {
+      best = score;
+      pr.xr = xr;
+      pr.sub_m = sm;
+      pr.sub_n = sn;
+    }
+  }
+}
+
+// Where the 128 x 256 kernel is chosen over the 64-row forms: launches it finishes in one round of its 512
+// resident workgroups (two per CU) and that still give most CUs one. A/B on one box, int8 rows in, bf16 out,
+// call incl. the operand re-ordering launch, 64-row kernels -> 128 x 256: 2048 x 2560 -> 6912 (432 blocks)
+// 47.9 -> 44.7 us; 1024 tokens (216) 30.0 -> 28.2; 512 tokens (108) 17.6 -> 24.8; 256 tokens 13.8 -> 23.6;
+// 2048 x 6912 -> 2560 (160) 52.0 -> 56.8; 2048 x 2560 -> 2560 (160) 27.7 -> 30.0; and with several rounds:
+// 8192 x 2560 -> 6912 (1728) 135 -> 140; 4096 x 5120 -> 17408 (2176) 288 -> 302; 4096 x 17408 -> 5120 (640)
+// 294 -> 330.
+static bool gemm128_pays(const tk_ctx *ctx, size_t rows, size_t blocks128) {
+  const size_t cus = (size_t)ctx->info.compute_units;
+  return rows >= 1024 && blocks128 * 4 >= cus * 3 && blocks128 <= 2 * cus;
+}
+
 static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_t k, size_t m, int mode,
                        int out_dtype, Plan *pl) {
   memset(pl, 0, sizeof *pl);
@@ -1007,6 +1053,18 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else if (pl.skinny) {
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
   } else {
+    // One plane under the int8 contract with whole 16-byte output pieces: the 128 x 256 kernel moves a third
+    // of the bytes per op through the CU's memory path (both operands shared through LDS).
+    const size_t esz = out_dtype == TK_BF16 ? 2 : 4;
+    const bool can128 = pr.planes == 1 && mode == TK_MODE_INT8 && (out_dtype == TK_F32 || out_dtype == TK_BF16) && !residual &&
+                        (n * esz) % 16 == 0 && ((uintptr_t)out & 15) == 0;
+    const size_t blocks128 = ((R + 127) / 128) * (((size_t)pr.n_tiles + 15) / 16);
+    const bool want128 = ctx->gemm_rows == 128 || (ctx->gemm_rows == 0 && gemm128_pays(ctx, R, blocks128));
+    if (can128 && want128) {
+      plan_gemm128(&pl);
+      HIPCHK(tk_launch_gemm128(ctx->stream, &pr));
+      return TK_OK;
+    }
     // A single launch with few workgroups is a latency chain over K per workgroup: cut K into slices.
     // The partial sums cost 4 bytes per accumulator and slice, so few slices: measured, call incl.
     // quantization, 64 tokens x 3 planes: 17408 -> 5120 (40 workgroups) 108 us unsplit, 72 / 56 / 54 / 72

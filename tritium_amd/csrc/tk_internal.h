@@ -172,6 +172,10 @@ hipError_t tk_launch_salt_flow(hipStream_t s, const TkProblem *single, const TkL
 hipError_t tk_launch_salt_seq(hipStream_t s, const TkProblem *single);
 hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                           const TkLaunchCfg &cfg);
+// 128 x 256 prefill kernel (tk_gemm128.hip): one plane, int8 contract, f32 / bf16 rows of whole 16-byte pieces,
+// no residual; grid from the problem's XCD split over 128-row x 16-tile blocks
+int tk_gemm128_lds_bytes(void);
+hipError_t tk_launch_gemm128(hipStream_t s, const TkProblem *single);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);
 // The three gradients of one packed mpGEMM (tk_vjp.hip); a null output is skipped.
 hipError_t tk_launch_projected_vjp(hipStream_t s, const uint8_t *codes, size_t nb, size_t n, size_t k, size_t m,
