@@ -2326,6 +2326,13 @@ __device__ __forceinline__ const TkPrep &find_prep_wave(const TkPrep &single, co
   if (team != 64) {
     gt = (int)blk;
     if (!table) {
+      // Eight consecutive tokens share every 128-byte line of the operand rows (16 bytes each): workgroups
+      // id, id + 8, ... run on one XCD, so give that XCD runs of eight tokens and its L2 whole lines to
+      // write back.
+      if ((gridDim.x & 63u) == 0) {
+        const unsigned xcd = blk & 7u, slot = blk >> 3;
+        gt = (int)((((slot >> 3) * 8u + xcd) * 8u) + (slot & 7u));
+      }
       row = gt;
       return single;
     }
