@@ -557,6 +557,48 @@ def bench_salt(T, be, rng, iters=30):
     return res
 
 
+def bench_salt_v2(T, be, rng, iters=10):
+    """SALT V2 exact matvec (the reference's pinned scalar order per output: correctness first, no matrix
+    cores): 4096 x 4096 coefficients in 65,536 allocation tiles of two planes each, D2 codec, scale groups
+    of 128; f32 activations and outputs. Sampled outputs are checked against a float64 product of the
+    dequantized matrix."""
+    n = k = 4096
+    tiles = n * k // 256
+    planes = []
+    for p0 in (0.4, 0.7):
+        trits = ternary(rng, n, k, p0).reshape(-1)
+        planes.append((trits, T.salt_v2_pack(T.SALT_V2_D2, trits).reshape(tiles, 64),
+                       rng.uniform(0.02, 1.0, (tiles, 2)).astype(np.float16)))
+    payload = np.stack([planes[0][1], planes[1][1]], axis=1).reshape(-1)   # tile after tile, planes in order
+    scales = np.stack([planes[0][2], planes[1][2]], axis=1).reshape(-1)    # one per (plane, group of 128)
+    dev = be.salt_v2_upload(T.SALT_V2_D2, 128, payload, scales.view(np.uint16), np.full(tiles, 2, np.uint8), n, k)
+    res = {"workload": f"SALT V2 {n} x {k}, two planes per tile, D2 codec, scale group 128, exact order, f32 in/out"}
+    rows = np.array([0, 1, n // 2, n - 1])
+    dense = np.zeros((rows.size, k))
+    for trits, _, sc in planes:
+        for i, r in enumerate(rows):
+            seg = slice(int(r) * k, int(r) * k + k)
+            dense[i] += trits[seg].astype(np.float64) * np.repeat(sc.reshape(-1)[int(r) * k // 128:(int(r) * k + k) // 128].astype(np.float64), 128)
+    for m in (1, 8):
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        act, out = be.to_device(a, "f32"), be.empty(m * n, "f32")
+        dev.forward(act, m, out)
+        got = out.to_host().reshape(m, n)[:, rows].astype(np.float64)
+        want = a.astype(np.float64) @ dense.T
+        err = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+        if err > 1e-4:
+            raise SystemExit(f"salt_v2 leg: output off by {err:.2e} of the largest value")
+        ms = time_calls(be, lambda i: dev.forward(act, m, out), iters)
+        by = payload.size + scales.size * 2 + m * k * 4 + m * n * 4
+        res[f"batch{m}"] = {"ms_per_call": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+                            "frac_of_hbm_peak": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+                            "verified": f"{m} token(s) x {rows.size} outputs within {err:.1e} of float64"}
+        act.free()
+        out.free()
+    dev.free()
+    return res
+
+
 def bench_vjp(T, be, rng, iters=5):
     """mpgemm_projected_vjp on the configs[2] projection (M=2048 tokens, K=2560, N=6912, one plane),
     device-resident f32 operands. Each gradient is timed on its own; flops = one multiply and one add
@@ -691,7 +733,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,base3,salt,vjp",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,base3,salt,salt_v2,vjp",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -750,6 +792,7 @@ def main():
                 "zero_skip": ("zero_chunk_skip", lambda: bench_zero_skip(T, be, rng)),
                 "base3": ("base3_stream_vs_two_bit", lambda: bench_base3(T, be, rng)),
                 "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng)),
+                "salt_v2": ("salt_v2_exact", lambda: bench_salt_v2(T, be, rng)),
                 "vjp": ("projected_vjp", lambda: bench_vjp(T, be, rng))}
         out["extra"] = {}
         for leg in [x for x in args.extra_legs.split(",") if x]:

@@ -73,7 +73,8 @@ def test_salt_rows_dense_and_sparse_through_the_block_scale_kernels(backend, ora
 @pytest.mark.parametrize("codec", [S.D2, S.B3, S.S34])
 @pytest.mark.parametrize("n,k,counts,group,m", [(3, 173, [1, 3, 2], 128, 2), (5, 173, [1, 3, 2, 3], 128, 1), (64, 256, None, 128, 9),
                                                  (7, 100, None, 64, 3), (33, 1024, None, 128, 17), (1, 4, [1], 128, 1),
-                                                 (130, 2048, None, 64, 8)])
+                                                 (130, 2048, None, 64, 8), (10, 384, None, 128, 5), (9, 192, None, 64, 2),
+                                                 (70, 640, None, 128, 13)])
 def test_v2_forward_and_gather_carry_the_reference_bits(backend, so, codec, n, k, counts, group, m):
     print("case salt-v2", codec, n, k, group, m, flush=True)
     if codec == S.S34 and (n * k) % 4:
@@ -130,6 +131,38 @@ def test_v2_refuses_non_finite_and_leaves_the_output_alone(backend, so):
     with pytest.raises(T.InvalidInput):
         dev.forward(dact, 1, dout)
     assert dout.to_host()[0] == np.float32(19.0)
+    dev.free()
+    dact.free()
+    dout.free()
+
+
+def test_v2_refusals_in_the_lane_per_row_form(backend, so):
+    """Rows of whole scale groups take the form that keeps its terms in a workspace: the same refusals there,
+    and the first row block's finiteness check covers every token."""
+    one16 = 0x3C00
+    fmax = np.float32(np.finfo(np.float32).max)
+    trits = np.zeros((1, 256), np.int8)
+    trits[0, :2] = 1          # row 0: columns 0 and 1
+    trits[0, 128 + 5] = -1    # row 1: column 5
+    t = S.V2Tensor(so, S.D2, 128, 2, 128, [(trits, np.array([[one16, one16]], np.uint16))])
+    dev = backend.salt_v2_upload(S.D2, 128, t.payload, t.scales, t.plane_counts, 2, 128)
+    m = 11
+    act = np.zeros((m, 128), np.float32)
+    act[:, 0], act[:, 1], act[:, 5] = 1.5, 2.25, 4.0
+    dact, dout = backend.to_device(act, "f32"), backend.to_device(np.full(m * 2, 19.0, np.float32), "f32")
+    dev.forward(dact, m, dout)
+    assert (dout.to_host().reshape(m, 2) == np.array([3.75, -4.0], np.float32)).all()
+    for bad_tok, a0, a1 in ((m - 1, fmax, fmax), (3, np.nan, 0.0), (8, 0.0, np.inf)):
+        dout.copy_from(np.full(m * 2, 19.0, np.float32))
+        bad = act.copy()
+        bad[bad_tok, 0], bad[bad_tok, 1] = a0, a1
+        if bad_tok == 8:
+            bad[bad_tok, 100] = a1  # a column under zero trits only: still an input that is not finite
+            bad[bad_tok, 1] = 0.0
+        dact.copy_from(bad)
+        with pytest.raises(T.InvalidInput):
+            dev.forward(dact, m, dout)
+        assert (dout.to_host() == np.float32(19.0)).all()
     dev.free()
     dact.free()
     dout.free()

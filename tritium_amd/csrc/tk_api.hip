@@ -1453,15 +1453,24 @@ extern "C" int tk_salt_v2_forward(tk_ctx *ctx, const tk_salt_v2 *t, const float 
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
   const size_t bytes = m * (size_t)t->dev.n * sizeof(float);
-  TKCHK(ensure(ctx, ctx->tmp, bytes));
+  // the lane-per-row form keeps the terms of up to `chunk` tokens at a time (at most 256 MiB of them)
+  const size_t per_token = tk_salt_v2_term_floats(t->dev) * sizeof(float);
+  size_t chunk = 0;
+  if (per_token && per_token <= ((size_t)256 << 20)) {
+    chunk = ((size_t)256 << 20) / per_token;
+    if (chunk > m) chunk = m;
+  }
+  const size_t out_bytes = (bytes + 255) & ~(size_t)255;
+  TKCHK(ensure(ctx, ctx->tmp, out_bytes + chunk * per_token));
   unsigned flag = 0;
   HIPCHK(hipMemsetAsync(ctx->d_count, 0, sizeof(unsigned), ctx->stream));
-  HIPCHK(tk_launch_salt_v2_forward(ctx->stream, t->dev, act, m, (float *)ctx->tmp.p, ctx->d_count));
+  HIPCHK(tk_launch_salt_v2_forward(ctx->stream, t->dev, act, m, (float *)ctx->tmp.p, ctx->d_count,
+                                   chunk ? (float *)((uint8_t *)ctx->tmp.p + out_bytes) : nullptr, chunk));
+  // the device commits the results only when the flag stayed clear: one synchronization per call
+  HIPCHK(tk_launch_salt_v2_commit(ctx->stream, (const float *)ctx->tmp.p, out, m * (size_t)t->dev.n, ctx->d_count));
   HIPCHK(hipMemcpyAsync(&flag, ctx->d_count, sizeof flag, hipMemcpyDeviceToHost, ctx->stream));
   HIPCHK(hipStreamSynchronize(ctx->stream));
   if (flag) return tk_fail(TK_ERR_INVALID_INPUT, "SALT V2 forward: a non-finite activation or result; the output was not written");
-  HIPCHK(hipMemcpyAsync(out, ctx->tmp.p, bytes, hipMemcpyDeviceToDevice, ctx->stream));
-  HIPCHK(hipStreamSynchronize(ctx->stream));
   return TK_OK;
 }
 

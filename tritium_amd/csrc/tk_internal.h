@@ -197,7 +197,13 @@ struct TkSaltV2 {
 #define TK_SALT_V2_TOKENS 8
 size_t tk_salt_v2_lds_bytes(size_t k, size_t group);
 // tmp receives the [m,n] results; *flag is raised when an activation or a result is not finite
-hipError_t tk_launch_salt_v2_forward(hipStream_t s, const TkSaltV2 &t, const float *act, size_t m, float *tmp, unsigned *flag);
+// terms: workspace of term_tokens * tk_salt_v2_term_floats(t) floats for the lane-per-row form (rows of whole scale
+// groups; tk_salt_v2_term_floats is 0 for other matrices), or null: the form that needs none
+size_t tk_salt_v2_term_floats(const TkSaltV2 &t);
+hipError_t tk_launch_salt_v2_forward(hipStream_t s, const TkSaltV2 &t, const float *act, size_t m, float *tmp, unsigned *flag,
+                                     float *terms, size_t term_tokens);
+// out[i] = tmp[i] for i < count unless *flag is set (then nothing is written)
+hipError_t tk_launch_salt_v2_commit(hipStream_t s, const float *tmp, float *out, size_t count, const unsigned *flag);
 hipError_t tk_launch_salt_v2_gather(hipStream_t s, const TkSaltV2 &t, const uint32_t *rows, size_t count, float *out);
 #ifdef __cplusplus
 }
