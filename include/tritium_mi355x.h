@@ -524,6 +524,10 @@ int tk_set_prep_team_rows(tk_ctx *ctx, int rows);
  * 64-row kernels, 128 = the 128 x 256 kernel, which shares both operands through LDS. Other launches take
  * the 64-row kernels whatever this says. A tuning and test knob: identical bits. */
 int tk_set_gemm_rows(tk_ctx *ctx, int rows);
+/* A grouped launch whose members partly fit LDS runs two kernels (the flow kernel for those that fit, the prefill
+ * kernel for the others). on != 0 (default): side by side on two streams of the context, joined before
+ * anything enqueued later; 0: one after the other. A measurement knob: identical results. */
+int tk_set_group_overlap(tk_ctx *ctx, int on);
 /* K slices of the prefill kernel in single launches: 0 = chosen per launch (a launch with fewer
  * workgroups than CUs is cut into about one workgroup per CU, at least two K blocks per slice), 1 =
  * never split, 2..64 = that many slices where K allows. Integer partial sums, added by the last

@@ -433,8 +433,18 @@ def test_group_with_rows_beyond_lds_takes_the_prefill_kernel(backend, oracle, de
             singles.append((layer, src, out_s))
             hosts.append((packed, scs, act, n))
         grp = backend.group(members, mode, "f32", "f32")
+        # the group's two kernels (flow part, prefill-kernel part) one after the other, then side by side on
+        # two streams (the default), several launches in a row: every launch leaves the same bits
+        backend.set_group_overlap(False)
         grp.launch()
-        grp.launch()
+        in_turn = [out_g.to_host().copy() for _, _, _, out_g in members]
+        backend.set_group_overlap(True)
+        for _ in range(3):
+            for _, _, _, out_g in members:
+                out_g.copy_from(np.full(out_g.count, np.float32(-7.0)))
+            grp.launch()
+            for (_, _, _, out_g), ref in zip(members, in_turn):
+                assert same_bits(out_g.to_host(), ref)
         for (layer, src, _, out_g), (_, _, out_s), (packed, scs, act, n) in zip(members, singles, hosts):
             k = act.shape[1]
             fn(layer, src, m, out_s)

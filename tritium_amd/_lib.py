@@ -139,6 +139,7 @@ SIGNATURES = {
     "tk_set_gemm_tiles": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_ksplit": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_rows": (C.c_int, [vp, C.c_int]),
+    "tk_set_group_overlap": (C.c_int, [vp, C.c_int]),
     "tk_set_stream_min_groups": (C.c_int, [vp, C.c_int]),
     "tk_get_stream_min_groups": (C.c_int, [vp]),
     "tk_set_exact_max_macs": (C.c_int, [vp, sz]),

@@ -581,6 +581,10 @@ class Mi355xBackend:
         """Activation prep: launches of up to `rows` tokens give a token the whole workgroup (default 384)."""
         _check(self._lib.tk_set_prep_team_rows(self._ctx, rows))
 
+    def set_group_overlap(self, on):
+        """Grouped launches of two kernels (flow part + prefill-kernel part): side by side (default) or in turn."""
+        _check(self._lib.tk_set_group_overlap(self._ctx, 1 if on else 0))
+
     def set_gemm_rows(self, rows):
         """0 = automatic, 64 / 128 = rows of the workgroup tile for one-plane int8-contract prefill launches."""
         _check(self._lib.tk_set_gemm_rows(self._ctx, rows))

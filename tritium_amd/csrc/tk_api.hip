@@ -66,6 +66,11 @@ struct DevBuf {
 struct tk_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
+  // A second stream and two events: the two kernels of a grouped launch that has both a flow part and a
+  // prefill-kernel part run side by side (lazily created; default priority like the first)
+  hipStream_t stream2 = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  int group_overlap = 1;   // 1 = run those two kernels side by side, 0 = one after the other
   std::mutex mu;
   tk_device_info info{};
   std::string device_id;
@@ -95,6 +100,9 @@ struct tk_ctx {
 static void ctx_release(tk_ctx *ctx) {
   if (ctx->refs.fetch_sub(1) != 1) return;
   (void)hipSetDevice(ctx->device);
+  if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+  if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
+  if (ctx->stream2) (void)hipStreamDestroy(ctx->stream2);
   (void)hipStreamDestroy(ctx->stream);
   delete ctx;
 }
@@ -337,6 +345,13 @@ extern "C" int tk_set_prep_team_rows(tk_ctx *ctx, int rows) {
   if (rows < 0) return tk_fail(TK_ERR_INVALID_INPUT, "prep_team_rows=%d - use 0 or more", rows);
   std::lock_guard<std::mutex> lk(ctx->mu);
   tk_prep_set_team_rows(rows);
+  return TK_OK;
+}
+
+extern "C" int tk_set_group_overlap(tk_ctx *ctx, int on) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_group_overlap: null context");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->group_overlap = on ? 1 : 0;
   return TK_OK;
 }
 
@@ -2125,10 +2140,30 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
     HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows,
                           g->prep_wave_pieces, g->prep_fast));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
+  // Members whose rows fit LDS take the flow kernel, the others one grouped launch of the prefill kernel. The
+  // two read and write disjoint members and fit a CU together (one eight-wave workgroup with its rows in LDS
+  // beside 49-KiB workgroups of the prefill kernel), so they run side by side on two streams: the second
+  // starts behind everything enqueued so far and the first waits for it at the end.
+  const bool both = do_main && g->has_flow_part && g->variant == DECODE_GEMM && g->cfg.grid > 0;
+  bool forked = false;
+  if (both && ctx->group_overlap) {
+    if (!ctx->stream2) {
+      HIPCHK(hipStreamCreateWithFlags(&ctx->stream2, hipStreamNonBlocking));
+      HIPCHK(hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
+      HIPCHK(hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+    }
+    HIPCHK(hipEventRecord(ctx->ev_fork, ctx->stream));
+    HIPCHK(hipStreamWaitEvent(ctx->stream2, ctx->ev_fork, 0));
+    HIPCHK(tk_launch_gemm(ctx->stream2, nullptr, probs, wg_prob, g->cfg));
+    HIPCHK(hipEventRecord(ctx->ev_join, ctx->stream2));
+    forked = true;
+  }
   if (do_main && g->has_flow_part)
     HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),
                           g->flow_cfg));
-  if (do_main && g->variant == DECODE_GEMM)
+  if (forked)
+    HIPCHK(hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0));
+  else if (do_main && g->variant == DECODE_GEMM)
     HIPCHK(tk_launch_gemm(ctx->stream, nullptr, probs, wg_prob, g->cfg));
   else if (do_main && g->variant == DECODE_FLOW && g->cfg.base3)
     HIPCHK(tk_launch_flow3(ctx->stream, nullptr, probs, wg_prob, g->cfg));
