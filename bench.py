@@ -259,8 +259,9 @@ def bench_config1(T, be, rng, iters=200):
     """configs[0]: one ternary linear, K=2560 N=6912, one plane, f32 N(0,1) activation, batch 1.
     (a) the HBM figure: COPIES distinct resident copies of the layer (0.57 GB of codes, above the 256 MB
         last-level cache) in one grouped launch; kernel alone and the whole step with its digit-split launch;
-    (b) one device-resident call on a single 4.4 MB layer (digit split + decode kernel back to back: cache
-        resident and launch-bound, so a latency figure, not a bandwidth one);
+    (b) one device-resident call on a single 4.4 MB layer (one launch: the decode kernel splits the token's digits
+        itself; beside it the same call as two launches -- cache resident and launch-bound, so latency figures,
+        not bandwidth ones);
     (c) the adapter call on host slices (upload, kernels, download, sync per call)."""
     n, k = 6912, 2560
     trits = [ternary(rng, n, k, 0.4) for _ in range(2)]
@@ -281,6 +282,9 @@ def bench_config1(T, be, rng, iters=200):
     by = COPIES * algorithmic_bytes(1, n, k, 1, 4, 4)
     g.destroy()
     ms_single = time_calls(be, lambda i: be.linear_float(layers[0], acts[0], 1, outs[0]), iters)
+    be.set_fuse_tokens(0)  # the same call as two launches (digit split, then the decode kernel)
+    ms_single_two = time_calls(be, lambda i: be.linear_float(layers[0], acts[0], 1, outs[0]), iters)
+    be.set_fuse_tokens(-1)
     buf = be.upload_weights(packed[0], T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0)
     out = np.zeros(n, np.float32)
     call = T.MpGemm(act_h[0].reshape(-1), buf, scs[0], T.GemmShape(1, n, k), T.TernaryFormat.Tq2_0, out)
@@ -302,6 +306,7 @@ def bench_config1(T, be, rng, iters=200):
             "step_GB/s_incl_digit_split": round(by / ms_step / 1e6, 1),
             "step_frac_of_hbm_peak": round(by / ms_step / 1e6 / HBM_PEAK_GBS, 4),
             "single_layer_device_resident_call_us": round(ms_single * 1e3, 2),
+            "single_layer_call_as_two_launches_us": round(ms_single_two * 1e3, 2),
             "single_layer_GB/s": round(by1 / ms_single / 1e6, 1),
             "adapter_call_on_host_slices_us": round(host_us, 1),
             "verified": verified}

@@ -519,6 +519,16 @@ int tk_set_gemm_two_by_two(tk_ctx *ctx, int on);
  * workgroup instead of one wave (few tokens: the launch lasts as long as one token's chain of instructions).
  * Default 384 (the digit split of the float contract: 8/3 of it). Process-wide; identical bits either way. A tuning and test knob. */
 int tk_set_prep_team_rows(tk_ctx *ctx, int rows);
+/* Single decode calls (tk_linear_a8, tk_linear_float and their variants without RMSNorm) of up to `tokens`
+ * tokens run as ONE launch: the decode kernel quantizes (or digit-splits) the tokens itself, every workgroup for
+ * itself, instead of a prep launch in front of it -- where the rows fit (K a multiple of 256 up to 8192, 16-byte
+ * aligned f32 or bf16 rows, operand rows within 62 KiB of LDS; 48 KiB in the K-split kernel of narrow launches).
+ * Every workgroup repeats the tokens' quantization, so the form pays for very few tokens: -1 (default) = one token,
+ * or two under the int8 contract in the K-split kernel; 0 = never; 1..4 = up to that many. Identical bits either way.
+ * A tuning and test knob. */
+int tk_set_fuse_tokens(tk_ctx *ctx, int tokens);
+/* Calls of this context so far that ran in that single-launch form (for tests of the dispatch). */
+int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count);
 /* Row count of the workgroup tile for single launches of one plane under the int8 contract (f32 or bf16
  * rows of whole 16-byte pieces at a 16-byte aligned address, no residual): 0 = chosen per launch, 64 = the
  * 64-row kernels, 128 = the 128 x 256 kernel, which shares both operands through LDS. Other launches take

@@ -1,0 +1,215 @@
+"""Single decode calls of one to four tokens run as ONE launch: the decode kernel (the K-split kernel of narrow
+launches and the flow kernel of wide ones) quantizes (W1.58A8) or digit-splits (float contract) the tokens itself.
+The launch must carry the bits of the two-launch form (same arithmetic, statement for statement) -- and under the
+int8 contract the CPU oracle's -- for every plane count, element type, ring size and runs-per-wave form, for rows that are all zero, hold one element, NaN, Inf or a range the digit
+grid does not carry (those take the exact fallback inside the kernel), and with a residual. Shapes the form does
+not take (K beyond 8192 or not whole blocks, more than four tokens, unaligned rows, RMSNorm in front) must fall
+through to the two launches. Reference behaviour for the special rows: crates/tritium-spec/src/lib.rs:351-378,
+crates/tritium-core/src/reference.rs:42-51."""
+import numpy as np
+import pytest
+
+import tritium_amd as T
+from helpers import accepts, bf16_bits_to_f32, f32_to_bf16_bits, same_bits, scales, ternary
+from oracle_lib import FMT_TQ2_0
+
+pytestmark = pytest.mark.gpu
+
+KSPLIT, FLOW = 1, 3
+
+
+@pytest.fixture(autouse=True, params=[KSPLIT, FLOW], ids=["ksplit", "flow"])
+def kernel(request, backend):
+    backend.set_decode_kernel(request.param)
+    backend.set_fuse_tokens(4)
+    yield request.param
+    backend.set_decode_kernel(0)
+    backend.set_fuse_tokens(-1)
+    backend.set_flow_ring(0)
+
+
+def _takes_one_launch(kernel, float_contract, m, k, planes):
+    """The library's rule: whole K blocks up to 8192, and the operand rows (256 bytes per K block and row; four rows
+    per token under the float contract) within 62 KiB of LDS for the flow kernel, within the 48 KiB that the
+    K-split kernel stages in one pass."""
+    nb, rows = k // 256, (4 * m if float_contract else m)
+    if k % 256 or nb * 16 > 512 or m > 4:
+        return False
+    if kernel == FLOW:
+        return nb * 256 * rows + 2048 <= 65536
+    return nb * 256 * rows <= 48 * 1024
+
+
+def _planes(rng, n, k, planes):
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)[:planes]]
+    scs = [scales(rng, n) for _ in range(planes)]
+    return ws, scs, [T.pack_rows(w, n, k) for w in ws]
+
+
+def _tokens(rng, m, k, special):
+    a = (rng.standard_normal((m, k)) * 10.0 ** rng.integers(-2, 3)).astype(np.float32)
+    if special == "zero":
+        a[0] = 0.0
+    elif special == "single":
+        a[m - 1] = 0.0
+        a[m - 1, k // 3] = -3.25
+    elif special == "nan":
+        a[0, 5] = np.nan
+    elif special == "inf":
+        a[m - 1, k - 1] = -np.inf
+    elif special == "narrow":  # one element 2^30 times the rest: the digit grid does not carry the small ones
+        a[0] = (rng.standard_normal(k) * 1e-3).astype(np.float32)
+        a[0, 7] = np.float32(2.0 ** 20)
+    return a
+
+
+def _same(a, b):
+    fin = ~np.isnan(a)
+    return (np.isnan(b) == ~fin).all() and same_bits(a[fin], b[fin])
+
+
+@pytest.mark.parametrize("special", ["plain", "zero", "single", "nan", "inf", "narrow"])
+@pytest.mark.parametrize("m,n,k,planes", [(1, 48, 256, 1), (1, 6912, 2560, 1), (2, 200, 2048, 2), (3, 130, 5120, 3),
+                                            (4, 64, 3840, 1), (4, 96, 1024, 2), (1, 40, 8192, 2), (2, 33, 6912, 1)])
+def test_one_launch_equals_two_launches(backend, oracle, kernel, m, n, k, planes, special):
+    print("case fused-decode", kernel, m, n, k, planes, special, flush=True)
+    rng = np.random.default_rng(m * 1000 + n + k + planes + len(special))
+    ws, scs, packed = _planes(rng, n, k, planes)
+    layer = backend.linear(packed, scs, n, k)
+    act = _tokens(rng, m, k, special)
+    for dt in ("f32", "bf16"):
+        host = f32_to_bf16_bits(act) if dt == "bf16" else act
+        seen = bf16_bits_to_f32(host).reshape(m, k) if dt == "bf16" else act
+        dact = backend.to_device(host, dt)
+        for odt in ("f32", "bf16"):
+            out = backend.empty(m * n, odt)
+            for call, name in ((backend.linear_a8, "a8"), (backend.linear_float, "float")):
+                got = {}
+                for fuse in (4, 0):
+                    backend.set_fuse_tokens(fuse)
+                    before = backend.fused_calls()
+                    call(layer, dact, m, out)
+                    got[fuse] = out.to_host().copy()
+                    one = fuse and _takes_one_launch(kernel, name == "float", m, k, planes)
+                    assert backend.fused_calls() - before == (1 if one else 0), (name, dt, odt, fuse)
+                if odt == "bf16":
+                    assert (got[4] == got[0]).all() or _same(bf16_bits_to_f32(got[4]), bf16_bits_to_f32(got[0]))
+                else:
+                    assert _same(got[4], got[0]), (name, dt, odt)
+                if odt == "f32" and name == "a8":
+                    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, seen, m, n, k)
+                    assert _same(want.reshape(-1), got[4].reshape(-1))
+                if odt == "f32" and name == "float":
+                    want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, seen, m, n, k).reshape(-1)
+                    fin = np.isfinite(want)
+                    top = max(float(np.abs(want[fin]).max()) if fin.any() else 0.0, 1e-30)
+                    assert accepts(got[4].reshape(-1)[fin], want[fin], rel=1e-4, floor=top).all()
+            out.free()
+        dact.free()
+    layer.free()
+
+
+@pytest.mark.parametrize("ring", [2, 3, 4, 5])
+@pytest.mark.parametrize("m,planes", [(1, 1), (2, 1), (1, 2), (3, 3)])
+def test_every_ring_size_and_run_count(backend, oracle, kernel, ring, m, planes):
+    """The ring of loads (2..5 positions) and one or two runs per wave are separate instantiations of the flow kernel."""
+    if kernel != FLOW:
+        pytest.skip("the ring belongs to the flow kernel")
+    print("case fused-decode ring", ring, m, planes, flush=True)
+    rng = np.random.default_rng(ring * 10 + m + planes)
+    n, k = 272, 2560
+    ws, scs, packed = _planes(rng, n, k, planes)
+    layer = backend.linear(packed, scs, n, k)
+    backend.set_flow_ring(ring)
+    act = _tokens(rng, m, k, "plain")
+    dact = backend.to_device(act, "f32")
+    out = backend.empty(m * n, "f32")
+    before = backend.fused_calls()
+    backend.linear_a8(layer, dact, m, out)
+    assert backend.fused_calls() == before + 1
+    assert same_bits(out.to_host(), oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+    backend.linear_float(layer, dact, m, out)
+    got = out.to_host().copy()
+    backend.set_fuse_tokens(0)
+    backend.linear_float(layer, dact, m, out)
+    assert same_bits(got, out.to_host())
+    for x in (dact, out):
+        x.free()
+    layer.free()
+
+
+def test_residual_rides_along(backend, oracle):
+    rng = np.random.default_rng(77)
+    m, n, k = 2, 160, 2048
+    ws, scs, packed = _planes(rng, n, k, 2)
+    layer = backend.linear(packed, scs, n, k)
+    act = _tokens(rng, m, k, "plain")
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    dact, dres, out = backend.to_device(act, "f32"), backend.to_device(res, "f32"), backend.empty(m * n, "f32")
+    before = backend.fused_calls()
+    backend.linear_a8_residual(layer, dact, m, dres, out)
+    assert backend.fused_calls() == before + 1
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k).reshape(m, n) + res
+    assert same_bits(out.to_host().reshape(m, n), want.astype(np.float32))
+    for x in (dact, dres, out):
+        x.free()
+    layer.free()
+
+
+@pytest.mark.parametrize("m,k,why", [(5, 2048, "tokens"), (1, 8448, "K beyond two pieces per thread"),
+                                      (1, 2000, "K not whole blocks"), (4, 4096, "rows beyond 63 KiB of LDS (float contract)")])
+def test_other_shapes_take_two_launches(backend, oracle, kernel, m, k, why):
+    print("case fused-decode fallthrough", kernel, m, k, why, flush=True)
+    rng = np.random.default_rng(m + k)
+    n = 80
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    act = _tokens(rng, m, k, "plain")
+    dact, out = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+    before = backend.fused_calls()
+    backend.linear_float(layer, dact, m, out)
+    assert backend.fused_calls() == before, why
+    want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k).reshape(-1)
+    assert accepts(out.to_host(), want, rel=1e-4, floor=float(np.abs(want).max())).all()
+    backend.linear_a8(layer, dact, m, out)
+    assert same_bits(out.to_host(), oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+    for x in (dact, out):
+        x.free()
+    layer.free()
+
+
+def test_automatic_dispatch_takes_one_launch_for_one_token(backend, oracle):
+    """Left to itself (no kernel forced, the knob on automatic) a one-token call on a layer of configs[0]'s shape is a
+    single launch under both contracts; two tokens under the int8 contract only; four under neither."""
+    backend.set_decode_kernel(0)
+    backend.set_fuse_tokens(-1)
+    rng = np.random.default_rng(5)
+    n, k = 6912, 2560
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    act = _tokens(rng, 1, k, "plain")
+    dact, out = backend.to_device(act, "f32"), backend.empty(n, "f32")
+    before = backend.fused_calls()
+    backend.linear_a8(layer, dact, 1, out)
+    backend.linear_float(layer, dact, 1, out)
+    assert backend.fused_calls() == before + 2
+    for x in (dact, out):
+        x.free()
+    for m, expect in ((2, 1), (4, 0)):
+        act = _tokens(rng, m, k, "plain")
+        dact, out = backend.to_device(act, "f32"), backend.empty(m * n, "f32")
+        before = backend.fused_calls()
+        backend.linear_a8(layer, dact, m, out)
+        assert same_bits(out.to_host(), oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+        backend.linear_float(layer, dact, m, out)
+        assert backend.fused_calls() == before + expect, m
+        for x in (dact, out):
+            x.free()
+    layer.free()
+
+
+def test_knob_rejects_other_values(backend):
+    with pytest.raises(T.BackendError):
+        backend.set_fuse_tokens(5)
+    with pytest.raises(T.BackendError):
+        backend.set_fuse_tokens(-2)

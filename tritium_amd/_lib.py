@@ -139,6 +139,8 @@ SIGNATURES = {
     "tk_set_gemm_tiles": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_ksplit": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_rows": (C.c_int, [vp, C.c_int]),
+    "tk_set_fuse_tokens": (C.c_int, [vp, C.c_int]),
+    "tk_get_fused_calls": (C.c_int, [vp, C.POINTER(C.c_ulonglong)]),
     "tk_set_group_overlap": (C.c_int, [vp, C.c_int]),
     "tk_set_stream_min_groups": (C.c_int, [vp, C.c_int]),
     "tk_get_stream_min_groups": (C.c_int, [vp]),

@@ -585,6 +585,17 @@ class Mi355xBackend:
         """Grouped launches of two kernels (flow part + prefill-kernel part): side by side (default) or in turn."""
         _check(self._lib.tk_set_group_overlap(self._ctx, 1 if on else 0))
 
+    def set_fuse_tokens(self, tokens):
+        """Single decode calls of up to `tokens` tokens (1..4) build their operand rows inside the decode kernel: one
+        launch instead of two. 0 = always the separate prep launch, -1 (default) = chosen per call."""
+        _check(self._lib.tk_set_fuse_tokens(self._ctx, tokens))
+
+    def fused_calls(self):
+        """Calls so far that ran as one launch (the decode kernel built the operand rows itself)."""
+        c = C.c_ulonglong(0)
+        _check(self._lib.tk_get_fused_calls(self._ctx, C.byref(c)))
+        return int(c.value)
+
     def set_gemm_rows(self, rows):
         """0 = automatic, 64 / 128 = rows of the workgroup tile for one-plane int8-contract prefill launches."""
         _check(self._lib.tk_set_gemm_rows(self._ctx, rows))

@@ -84,6 +84,8 @@ struct tk_ctx {
   int gemm_tiles = 0;      // 0 = automatic, 2 / 4 = tiles per wave of the one-plane prefill kernel
   int gemm_two_by_two = 0;  // one-plane prefill kernel, 64 x 128 form: 0 = four waves side by side, 1 = two by two
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
+  unsigned long long fused_calls = 0;  // calls that ran as one launch (tk_get_fused_calls)
+  int fuse_tokens = -1;    // single decode calls of up to this many tokens build their operand rows inside the decode kernel (-1 = chosen per call, 0 = never)
   int gemm_rows = 0;       // one-plane int8-contract prefill, single launches: 0 = tile rows chosen per launch, 64 / 128 = force
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
   int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
@@ -352,6 +354,21 @@ extern "C" int tk_set_group_overlap(tk_ctx *ctx, int on) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_group_overlap: null context");
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->group_overlap = on ? 1 : 0;
+  return TK_OK;
+}
+
+extern "C" int tk_set_fuse_tokens(tk_ctx *ctx, int tokens) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_fuse_tokens: null context");
+  if (tokens < -1 || tokens > 4) return tk_fail(TK_ERR_INVALID_INPUT, "fuse_tokens=%d - use -1 (automatic), 0 (never) or 1..4", tokens);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->fuse_tokens = tokens;
+  return TK_OK;
+}
+
+extern "C" int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count) {
+  if (!ctx || !count) return tk_fail(TK_ERR_INVALID_INPUT, "tk_get_fused_calls: null argument");
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  *count = ctx->fused_calls;
   return TK_OK;
 }
 
@@ -1000,6 +1017,25 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
       plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units, ctx->gemm_tiles);
     }
   }
+  // A single decode call of few tokens is two short dependent launches, and the gap between them costs more than
+  // either: the flow kernel then builds the operand rows itself, every workgroup for itself (256 threads, at most
+  // two 16-byte pieces of a token per thread, straight-line loads: whole K blocks, aligned f32 or bf16 rows).
+  // Every workgroup repeats the tokens' arithmetic (about 25 instructions per element under the float contract),
+  // which the prep launch does once, so the form pays for very few tokens. Measured, back-to-back calls, two
+  // launches -> one: K=2560 N=6912 one plane f32, int8 contract 1 / 2 / 4 tokens 8.4 -> 5.3 / 9.0 -> 7.1 /
+  // 10.0 -> 10.8 us, float contract 9.5 -> 6.4 / 10.0 -> 10.0 / 11.4 -> 16.3 us; K=2048 N=8192 two planes bf16
+  // 9.0 -> 5.6 and 9.7 -> 6.7 us for one token; K=6912 N=2560 10.3 -> 6.8 and 12.7 -> 8.2; the flow kernel on
+  // K=5120 N=17408 three planes 20.4 -> 17.7 and 22.1 -> 19.1 for one token, nothing for two. Left to itself: one
+  // token, or two under the int8 contract in the K-split kernel.
+  const int fuse_limit = ctx->fuse_tokens >= 0 ? ctx->fuse_tokens : ((prep_kind == TK_PREP_A8 && variant == DECODE_KSPLIT) ? 2 : 1);
+  // Both decode kernels of single launches have the form: the K-split kernel (its rows fit LDS in one pass) and the
+  // flow kernel in its 16x16x64 form.
+  const bool fuse_rows = pl.skinny && !norm && pl.cfg.rt == 1 && (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) &&
+                         m <= (size_t)fuse_limit && nb * 16 <= 512 && k % 256 == 0 && ((uintptr_t)act & 15) == 0 &&
+                         (act_dtype == TK_F32 || act_dtype == TK_BF16);
+  const bool fused_flow = fuse_rows && variant == DECODE_FLOW && !wide && !b3 && flow_lds + 2048 <= 64 * 1024;
+  const bool fused_ksplit = fuse_rows && variant == DECODE_KSPLIT && (size_t)pl.pr.kc >= nb && pl.cfg.lds_bytes + 2048 <= 64 * 1024;
+  const bool fused = fused_flow || fused_ksplit;
   Workspace ws;
   TKCHK(take_workspace(ctx, static_ws, (size_t)pl.pr.rs * nb * 256, R, m, norm ? m * k * 4 : 0, &ws));
 
@@ -1023,7 +1059,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   pp.rs = (size_t)pl.pr.rs;
   pp.act_dtype = act_dtype;
   pp.m = (int)m;
-  HIPCHK(tk_launch_prep(ctx->stream, prep_kind, &pp, nullptr, 0, 0, (unsigned)m));
+  if (!fused) HIPCHK(tk_launch_prep(ctx->stream, prep_kind, &pp, nullptr, 0, 0, (unsigned)m));
 
   TkProblem &pr = pl.pr;
   pr.ap = pp.ap;
@@ -1052,8 +1088,14 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R));
     size_t ztiles = pr.zskip && !wide && !b3 ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0;
     if (ztiles && flow_lds + (size_t)cfg.planes * tk_flow_zmap_words(ztiles, nb) * 4 > kLdsFlowMax) ztiles = 0;
+    if (fused) ztiles = 0;      // the row constants take the maps' place behind the rows
     if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or another form of the kernel): plain loads
     flow_cfg_form(&cfg, wide, b3, flow_lds, R, ztiles, nb);
+    if (fused) {
+      cfg.fused = 1;
+      cfg.lds_bytes += 1024;
+      ctx->fused_calls++;
+    }
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
     if (b3) HIPCHK(tk_launch_flow3(ctx->stream, &pr, nullptr, nullptr, cfg));
@@ -1066,6 +1108,11 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     pr.group_begin = 0;
     HIPCHK(tk_launch_stream(ctx->stream, &pr, nullptr, nullptr, cfg));
   } else if (pl.skinny) {
+    if (fused) {
+      pl.cfg.fused = 1;
+      pl.cfg.lds_bytes += 1024;
+      ctx->fused_calls++;
+    }
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
   } else {
     // One plane under the int8 contract with whole 16-byte output pieces: the 128 x 256 kernel moves a third

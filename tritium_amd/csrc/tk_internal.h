@@ -119,6 +119,7 @@ struct TkLaunchCfg {
   int gemm_two_by_two;  // ... the 64 x 128 form with its waves two by two (32 rows x 4 tiles each) instead of side by side
   int tw;       // flow kernel, 16x16x64 form: runs per wave (tk_flow_runs_per_wave)
   int base3;    // flow kernel: stream the planes' base-3 copies (tk_launch_flow3)
+  int fused;    // flow kernel, one row tile, one problem: build the operand rows in the kernel (no prep launch)
 };
 
 #ifdef __cplusplus

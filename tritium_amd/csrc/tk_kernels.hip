@@ -29,13 +29,20 @@
 // lane, expands, and issues MFMAs against A operands held in LDS.
 // ------------------------------------------------------------------------------------------
 
-template <int P, int RT>
+// FUSED (one row tile, a single problem whose operand rows fit LDS in one pass): the kernel builds the operand rows
+// of its one to four tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of
+// two; the row constants sit in LDS behind the rows (and behind the reduction's buffer).
+__device__ __forceinline__ void fused_stage_rows(const TkProblem &pr, uint4 *rows, uint8_t *cst);
+__device__ __forceinline__ RowConst row_const_from_lds(const uint8_t *cst, int mode, int R, int M, int rowbase);
+__device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int rowbase, unsigned flag, const uint8_t *cst);
+template <int P, int RT, bool FUSED = false>
 __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, const TkProblem *__restrict__ table,
                                                           int nprobs) {
+  static_assert(!FUSED || RT == 1, "the fused form: one row tile");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tile = blockIdx.x;
   const TkProblem *prp = &single;
-  if (table) {
+  if (!FUSED && table) {
     int lo = 0, hi = nprobs - 1;  // last problem with tile_begin <= tile
     while (lo < hi) {
       int mid = (lo + hi + 1) >> 1;
@@ -58,13 +65,19 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
   const uint4 *ap4 = (const uint4 *)pr.ap;
   uint4 *lds4 = (uint4 *)smem;
 
+  const size_t rows_bytes = (size_t)nb * 256 * R, red_bytes = (size_t)4 * P * RT * 1024;
+  uint8_t *const cst = smem + (rows_bytes > red_bytes ? rows_bytes : red_bytes);  // fused form only
   for (int kb0 = 0; kb0 < nb; kb0 += kc) {
     const int kcn = min(kc, nb - kb0);
-    __syncthreads();
-    const int cnt = kcn * 16 * R;  // 16-byte pieces in this K chunk
-    const uint4 *src = ap4 + (size_t)kb0 * 16 * R;
-    for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4[idx] = src[idx];
-    __syncthreads();
+    if constexpr (FUSED) {  // (kc >= nb: one pass)
+      fused_stage_rows(pr, lds4, cst);
+    } else {
+      __syncthreads();
+      const int cnt = kcn * 16 * R;  // 16-byte pieces in this K chunk
+      const uint4 *src = ap4 + (size_t)kb0 * 16 * R;
+      for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4[idx] = src[idx];
+      __syncthreads();
+    }
 
     for (int kbl = wave; kbl < kcn; kbl += 4) {
       uint4 w[P];
@@ -103,6 +116,24 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
   __syncthreads();
 
   const int n = t * 16 + i;
+  if constexpr (FUSED) {
+    if (wave == 0 && n < pr.n) {
+      const int rowbase = 4 * g;
+      v4i sum[P];
+      float sc[P];
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        sum[p] = red[(0 * P + p) * 64 + lane];
+#pragma unroll
+        for (int w2 = 1; w2 < 4; ++w2) sum[p] += red[(w2 * P + p) * 64 + lane];
+        sc[p] = pr.scales[p][n];
+      }
+      const RowConst rc = row_const_from_lds(cst, pr.mode, R, pr.M, rowbase);
+      flow_epilogue<P>(pr, n, rowbase, sum, sc, rc);
+      if (rc.flag) exact_rows_fused(pr, n, rowbase, rc.flag, cst);
+    }
+    return;
+  }
   for (int rt = wave; rt < RT; rt += 4) {
     const int rowbase = rt * 16 + 4 * g;
     float out[4] = {0.f, 0.f, 0.f, 0.f};
@@ -251,9 +282,12 @@ __global__ __launch_bounds__(TK_WG) void tk_stream_kernel(TkProblem single, cons
 // three (168 registers) -- left alone it takes 169, which costs a third of the waves in flight and 8% of
 // the rate at 9..16 operand rows.
 #define TK_FLOW_MIN_WAVES(P, RT, TW, DR) (((P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
-template <int P, int RT, int TW, int DR, bool TABLE>
+// FUSED (one row tile, a single problem, 256 threads): the kernel builds the operand rows of its one to four
+// tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of two.
+template <int P, int RT, int TW, int DR, bool TABLE, bool FUSED = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                       const int *__restrict__ wg_prob) {
+  static_assert(!FUSED || (RT == 1 && !TABLE), "the fused form: one row tile, one problem");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : *single_problem();
   const int NW = (int)(blockDim.x >> 6);  // 4 or 8 waves
@@ -304,7 +338,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
   // issued before that staging and read their map words from memory (with runs of one tile they are
   // three of a tile's eight chunks: left unmapped, a plane with 75% zero chunks fetched 23% less instead
   // of 37%).
-  const bool zskip = pr.zskip != 0;
+  const bool zskip = !FUSED && pr.zskip != 0;  // (the fused form keeps its row constants where the maps would go)
   const uint32_t *lds_z = (const uint32_t *)(smem + (size_t)nb * 256 * R);
   const unsigned zero_off = (unsigned)n_tiles * (unsigned)nb * 1024u + (unsigned)lane * 16u;
   const unsigned wg_first = (unsigned)(blockIdx.x - pr.group_begin) * (unsigned)(NW * TW * S);
@@ -341,7 +375,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
   for (int d = 0; d < D; ++d) request(d, d < nb, d == 0, false);  // (the map is not staged yet: read from memory)
 
   // stage every operand row of the problem in LDS
-  {
+  uint8_t *const cst = smem + (size_t)nb * 256 * R;  // fused form: the row constants behind the rows
+  if constexpr (FUSED) {
+    fused_stage_rows(pr, (uint4 *)smem, cst);
+  } else {
     const uint4 *ap4 = (const uint4 *)pr.ap;
     uint4 *lds4w = (uint4 *)smem;
     const int cnt = nb * 16 * R;
@@ -358,10 +395,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
   unsigned any_flag = 0;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    rc[rt] = load_row_const(hot, rt * 16 + 4 * g);
+    if constexpr (FUSED) rc[rt] = row_const_from_lds(cst, hot.mode, R, hot.M, rt * 16 + 4 * g);  // (staged behind a barrier)
+    else rc[rt] = load_row_const(hot, rt * 16 + 4 * g);
     any_flag |= rc[rt].flag;
   }
-  __syncthreads();
+  if constexpr (!FUSED) __syncthreads();
   const uint4 *lds4 = (const uint4 *)smem;
   // operand rows past R re-read the last row: their results are never stored
   int arow[RT];
@@ -439,8 +477,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
         if (t >= pr.n_tiles || n >= pr.n) continue;
         for (int rt = 0; rt < RT; ++rt) {
           const int rowbase = rt * 16 + 4 * g;
-          const unsigned fl = row_flags(pr, rowbase);
-          if (fl) exact_rows(pr, n, rowbase, fl);
+          if constexpr (FUSED) {
+            if (rc[rt].flag) exact_rows_fused(pr, n, rowbase, rc[rt].flag, cst);
+          } else {
+            const unsigned fl = row_flags(pr, rowbase);
+            if (fl) exact_rows(pr, n, rowbase, fl);
+          }
         }
       }
     }
@@ -2630,6 +2672,163 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Decode in one launch: the flow kernel builds the operand rows of its one to four tokens itself. Every workgroup
+// repeats the prep kernels' work for all tokens -- a few elements per thread -- in place of a second launch in
+// front of every call, which costs more than the kernel itself on a single layer. The arithmetic is that of
+// tk_prep_a8_wave_kernel / tk_prep_digits_wave_kernel in their straight-line form with the workgroup as the team
+// (whole K blocks, 16-byte aligned rows of f32 or bf16, at most two pieces per thread of the 256), statement for
+// statement, so rows, row sums, scales, exponents and flags carry the same bits. They go to LDS: the rows in
+// operand order at `rows`, the constants at `cst` (int rowsum[64] | float scale or int exponent [64] |
+// uint flag[64] | float 127/gamma [64]).
+// ------------------------------------------------------------------------------------------
+// The tokens are taken one after the other (a version with the loads and reductions of four tokens at once was
+// slower for one token and no faster for four: the kernel's code grows fourfold, and what a token costs is its
+// arithmetic, about 25 instructions per element under the float contract, repeated by every workgroup).
+#define TK_FUSED_HELD 2
+template <int FAST>
+__device__ __forceinline__ void fused_token_a8(const void *act, int tok, size_t k, size_t nb, size_t R, uint4 *rows,
+                                               uint8_t *cst, float *shf, int *shi) {
+  const int lane = threadIdx.x;
+  const size_t npieces = nb * 16, base = (size_t)tok * k;
+  float held[TK_FUSED_HELD][16];
+  float gamma;
+  int nonfinite;
+  wave_absmax_held<TK_FUSED_HELD, FAST, 256>(act, 0, base, k, npieces, true, lane, held, gamma, nonfinite, shf, shi);
+  const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
+  const bool live = gamma != 0.0f && !nonfinite;
+  const float sl_ = live ? s : 0.0f;
+  int sum = 0;
+#pragma unroll
+  for (int it = 0; it < TK_FUSED_HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 256;
+    if (pc >= npieces) continue;
+    uint4 piece;
+    uint32_t *pw = (uint32_t *)&piece;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      uint32_t packed = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        float x = held[it][sl * 4 + b];
+        if (!live) x = 0.0f;  // (a NaN or Inf times zero would not be zero)
+        float r = rintf(__fmul_rn(x, sl_));  // one multiply, ties to even
+        r = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+        const int q = (int)r;
+        sum += q;
+        packed |= ((uint32_t)q & 0xFFu) << (8 * b);
+      }
+      pw[sl] = packed;
+    }
+    rows[piece_offset(pc >> 4, (int)(pc & 15), R, (size_t)tok) >> 4] = piece;
+  }
+  sum = block_sum(sum, shi);
+  if (lane == 0) {
+    ((int *)cst)[tok] = sum;
+    ((float *)(cst + 256))[tok] = gamma == 0.0f ? 0.0f : __fdiv_rn(gamma, 127.0f);
+    ((uint32_t *)(cst + 512))[tok] = nonfinite ? 1u : 0u;
+    ((float *)(cst + 768))[tok] = s;
+  }
+}
+
+template <int FAST>
+__device__ __forceinline__ void fused_token_digits(const void *act, int tok, size_t k, size_t nb, size_t R, uint4 *rows,
+                                                   uint8_t *cst, float *shf, int *shi) {
+  const int lane = threadIdx.x;
+  const size_t npieces = nb * 16, base = (size_t)tok * k;
+  float held[TK_FUSED_HELD][16];
+  float gamma;
+  int nonfinite;
+  wave_absmax_held<TK_FUSED_HELD, FAST, 256>(act, 0, base, k, npieces, true, lane, held, gamma, nonfinite, shf, shi);
+  int E = 0;
+  if (gamma != 0.0f && !nonfinite) (void)frexpf(gamma, &E);
+  const int shift = 30 - E;
+  const bool live = gamma != 0.0f && !nonfinite;
+  int five[5] = {0, 0, 0, 0, 0};  // four digit-row sums, poor elements
+#pragma unroll
+  for (int it = 0; it < TK_FUSED_HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 256;
+    if (pc >= npieces) continue;
+    uint4 piece[4];
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const float r = ldexpf(live ? held[it][sl * 4 + b] : 0.0f, shift);
+        int q = __float2int_rn(r);  // |q| <= 2^30
+        five[4] += digit_poor(r, q) ? 1 : 0;
+#pragma unroll
+        for (int dg = 0; dg < 4; ++dg) {
+          int dv = dg == 3 ? q : (((q + 128) & 0xFF) - 128);  // balanced digit in [-128,127]
+          q = (q - dv) >> 8;
+          five[dg] += dv;
+          packed[dg] |= ((uint32_t)dv & 0xFFu) << (8 * b);
+        }
+      }
+#pragma unroll
+      for (int dg = 0; dg < 4; ++dg) ((uint32_t *)&piece[dg])[sl] = packed[dg];
+    }
+#pragma unroll
+    for (int dg = 0; dg < 4; ++dg) rows[piece_offset(pc >> 4, (int)(pc & 15), R, (size_t)tok * 4 + dg) >> 4] = piece[dg];
+  }
+  block_sums<5>(five, shi);
+  bool narrow = false;
+  if (five[4] > 0) {  // uniform over the workgroup
+    int bands[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int it = 0; it < TK_FUSED_HELD; ++it) {
+      const size_t pc = (size_t)lane + (size_t)it * 256;
+      if (pc < npieces) count_bands(held[it], shift, bands);
+    }
+    block_sums<8>(bands, shi);
+    narrow = digits_narrow(five[4], bands);
+  }
+  if (lane < 4) ((int *)cst)[tok * 4 + lane] = lane == 0 ? five[0] : lane == 1 ? five[1] : lane == 2 ? five[2] : five[3];
+  if (lane == 0) {
+    ((int *)(cst + 256))[tok] = -shift;
+    ((uint32_t *)(cst + 512))[tok] = (nonfinite || narrow) ? 1u : 0u;
+  }
+}
+
+__device__ __forceinline__ void fused_stage_rows(const TkProblem &pr, uint4 *rows, uint8_t *cst) {
+  __shared__ float shf[4];
+  __shared__ int shi[32];
+  const int M = pr.M;
+  const size_t k = (size_t)pr.k, nb = (size_t)pr.nb, R = (size_t)pr.R;
+  const void *act = pr.raw_act;
+  const bool bf16 = pr.raw_dtype == TK_BF16;
+  for (int tok = 0; tok < M; ++tok) {
+    if (pr.mode == TK_MODE_INT8) {
+      if (bf16) fused_token_a8<2>(act, tok, k, nb, R, rows, cst, shf, shi);
+      else fused_token_a8<1>(act, tok, k, nb, R, rows, cst, shf, shi);
+    } else {
+      if (bf16) fused_token_digits<2>(act, tok, k, nb, R, rows, cst, shf, shi);
+      else fused_token_digits<1>(act, tok, k, nb, R, rows, cst, shf, shi);
+    }
+  }
+  __syncthreads();
+}
+
+// exact_rows() with the per-token constants of the fused form (in LDS, not in the problem's arrays)
+__device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int rowbase, unsigned flag, const uint8_t *cst) {
+  if (pr.out_dtype == TK_I32) return;
+  const bool a8 = pr.mode == TK_MODE_INT8;
+  for (int r = 0; r < (a8 ? 4 : 1); ++r) {
+    const int m = a8 ? rowbase + r : rowbase >> 2;  // the token
+    if (m >= pr.M || !(flag & (1u << r))) continue;
+    const float as = a8 ? ((const float *)(cst + 256))[m] : 1.0f;
+    const float s = a8 ? ((const float *)(cst + 768))[m] : 0.0f;
+    float f = 0.0f;
+    for (int p = 0; p < pr.planes; ++p) {
+      float t = __fmul_rn(seq_dot_raw(pr.codes[p], pr.nb, pr.k, pr.raw_act, pr.raw_dtype, n, m, a8 ? 1 : 0, s, a8 && as == 0.0f), pr.scales[p][n]);
+      f = p == 0 ? t : __fadd_rn(f, t);
+    }
+    if (a8) f = __fmul_rn(f, as);
+    store_out(pr.out, pr.out_dtype, (size_t)m * pr.n + n, with_residual(pr.residual, pr.out_dtype, (size_t)m * pr.n + n, f));
+  }
+}
+
 // Already-quantized int8 rows -> operand order + row sums.
 __global__ __launch_bounds__(TK_WG) void tk_prep_i8_kernel(TkPrep single, const TkPrep *__restrict__ table,
                                                            int nprep, int uniform_m) {
@@ -2805,6 +3004,11 @@ static hipError_t launch_skinny_p(hipStream_t s, const TkProblem *single, const 
   TkProblem dummy = {};
   const TkProblem &sg = single ? *single : dummy;
   dim3 grid(cfg.grid), block(TK_WG);
+  if (cfg.fused) {  // the operand rows are built inside the kernel: one problem, one row tile
+    if (table || cfg.rt != 1) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((tk_skinny_kernel<P, 1, true>), grid, block, cfg.lds_bytes, s, sg, table, nprobs);
+    return hipGetLastError();
+  }
   switch (cfg.rt) {
     case 1: hipLaunchKernelGGL((tk_skinny_kernel<P, 1>), grid, block, cfg.lds_bytes, s, sg, table, nprobs); break;
     case 2: hipLaunchKernelGGL((tk_skinny_kernel<P, 2>), grid, block, cfg.lds_bytes, s, sg, table, nprobs); break;
@@ -2888,6 +3092,29 @@ static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkPro
                                  const TkLaunchCfg &cfg) {
   constexpr int TW = ((RT >= 4 && P <= 2) || (RT == 2 && P == 1)) ? 2 : 1;
   const int threads = cfg.waves * 64;
+  if constexpr (RT == 1) {
+    if (cfg.fused) {  // the operand rows are built inside the kernel: one problem, 256 threads
+      if (table || threads != 256) return hipErrorInvalidValue;
+      if constexpr (P <= 2) {
+        if (cfg.tw == 2) {
+          switch (cfg.ring) {
+            case 2: return flow_launch_one(tk_flow_kernel<P, 1, 2, 2, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 3: return flow_launch_one(tk_flow_kernel<P, 1, 2, 3, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 4: return flow_launch_one(tk_flow_kernel<P, 1, 2, 4, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 5: return flow_launch_one(tk_flow_kernel<P, 1, 2, 5, false, true>, s, sg, table, wg_prob, cfg, threads);
+            default: return hipErrorInvalidValue;
+          }
+        }
+      }
+      switch (cfg.ring) {
+        case 2: return flow_launch_one(tk_flow_kernel<P, 1, 1, 2, false, true>, s, sg, table, wg_prob, cfg, threads);
+        case 3: return flow_launch_one(tk_flow_kernel<P, 1, 1, 3, false, true>, s, sg, table, wg_prob, cfg, threads);
+        case 4: return flow_launch_one(tk_flow_kernel<P, 1, 1, 4, false, true>, s, sg, table, wg_prob, cfg, threads);
+        case 5: return flow_launch_one(tk_flow_kernel<P, 1, 1, 5, false, true>, s, sg, table, wg_prob, cfg, threads);
+        default: return hipErrorInvalidValue;
+      }
+    }
+  }
   if constexpr (P <= 2 && RT == 1) {  // one row tile: one or two runs per wave, the host's choice by row count
     if (cfg.tw == 2) {
       switch (cfg.ring) {
