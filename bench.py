@@ -686,6 +686,33 @@ def bench_stack(T, be, rng, iters=100):
         ms = time_calls(be, lambda i: g.launch(), iters)
         res[f"batch{m}_rmsnorm_fused"] = {"ms_per_step_incl_norm_and_quant": round(ms, 4), "tokens_per_s": round(m / ms * 1e3, 1)}
         g.destroy()
+        # the same projections in the order a decoder runs them, one dependent launch after the other: per layer the
+        # q,k,v group (attention norm inside), o, the gate,up group (FFN norm inside), down -- 120 calls per step
+        qkv, gu = [], []
+        for li, L in enumerate(lins):
+            base = li * 7
+            qkv.append(be.group(members[base:base + 3], 1, "bf16", "bf16", norms=[(nw[li][0], 1e-5, False)] * 3))
+            gu.append(be.group(members[base + 4:base + 6], 1, "bf16", "bf16", norms=[(nw[li][1], 1e-5, False)] * 2))
+
+        def chain(_):
+            for li, L in enumerate(lins):
+                base = li * 7
+                qkv[li].launch()
+                be.linear_a8(L["o"], att, m, outs[base + 3])
+                gu[li].launch()
+                be.linear_a8(L["down"], mid, m, outs[base + 6])
+
+        chain_ms = {}
+        for label, fuse in (("two_launches_per_call", 0), ("default", -1)):
+            be.set_fuse_tokens(fuse)
+            chain_ms[label] = time_calls(be, chain, max(5, iters // 10))
+        be.set_fuse_tokens(-1)
+        res[f"batch{m}_layer_by_layer"] = {
+            "ms_per_step": round(chain_ms["default"], 4), "tokens_per_s": round(m / chain_ms["default"] * 1e3, 1),
+            "ms_per_step_with_every_call_as_two_launches": round(chain_ms["two_launches_per_call"], 4),
+            "calls_per_step": 4 * layers_n}
+        for grp in qkv + gu:
+            grp.destroy()
         for x in outs + [hid, att, mid]:
             x.free()
     for L in lins:
@@ -696,7 +723,9 @@ def bench_stack(T, be, rng, iters=100):
             w.free()
     res["workload"] = ("30 layers x (q,k,v,o,gate,up,down), hidden 2560, FFN 6912, 20/5 heads of 128, 1 plane, "
                        "W1.58A8, bf16 in/out; 210 projections in one grouped launch on given inputs; "
-                       "*_rmsnorm_fused: q,k,v and gate,up read RMSNorm(input), computed inside the quantization launch")
+                       "*_rmsnorm_fused: q,k,v and gate,up read RMSNorm(input), computed inside the quantization launch; "
+                       "*_layer_by_layer: the same projections as 120 dependent calls in a decoder's order (q,k,v group with "
+                       "its norm, o, gate,up group with its norm, down), launch-bound")
     res["code_bytes_per_step"] = code_bytes
     return res
 

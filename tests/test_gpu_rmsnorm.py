@@ -120,6 +120,41 @@ def test_rows_with_nan_or_inf_follow_the_host(backend, oracle):
     layer.free()
 
 
+@pytest.mark.parametrize("zero_centered", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("m,k", [(1, 256), (3, 2560), (2, 4096), (4, 6912), (1, 8192), (300, 1024)])
+def test_rows_of_whole_blocks_take_one_pass(backend, oracle, m, k, dtype, zero_centered):
+    """Rows of whole K blocks up to K = 8192 go through the kernel that reads the row once (the sum of squares folds in
+    the canonical order through LDS and lane shuffles): same bits as the host's rmsnorm + quantization for plain rows,
+    an all-zero row, a row with NaN and a row with Inf (whose normalized values the exact fallback reads back)."""
+    print("case rmsnorm-one-pass", m, k, dtype, zero_centered, flush=True)
+    rng = np.random.default_rng(m * 13 + k + zero_centered)
+    n = 40
+    wt, sc = ternary(rng, n, k), scales(rng, n)
+    packed = oracle.pack_matrix(wt, n, k, FMT_TQ2_0)
+    layer = backend.linear([packed], [sc], n, k, T.TernaryFormat(FMT_TQ2_0))
+    x = (rng.standard_normal((m, k)) * 10.0 ** rng.integers(-2, 3)).astype(np.float32)
+    if m >= 2:
+        x[1] = 0.0
+    if m >= 3:
+        x[2, k // 2] = np.nan
+    if m >= 4:
+        x[3, 7] = np.inf
+    host = f32_to_bf16_bits(x) if dtype == "bf16" else x
+    seen = bf16_bits_to_f32(host).reshape(m, k) if dtype == "bf16" else x
+    w = (rng.uniform(-0.5, 0.5, k) if zero_centered else rng.uniform(0.5, 1.5, k)).astype(np.float32)
+    y = np.stack([oracle.rmsnorm(seen[r], w, EPS, zero_centered) for r in range(m)])
+    rc, want = oracle.cpu_mpgemm_with_act_quant(packed, FMT_TQ2_0, y, sc, m, n, k)
+    dx, dw, dout = backend.to_device(host, dtype), backend.to_device(w, "f32"), backend.empty(m * n, "f32")
+    backend.linear_rmsnorm_a8(layer, dx, dw, EPS, m, dout, zero_centered=zero_centered)
+    got = dout.to_host()
+    fin = ~np.isnan(want.reshape(-1))
+    assert (np.isnan(got) == ~fin).all() and same_bits(got[fin], want.reshape(-1)[fin])
+    for a in (dx, dw, dout):
+        a.free()
+    layer.free()
+
+
 def test_group_shares_one_norm_per_activation(backend, oracle):
     """q/k/v read norm1(hid), o reads att as it is, gate/up read norm2(hid): one grouped launch equals
     the single launches, bit for bit, and relaunching it changes nothing."""

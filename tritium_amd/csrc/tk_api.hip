@@ -1824,6 +1824,8 @@ struct tk_group {
   int prep_uniform_m = 0;    // > 0: prep entry j starts at token j * prep_uniform_m
   int prep_wave_pieces = 0;  // > 0: every entry fits the one-wave-per-token prep kernels; the largest piece count
   int prep_fast = 0;         // tk_prep_fast of every entry when they agree
+  int prep_norm_fast = 0;    // some entry has an RMSNorm and tk_prep_norm_fast agrees for every entry: that value
+  int prep_norm_pieces = 0;  // ... and the largest piece count
   unsigned prep_rows = 0;
   int variant = 1;
   size_t wg_prob_off = 0;
@@ -2153,6 +2155,14 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     g->prep_fast = preps.empty() ? 0 : tk_prep_fast(preps[0]);
     for (const TkPrep &pp : preps)
       if (tk_prep_fast(pp) != g->prep_fast) g->prep_fast = 0;
+    bool any_norm = false;
+    g->prep_norm_fast = preps.empty() ? 0 : tk_prep_norm_fast(preps[0]);
+    for (const TkPrep &pp : preps) {
+      any_norm = any_norm || pp.norm_kind != 0;
+      if (tk_prep_norm_fast(pp) != g->prep_norm_fast) g->prep_norm_fast = 0;
+    }
+    if (!any_norm || prep_kind != TK_PREP_A8) g->prep_norm_fast = 0;
+    g->prep_norm_pieces = (int)pieces;
   }
   g->cfg.planes = planes;
   g->cfg.rt = rt;
@@ -2185,7 +2195,7 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
   if (do_prep)
     HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows,
-                          g->prep_wave_pieces, g->prep_fast));
+                          g->prep_wave_pieces, g->prep_fast, g->prep_norm_fast, g->prep_norm_pieces));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);
   // Members whose rows fit LDS take the flow kernel, the others one grouped launch of the prefill kernel. The
   // two read and write disjoint members and fit a CU together (one eight-wave workgroup with its rows in LDS

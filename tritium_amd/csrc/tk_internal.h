@@ -139,11 +139,15 @@ hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n,
 // table_wave_pieces: for a table, the largest piece count (16 * K blocks) of its entries when every entry can
 // take the one-wave-per-token kernels (at most 256 pieces, no norm, no per-block sums), else 0.
 // table_fast: for a table, 1 (f32) or 2 (bf16) when tk_prep_fast says so for every entry (and the same), else 0.
+// table_norm_fast / table_norm_pieces: for a table of quantizations with an RMSNorm in some entry, 1 / 2 when
+// tk_prep_norm_fast says so for every entry (and the same), and the largest piece count; else 0.
 hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
-                          unsigned rows, int table_wave_pieces = 0, int table_fast = 0);
+                          unsigned rows, int table_wave_pieces = 0, int table_fast = 0, int table_norm_fast = 0,
+                          int table_norm_pieces = 0);
 // 1 / 2: rows of f32 / bf16 that the one-wave-per-token kernels may take without per-element tests (whole K
 // blocks, 16-byte aligned, operand rows only); 0 otherwise
 int tk_prep_fast(const TkPrep &pp);
+int tk_prep_norm_fast(const TkPrep &pp);
 void tk_prep_set_team_rows(int rows);  // process-wide: launches of up to `rows` tokens give a token the whole workgroup
 hipError_t tk_launch_skinny(hipStream_t s, const TkProblem *single, const TkProblem *table, int nprobs,
                             const TkLaunchCfg &cfg);

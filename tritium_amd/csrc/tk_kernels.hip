@@ -2672,6 +2672,133 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
   }
 }
 
+// RMSNorm + quantization of rows of whole K blocks (16-byte aligned f32 or bf16 rows and norm weights, at most
+// HELD pieces per thread, operand rows only) in one pass over memory: the token's pieces and their norm weights are
+// loaded once and stay in registers. The sum of squares has to fold in the canonical order (slot t of 256 takes
+// x[t], x[t+256], ... ascending, then the power-of-two tree; see row_inv_rms), which is not the order the pieces
+// are held in, so the values cross LDS once in element order; the tree's levels below 64 pair lanes of the first
+// wave exactly as the slots pair (slot t with slot t + off), by shuffles. Same bits as tk_prep_a8_kernel, which
+// reads the row three times and crosses nine barriers for the tree alone. Entries without a norm skip that part.
+template <int HELD, int FAST>
+__global__ __launch_bounds__(TK_WG) void tk_prep_a8_norm_kernel(TkPrep single, const TkPrep *__restrict__ table,
+                                                                int nprep, int uniform_m) {
+  static_assert(TK_WG == 256, "the canonical reduction has 256 slots");
+  __shared__ __attribute__((aligned(16))) float xs[HELD * 256 * 16];
+  __shared__ float part[TK_WG];
+  __shared__ float shf[4];
+  __shared__ int shi[4];
+  int rowi;
+  const TkPrep &pp = find_prep(single, table, nprep, uniform_m, rowi);
+  const size_t row = rowi, k = pp.k, nb = pp.nb, R = pp.rs;
+  const size_t base = row * k, npieces = nb * 16;
+  const int tid = threadIdx.x;
+  float held[HELD][16];
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)tid + (size_t)it * TK_WG;
+    if (pc < npieces) load_piece_fast<FAST>(pp.act, base, piece_elem0(pc >> 4, (int)(pc & 15)), held[it]);
+  }
+  if (pp.norm_kind) {  // uniform over the workgroup
+    float w[HELD][16];
+#pragma unroll
+    for (int it = 0; it < HELD; ++it) {
+      const size_t pc = (size_t)tid + (size_t)it * TK_WG;
+      if (pc >= npieces) continue;
+      const size_t e0 = piece_elem0(pc >> 4, (int)(pc & 15));
+#pragma unroll
+      for (int sl = 0; sl < 4; ++sl) {
+        const v4u u = *(const TK_GLOBAL v4u *)(pp.norm_w + e0 + (size_t)sl * 32);
+        w[it][sl * 4 + 0] = __uint_as_float(u.x);
+        w[it][sl * 4 + 1] = __uint_as_float(u.y);
+        w[it][sl * 4 + 2] = __uint_as_float(u.z);
+        w[it][sl * 4 + 3] = __uint_as_float(u.w);
+        *(float4 *)(xs + e0 + (size_t)sl * 32) =
+            make_float4(held[it][sl * 4], held[it][sl * 4 + 1], held[it][sl * 4 + 2], held[it][sl * 4 + 3]);
+      }
+    }
+    __syncthreads();
+    float acc = 0.0f;
+    for (size_t i = tid; i < k; i += TK_WG) {
+      const float v = xs[i];
+      acc = __fadd_rn(acc, __fmul_rn(v, v));
+    }
+    part[tid] = acc;
+    __syncthreads();
+    if (tid < 128) part[tid] = __fadd_rn(part[tid], part[tid + 128]);
+    __syncthreads();
+    if (tid < 64) {
+      float p = __fadd_rn(part[tid], part[tid + 64]);
+      for (int off = 32; off > 0; off >>= 1) p = __fadd_rn(p, __shfl_down(p, off));  // lanes >= off hold values no one reads
+      if (tid == 0) part[0] = p;
+    }
+    __syncthreads();
+    const float mean_sq = __fdiv_rn(part[0], (float)k);
+    const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean_sq, pp.norm_eps)));  // (see row_inv_rms on sqrtf)
+#pragma unroll
+    for (int it = 0; it < HELD; ++it)
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const float sc = pp.norm_kind == 2 ? __fadd_rn(1.0f, w[it][x]) : w[it][x];
+        held[it][x] = __fmul_rn(__fmul_rn(held[it][x], inv), sc);  // y = (x * inv) * scale(w), left to right
+      }
+  }
+  float g = 0.0f;
+  int nf = 0;
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)tid + (size_t)it * TK_WG;
+    if (pc >= npieces) continue;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) {
+      const float a = fabsf(held[it][x]);
+      if (a > g) g = a;  // NaN never wins (crates/tritium-spec/src/lib.rs:351-360)
+      nf |= !(a <= 3.402823466e38f);
+    }
+  }
+  block_max_any(g, nf, shf, shi);
+  const float gamma = g;
+  const bool nonfinite = nf != 0;
+  const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
+  const bool live = gamma != 0.0f && !nonfinite;
+  const float sl_ = live ? s : 0.0f;
+  float *ynorm = (pp.norm_kind && nonfinite) ? pp.ynorm : nullptr;  // only the exact fallback reads the normalized row
+  int sum = 0;
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)tid + (size_t)it * TK_WG;
+    if (pc >= npieces) continue;
+    const size_t e0 = piece_elem0(pc >> 4, (int)(pc & 15));
+    v4u piece;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      if (ynorm) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) gstore(ynorm + base + e0 + (size_t)sl * 32 + b, held[it][sl * 4 + b]);
+      }
+      uint32_t packed = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        float x = held[it][sl * 4 + b];
+        if (!live) x = 0.0f;  // (a NaN or Inf times zero would not be zero)
+        float r = rintf(__fmul_rn(x, sl_));  // one multiply, ties to even
+        r = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+        const int q = (int)r;
+        sum += q;
+        packed |= ((uint32_t)q & 0xFFu) << (8 * b);
+      }
+      piece[sl] = packed;
+    }
+    *(TK_GLOBAL v4u *)(pp.ap + piece_offset(pc >> 4, (int)(pc & 15), R, row)) = piece;
+  }
+  sum = block_sum(sum, shi);
+  if (tid == 0) {
+    if (pp.rowsum) pp.rowsum[row] = sum;
+    pp.act_scale[row] = gamma == 0.0f ? 0.0f : __fdiv_rn(gamma, 127.0f);
+    if (pp.aux) pp.aux[row] = s;
+    if (pp.flags) pp.flags[row] = nonfinite ? 1u : 0u;
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // Decode in one launch: the flow kernel builds the operand rows of its one to four tokens itself. Every workgroup
 // repeats the prep kernels' work for all tokens -- a few elements per thread -- in place of a second launch in
@@ -2933,12 +3060,34 @@ int tk_prep_fast(const TkPrep &pp) {
   if (!ok) return 0;
   return pp.act_dtype == TK_F32 ? 1 : (pp.act_dtype == TK_BF16 ? 2 : 0);
 }
+// ... the same for the one-pass RMSNorm + quantization kernel, which takes entries with and without a norm (at most
+// 512 pieces, i.e. K <= 8192; aligned norm weights): 1 (f32) or 2 (bf16), else 0
+int tk_prep_norm_fast(const TkPrep &pp) {
+  const bool ok = pp.k % 256 == 0 && (((size_t)pp.act) & 15) == 0 && pp.ap && !pp.q_rowmajor && !pp.blocksum &&
+                  pp.nb * 16 <= 2 * (size_t)TK_WG && (!pp.norm_kind || (pp.norm_w && (((size_t)pp.norm_w) & 15) == 0));
+  if (!ok) return 0;
+  return pp.act_dtype == TK_F32 ? 1 : (pp.act_dtype == TK_BF16 ? 2 : 0);
+}
 
 hipError_t tk_launch_prep(hipStream_t s, int kind, const TkPrep *single, const TkPrep *table, int nprep, int uniform_m,
-                          unsigned rows, int table_wave_pieces, int table_fast) {
+                          unsigned rows, int table_wave_pieces, int table_fast, int table_norm_fast, int table_norm_pieces) {
   if (!rows) return hipSuccess;
   TkPrep dummy = {};
   const TkPrep &sg = single ? *single : dummy;
+  // RMSNorm in front of the quantization, rows of whole K blocks: one pass over memory
+  const int norm_fast = kind != TK_PREP_A8 ? 0 : (single ? (single->norm_kind ? tk_prep_norm_fast(*single) : 0) : table_norm_fast);
+  if (norm_fast) {
+    const size_t pieces = single ? single->nb * 16 : (size_t)table_norm_pieces;
+    const dim3 grid(rows), block(TK_WG);
+    if (pieces <= (size_t)TK_WG) {
+      if (norm_fast == 2) hipLaunchKernelGGL((tk_prep_a8_norm_kernel<1, 2>), grid, block, 0, s, sg, table, nprep, uniform_m);
+      else hipLaunchKernelGGL((tk_prep_a8_norm_kernel<1, 1>), grid, block, 0, s, sg, table, nprep, uniform_m);
+    } else {
+      if (norm_fast == 2) hipLaunchKernelGGL((tk_prep_a8_norm_kernel<2, 2>), grid, block, 0, s, sg, table, nprep, uniform_m);
+      else hipLaunchKernelGGL((tk_prep_a8_norm_kernel<2, 1>), grid, block, 0, s, sg, table, nprep, uniform_m);
+    }
+    return hipGetLastError();
+  }
   // Rows that need neither a norm nor per-block sums, whose pieces the threads working on a token can keep
   // in registers. Team = the threads of one token: a wave (four tokens per workgroup, no barrier), up to 4
   // pieces per lane (K <= 4096) or 8 in the straight-line form (whole K blocks, aligned rows of one element
