@@ -519,13 +519,15 @@ int tk_set_gemm_two_by_two(tk_ctx *ctx, int on);
  * workgroup instead of one wave (few tokens: the launch lasts as long as one token's chain of instructions).
  * Default 384 (the digit split of the float contract: 8/3 of it). Process-wide; identical bits either way. A tuning and test knob. */
 int tk_set_prep_team_rows(tk_ctx *ctx, int rows);
-/* Single decode calls (tk_linear_a8, tk_linear_float and their variants without RMSNorm) of up to `tokens`
- * tokens run as ONE launch: the decode kernel quantizes (or digit-splits) the tokens itself, every workgroup for
- * itself, instead of a prep launch in front of it -- where the rows fit (K a multiple of 256 up to 8192, 16-byte
- * aligned f32 or bf16 rows, operand rows within 62 KiB of LDS; 48 KiB in the K-split kernel of narrow launches).
- * Every workgroup repeats the tokens' quantization, so the form pays for very few tokens: -1 (default) = one token,
- * or two under the int8 contract in the K-split kernel; 0 = never; 1..4 = up to that many. Identical bits either way.
- * A tuning and test knob. */
+/* Decode calls of very few tokens run as ONE launch: the decode kernel quantizes (or digit-splits) the tokens
+ * itself, every workgroup for itself, instead of a prep launch in front of it. Single calls (tk_linear_a8,
+ * tk_linear_float, tk_linear_a8_residual; tk_linear_rmsnorm_a8 for one token, norm included) and groups created
+ * after the call (every member within the limits; a member behind an RMSNorm holds one token). Limits: K a multiple
+ * of 256 up to 8192, 16-byte aligned f32 or bf16 rows (and norm weights), operand rows within 62 KiB of LDS in the
+ * flow kernel or 48 KiB in the K-split kernel of narrow launches, and there at most two workgroups per CU (beyond
+ * that the repeated quantization costs more than the launch saved). tokens: -1 (default) = one token, or two under
+ * the int8 contract in the K-split kernel (single calls); 0 = never; 1..4 = up to that many. Identical bits either
+ * way. A tuning and test knob. */
 int tk_set_fuse_tokens(tk_ctx *ctx, int tokens);
 /* Calls of this context so far that ran in that single-launch form (for tests of the dispatch). */
 int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count);

@@ -208,6 +208,98 @@ def test_automatic_dispatch_takes_one_launch_for_one_token(backend, oracle):
     layer.free()
 
 
+@pytest.mark.parametrize("special", ["plain", "zero", "nan", "inf"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("m,normed", [(1, True), (1, False), (2, False), (2, True)])
+def test_group_of_single_tokens_is_one_launch(backend, oracle, kernel, m, normed, dtype, special):
+    """q,k,v behind the attention norm, o on another tensor, gate,up behind a zero-centred norm, as one group: with one
+    token per member the K-split kernel builds every member's rows (norm included) itself. Same bits as the single
+    two-launch calls; two tokens behind a norm keep the prep launch."""
+    if kernel != KSPLIT:
+        pytest.skip("groups take the form in the K-split kernel")
+    print("case fused-group", m, normed, dtype, special, flush=True)
+    backend.set_decode_kernel(0)
+    rng = np.random.default_rng(m * 7 + normed + len(special))
+    h, f, kv = 512, 1280, 128
+    hid_h, att_h = _tokens(rng, m, h, special), _tokens(rng, m, h, "plain")
+    conv = (lambda a: f32_to_bf16_bits(a)) if dtype == "bf16" else (lambda a: a)
+    hid, att = backend.to_device(conv(hid_h), dtype), backend.to_device(conv(att_h), dtype)
+    w1 = backend.to_device(rng.uniform(0.5, 1.5, h).astype(np.float32), "f32")
+    w2 = backend.to_device(rng.uniform(-0.5, 0.5, h).astype(np.float32), "f32")
+    n1, n2 = ((w1, 1e-5, False), (w2, 1e-5, True)) if normed else (None, None)
+    spec = [("q", h, hid, n1), ("k", kv, hid, n1), ("v", kv, hid, n1), ("o", h, att, None), ("gate", f, hid, n2), ("up", f, hid, n2)]
+    members, norms, singles = [], [], []
+    for name, n, src, nm in spec:
+        layer = backend.linear([T.pack_rows(ternary(rng, n, h, 0.4), n, h)], [scales(rng, n)], n, h)
+        members.append((layer, src, m, backend.empty(m * n, "f32")))
+        norms.append(nm)
+        singles.append(backend.empty(m * n, "f32"))
+    backend.set_fuse_tokens(4)
+    grp = backend.group(members, 1, dtype, "f32", norms=norms if normed else None)
+    before = backend.fused_calls()
+    grp.launch()
+    grp.launch()
+    one = not (normed and m > 1)
+    assert backend.fused_calls() - before == (2 if one else 0)
+    backend.set_fuse_tokens(0)
+    for (layer, src, _, out_g), nm, out_s in zip(members, norms, singles):
+        if nm is None:
+            backend.linear_a8(layer, src, m, out_s)
+        else:
+            backend.linear_rmsnorm_a8(layer, src, nm[0], nm[1], m, out_s, zero_centered=nm[2])
+        assert _same(out_s.to_host(), out_g.to_host()), (m, normed, dtype, special)
+    if not normed:  # the float contract has groups too (no norm there)
+        backend.set_fuse_tokens(4)
+        fmembers = [(layer, src, m, backend.empty(m * layer.n, "f32")) for (layer, src, _, _) in members]
+        fgrp = backend.group(fmembers, 0, dtype, "f32")
+        before = backend.fused_calls()
+        fgrp.launch()
+        assert backend.fused_calls() == before + 1
+        backend.set_fuse_tokens(0)
+        for (layer, src, _, out_g), out_s in zip(fmembers, singles):
+            backend.linear_float(layer, src, m, out_s)
+            assert _same(out_s.to_host(), out_g.to_host())
+        fgrp.destroy()
+        for mem in fmembers:
+            mem[3].free()
+    grp.destroy()
+    for (layer, _, _, out_g), out_s in zip(members, singles):
+        out_g.free()
+        out_s.free()
+        layer.free()
+    for a in (hid, att, w1, w2):
+        a.free()
+
+
+def test_single_call_behind_a_norm_is_one_launch(backend, oracle, kernel):
+    """tk_linear_rmsnorm_a8 on one token: norm, quantization and contraction in one launch, the oracle's bits (a row
+    with an Inf goes through the exact fallback, which reads the normalized row from LDS)."""
+    print("case fused-normed-single", kernel, flush=True)
+    rng = np.random.default_rng(11)
+    n, k = 6912, 2560
+    ws, scs, packed = _planes(rng, n, k, 2)
+    layer = backend.linear(packed, scs, n, k)
+    w = rng.uniform(0.5, 1.5, k).astype(np.float32)
+    dw = backend.to_device(w, "f32")
+    for special in ("plain", "inf", "zero"):
+        x = _tokens(rng, 1, k, special)
+        y = oracle.rmsnorm(x[0], w, 1e-5).reshape(1, k)
+        want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, y, 1, n, k).reshape(-1)
+        dx, out = backend.to_device(x, "f32"), backend.empty(n, "f32")
+        got = {}
+        for fuse in (4, 0):
+            backend.set_fuse_tokens(fuse)
+            before = backend.fused_calls()
+            backend.linear_rmsnorm_a8(layer, dx, dw, 1e-5, 1, out)
+            assert backend.fused_calls() - before == (1 if fuse else 0)
+            got[fuse] = out.to_host().copy()
+        assert _same(got[0], got[4]) and _same(want, got[4]), special
+        for a in (dx, out):
+            a.free()
+    dw.free()
+    layer.free()
+
+
 def test_knob_rejects_other_values(backend):
     with pytest.raises(T.BackendError):
         backend.set_fuse_tokens(5)

@@ -586,8 +586,9 @@ class Mi355xBackend:
         _check(self._lib.tk_set_group_overlap(self._ctx, 1 if on else 0))
 
     def set_fuse_tokens(self, tokens):
-        """Single decode calls of up to `tokens` tokens (1..4) build their operand rows inside the decode kernel: one
-        launch instead of two. 0 = always the separate prep launch, -1 (default) = chosen per call."""
+        """Decode calls (and groups created afterwards) of up to `tokens` tokens (1..4) build their operand rows inside
+        the decode kernel: one launch instead of two. 0 = always the separate prep launch, -1 (default) = chosen per
+        call (one token; two under the int8 contract in single narrow calls)."""
         _check(self._lib.tk_set_fuse_tokens(self._ctx, tokens))
 
     def fused_calls(self):

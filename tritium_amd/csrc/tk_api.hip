@@ -1030,11 +1030,19 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   const int fuse_limit = ctx->fuse_tokens >= 0 ? ctx->fuse_tokens : ((prep_kind == TK_PREP_A8 && variant == DECODE_KSPLIT) ? 2 : 1);
   // Both decode kernels of single launches have the form: the K-split kernel (its rows fit LDS in one pass) and the
   // flow kernel in its 16x16x64 form.
-  const bool fuse_rows = pl.skinny && !norm && pl.cfg.rt == 1 && (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) &&
+  // An RMSNorm in front (one token): the row crosses LDS once more for the canonical sum of squares (k floats and
+  // 1 KiB behind the row constants).
+  const size_t fuse_lds = 1024 + (norm ? k * 4 + 1024 : 0);
+  const bool fuse_rows = pl.skinny && pl.cfg.rt == 1 && (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) &&
                          m <= (size_t)fuse_limit && nb * 16 <= 512 && k % 256 == 0 && ((uintptr_t)act & 15) == 0 &&
-                         (act_dtype == TK_F32 || act_dtype == TK_BF16);
-  const bool fused_flow = fuse_rows && variant == DECODE_FLOW && !wide && !b3 && flow_lds + 2048 <= 64 * 1024;
-  const bool fused_ksplit = fuse_rows && variant == DECODE_KSPLIT && (size_t)pl.pr.kc >= nb && pl.cfg.lds_bytes + 2048 <= 64 * 1024;
+                         (act_dtype == TK_F32 || act_dtype == TK_BF16) &&
+                         (!norm || (m == 1 && fuse_limit >= 1 && ((uintptr_t)norm->weight & 15) == 0));
+  const bool fused_flow = fuse_rows && variant == DECODE_FLOW && !wide && !b3 && flow_lds + fuse_lds + 1024 <= 64 * 1024;
+  // (the K-split kernel has one workgroup per output tile, each repeating the tokens' prep: beyond two workgroups per
+  // CU they queue up behind each other and the repeats cost more than the launch saved -- gate,up of hidden 2560,
+  // 864 tiles: 8.4 -> 10.4 us, 10.1 -> 13.1 us behind a norm; q,k,v, 240 tiles: 8.0 -> 5.6 and 9.6 -> 7.0 us)
+  const bool fused_ksplit = fuse_rows && variant == DECODE_KSPLIT && (size_t)pl.pr.kc >= nb && pl.cfg.lds_bytes + fuse_lds + 1024 <= 64 * 1024 &&
+                            pl.cfg.grid <= 2u * (unsigned)ctx->info.compute_units;
   const bool fused = fused_flow || fused_ksplit;
   Workspace ws;
   TKCHK(take_workspace(ctx, static_ws, (size_t)pl.pr.rs * nb * 256, R, m, norm ? m * k * 4 : 0, &ws));
@@ -1072,6 +1080,13 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     pr.flags = pp.flags;
     pr.raw_act = norm ? (const void *)pp.ynorm : act;  // the exact fallback re-quantizes the normalized row
     pr.raw_dtype = norm ? TK_F32 : act_dtype;
+    if (fused && norm) {  // the kernel normalizes the raw row itself
+      pr.raw_act = act;
+      pr.raw_dtype = act_dtype;
+      pr.norm_kind = pp.norm_kind;
+      pr.norm_eps = pp.norm_eps;
+      pr.norm_w = pp.norm_w;
+    }
   } else if (prep_kind == TK_PREP_DIGITS) {
     pr.exps = pp.exps;
     pr.flags = pp.flags;
@@ -1093,7 +1108,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     flow_cfg_form(&cfg, wide, b3, flow_lds, R, ztiles, nb);
     if (fused) {
       cfg.fused = 1;
-      cfg.lds_bytes += 1024;
+      cfg.lds_bytes += fuse_lds;
       ctx->fused_calls++;
     }
     pr.run_tiles = run_tiles;
@@ -1110,7 +1125,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else if (pl.skinny) {
     if (fused) {
       pl.cfg.fused = 1;
-      pl.cfg.lds_bytes += 1024;
+      pl.cfg.lds_bytes += fuse_lds;
       ctx->fused_calls++;
     }
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
@@ -1824,6 +1839,7 @@ struct tk_group {
   int prep_uniform_m = 0;    // > 0: prep entry j starts at token j * prep_uniform_m
   int prep_wave_pieces = 0;  // > 0: every entry fits the one-wave-per-token prep kernels; the largest piece count
   int prep_fast = 0;         // tk_prep_fast of every entry when they agree
+  bool fused = false;        // the K-split kernel builds the operand rows itself: no prep launch (decided at creation)
   int prep_norm_fast = 0;    // some entry has an RMSNorm and tk_prep_norm_fast agrees for every entry: that value
   int prep_norm_pieces = 0;  // ... and the largest piece count
   unsigned prep_rows = 0;
@@ -2072,9 +2088,28 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     if (!group_ztiles)
       for (size_t i = 0; i < count; ++i) plans[i].pr.zskip = 0;
   }
+  // One launch for a group of single tokens (q,k,v or gate,up of a decode step, with their RMSNorm): the K-split
+  // kernel builds every member's operand rows itself, as for single calls (run_linear). Measured on q,k,v of
+  // hidden 2560 behind a norm, one token: prep 4.8 us + kernel 4.2 us as two dependent launches.
+  bool gfused = variant == DECODE_KSPLIT && rt == 1 && (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) &&
+                (act_dtype == TK_F32 || act_dtype == TK_BF16);
+  size_t fuse_lds = 1024;
+  {
+    const size_t glimit = ctx->fuse_tokens >= 0 ? (size_t)ctx->fuse_tokens : 1;
+    for (size_t i = 0; i < count && gfused; ++i) {
+      const TkPrep &pp = preps[prep_of[i]];
+      const size_t k = (size_t)plans[i].pr.k, nb = (size_t)plans[i].pr.nb;
+      gfused = (size_t)members[i].m <= glimit && nb * 16 <= 512 && k % 256 == 0 && ((uintptr_t)members[i].act & 15) == 0 &&
+               (size_t)plans[i].pr.kc >= nb &&
+               (!pp.norm_kind || (members[i].m == 1 && ((uintptr_t)pp.norm_w & 15) == 0));
+      if (pp.norm_kind && 2048 + k * 4 > fuse_lds) fuse_lds = 2048 + k * 4;
+    }
+    gfused = gfused && lds + fuse_lds + 1024 <= 64 * 1024 && tiles <= 2u * (unsigned)ctx->info.compute_units;  // (as for single calls)
+  }
   tk_group *g = new (std::nothrow) tk_group();
   if (!g) return tk_fail(TK_ERR_BACKEND, "tk_group_create: host allocation failed");
   g->ctx = ctx;
+  g->fused = gfused;
   int rc = dev_malloc(ws_bytes, &g->ws);
   const size_t wg_prob_off = count * sizeof(TkProblem) + preps.size() * sizeof(TkPrep);
   const size_t flow_wg_prob_off = wg_prob_off + wg_prob.size() * sizeof(int);
@@ -2112,6 +2147,13 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       pr.aux = pp.aux;
     } else {
       pr.exps = pp.exps;
+    }
+    if (gfused) {  // the kernel reads (and normalizes) the raw rows itself
+      pr.raw_act = members[i].act;
+      pr.raw_dtype = act_dtype;
+      pr.norm_kind = pp.norm_kind;
+      pr.norm_eps = pp.norm_eps;
+      pr.norm_w = pp.norm_w;
     }
     probs[i] = pr;
   }
@@ -2182,6 +2224,10 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max));
   }
   if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max);
+  if (gfused) {
+    g->cfg.fused = 1;
+    g->cfg.lds_bytes += fuse_lds;
+  }
   ctx->refs.fetch_add(1);
   *out = g;
   return TK_OK;
@@ -2193,7 +2239,8 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   HIPCHK(hipSetDevice(ctx->device));
   const TkProblem *probs = (const TkProblem *)g->tables;
   const TkPrep *preps = (const TkPrep *)((const uint8_t *)g->tables + (size_t)g->nprobs * sizeof(TkProblem));
-  if (do_prep)
+  if (do_main && g->fused) ctx->fused_calls++;
+  if (do_prep && !g->fused)  // (a group that runs as one launch has no prep part)
     HIPCHK(tk_launch_prep(ctx->stream, g->prep_kind, nullptr, preps, g->nprep, g->prep_uniform_m, g->prep_rows,
                           g->prep_wave_pieces, g->prep_fast, g->prep_norm_fast, g->prep_norm_pieces));
   const int *wg_prob = (const int *)((const uint8_t *)g->tables + g->wg_prob_off);

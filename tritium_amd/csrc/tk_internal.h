@@ -50,6 +50,11 @@ struct TkProblem {
   const int32_t *exps;       // DIGITS: [M] binary exponent of the fixed-point grid
   const uint32_t *flags;     // [M] non-zero -> row takes the exact sequential fallback (or null)
   const void *raw_act;       // original activations [M,K] for the fallback (or null)
+  // kernels that build the operand rows themselves (one launch per call): an RMSNorm in front of the quantization
+  // of raw_act (norm_kind 0 = none, 1 = scale w, 2 = scale 1 + w), one token
+  const float *norm_w;
+  float norm_eps;
+  int norm_kind;
   // block-scale planes only: per plane the f32 block scales [(tile, K block), 16 rows], and the sums
   // of every operand row over each K block [nb][R]
   const float *bscale[TK_MAX_PLANES];

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tile = blockIdx.x;
   const TkProblem *prp = &single;
-  if (!FUSED && table) {
+  if (table) {
     int lo = 0, hi = nprobs - 1;  // last problem with tile_begin <= tile
     while (lo < hi) {
       int mid = (lo + hi + 1) >> 1;
@@ -2672,6 +2672,58 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_digits_wave_kernel(TkPrep singl
   }
 }
 
+// y = RMSNorm(x) in place for the pieces of one token that the 256 threads hold (thread t: pieces t, t + 256, ...),
+// through xs [k] and part [256] floats of LDS; see tk_prep_a8_norm_kernel. Every thread passes every barrier, and
+// xs and part are free again on return.
+template <int HELD>
+__device__ __forceinline__ void norm_held_pieces(float (&held)[HELD][16], const float *norm_w, int norm_kind, float eps,
+                                                 size_t k, size_t npieces, float *xs, float *part) {
+  const int tid = threadIdx.x;
+  float w[HELD][16];
+#pragma unroll
+  for (int it = 0; it < HELD; ++it) {
+    const size_t pc = (size_t)tid + (size_t)it * TK_WG;
+    if (pc >= npieces) continue;
+    const size_t e0 = piece_elem0(pc >> 4, (int)(pc & 15));
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      const v4u u = *(const TK_GLOBAL v4u *)(norm_w + e0 + (size_t)sl * 32);
+      w[it][sl * 4 + 0] = __uint_as_float(u.x);
+      w[it][sl * 4 + 1] = __uint_as_float(u.y);
+      w[it][sl * 4 + 2] = __uint_as_float(u.z);
+      w[it][sl * 4 + 3] = __uint_as_float(u.w);
+      *(float4 *)(xs + e0 + (size_t)sl * 32) =
+          make_float4(held[it][sl * 4], held[it][sl * 4 + 1], held[it][sl * 4 + 2], held[it][sl * 4 + 3]);
+    }
+  }
+  __syncthreads();
+  float acc = 0.0f;
+  for (size_t i = tid; i < k; i += TK_WG) {
+    const float v = xs[i];
+    acc = __fadd_rn(acc, __fmul_rn(v, v));
+  }
+  part[tid] = acc;
+  __syncthreads();
+  if (tid < 128) part[tid] = __fadd_rn(part[tid], part[tid + 128]);
+  __syncthreads();
+  if (tid < 64) {
+    float p = __fadd_rn(part[tid], part[tid + 64]);
+    for (int off = 32; off > 0; off >>= 1) p = __fadd_rn(p, __shfl_down(p, off));  // lanes >= off hold values no one reads
+    if (tid == 0) part[0] = p;  // (only this lane read part[0])
+  }
+  __syncthreads();
+  const float mean_sq = __fdiv_rn(part[0], (float)k);
+  __syncthreads();
+  const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean_sq, eps)));  // (see row_inv_rms on sqrtf)
+#pragma unroll
+  for (int it = 0; it < HELD; ++it)
+#pragma unroll
+    for (int x = 0; x < 16; ++x) {
+      const float sc = norm_kind == 2 ? __fadd_rn(1.0f, w[it][x]) : w[it][x];
+      held[it][x] = __fmul_rn(__fmul_rn(held[it][x], inv), sc);  // y = (x * inv) * scale(w), left to right
+    }
+}
+
 // RMSNorm + quantization of rows of whole K blocks (16-byte aligned f32 or bf16 rows and norm weights, at most
 // HELD pieces per thread, operand rows only) in one pass over memory: the token's pieces and their norm weights are
 // loaded once and stay in registers. The sum of squares has to fold in the canonical order (slot t of 256 takes
@@ -2698,50 +2750,7 @@ __global__ __launch_bounds__(TK_WG) void tk_prep_a8_norm_kernel(TkPrep single, c
     const size_t pc = (size_t)tid + (size_t)it * TK_WG;
     if (pc < npieces) load_piece_fast<FAST>(pp.act, base, piece_elem0(pc >> 4, (int)(pc & 15)), held[it]);
   }
-  if (pp.norm_kind) {  // uniform over the workgroup
-    float w[HELD][16];
-#pragma unroll
-    for (int it = 0; it < HELD; ++it) {
-      const size_t pc = (size_t)tid + (size_t)it * TK_WG;
-      if (pc >= npieces) continue;
-      const size_t e0 = piece_elem0(pc >> 4, (int)(pc & 15));
-#pragma unroll
-      for (int sl = 0; sl < 4; ++sl) {
-        const v4u u = *(const TK_GLOBAL v4u *)(pp.norm_w + e0 + (size_t)sl * 32);
-        w[it][sl * 4 + 0] = __uint_as_float(u.x);
-        w[it][sl * 4 + 1] = __uint_as_float(u.y);
-        w[it][sl * 4 + 2] = __uint_as_float(u.z);
-        w[it][sl * 4 + 3] = __uint_as_float(u.w);
-        *(float4 *)(xs + e0 + (size_t)sl * 32) =
-            make_float4(held[it][sl * 4], held[it][sl * 4 + 1], held[it][sl * 4 + 2], held[it][sl * 4 + 3]);
-      }
-    }
-    __syncthreads();
-    float acc = 0.0f;
-    for (size_t i = tid; i < k; i += TK_WG) {
-      const float v = xs[i];
-      acc = __fadd_rn(acc, __fmul_rn(v, v));
-    }
-    part[tid] = acc;
-    __syncthreads();
-    if (tid < 128) part[tid] = __fadd_rn(part[tid], part[tid + 128]);
-    __syncthreads();
-    if (tid < 64) {
-      float p = __fadd_rn(part[tid], part[tid + 64]);
-      for (int off = 32; off > 0; off >>= 1) p = __fadd_rn(p, __shfl_down(p, off));  // lanes >= off hold values no one reads
-      if (tid == 0) part[0] = p;
-    }
-    __syncthreads();
-    const float mean_sq = __fdiv_rn(part[0], (float)k);
-    const float inv = __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean_sq, pp.norm_eps)));  // (see row_inv_rms on sqrtf)
-#pragma unroll
-    for (int it = 0; it < HELD; ++it)
-#pragma unroll
-      for (int x = 0; x < 16; ++x) {
-        const float sc = pp.norm_kind == 2 ? __fadd_rn(1.0f, w[it][x]) : w[it][x];
-        held[it][x] = __fmul_rn(__fmul_rn(held[it][x], inv), sc);  // y = (x * inv) * scale(w), left to right
-      }
-  }
+  if (pp.norm_kind) norm_held_pieces<HELD>(held, pp.norm_w, pp.norm_kind, pp.norm_eps, k, npieces, xs, part);  // uniform over the workgroup
   float g = 0.0f;
   int nf = 0;
 #pragma unroll
@@ -2918,9 +2927,83 @@ __device__ __forceinline__ void fused_token_digits(const void *act, int tok, siz
   }
 }
 
+// One token whose quantization has an RMSNorm in front (the int8 contract): xs [k] and part [256] floats of LDS lie
+// behind the row constants. A normalized row that holds NaN or Inf stays in xs, where the exact fallback reads it.
+template <int FAST>
+__device__ __forceinline__ void fused_token_a8_normed(const TkProblem &pr, uint4 *rows, uint8_t *cst, float *shf, int *shi) {
+  const int lane = threadIdx.x;
+  const size_t k = (size_t)pr.k, nb = (size_t)pr.nb, R = (size_t)pr.R, npieces = nb * 16;
+  float *xs = (float *)(cst + 1024), *part = xs + k;
+  float held[TK_FUSED_HELD][16];
+#pragma unroll
+  for (int it = 0; it < TK_FUSED_HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 256;
+    if (pc < npieces) load_piece_fast<FAST>(pr.raw_act, 0, piece_elem0(pc >> 4, (int)(pc & 15)), held[it]);
+  }
+  norm_held_pieces<TK_FUSED_HELD>(held, pr.norm_w, pr.norm_kind, pr.norm_eps, k, npieces, xs, part);
+  float gamma = 0.0f;
+  int nonfinite = 0;
+#pragma unroll
+  for (int it = 0; it < TK_FUSED_HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 256;
+    if (pc >= npieces) continue;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) {
+      const float a = fabsf(held[it][x]);
+      if (a > gamma) gamma = a;  // NaN never wins (crates/tritium-spec/src/lib.rs:351-360)
+      nonfinite |= !(a <= 3.402823466e38f);
+    }
+  }
+  block_max_any(gamma, nonfinite, shf, shi);
+  const float s = gamma == 0.0f ? 0.0f : __fdiv_rn(127.0f, gamma);  // one divide
+  const bool live = gamma != 0.0f && !nonfinite;
+  const float sl_ = live ? s : 0.0f;
+  int sum = 0;
+#pragma unroll
+  for (int it = 0; it < TK_FUSED_HELD; ++it) {
+    const size_t pc = (size_t)lane + (size_t)it * 256;
+    if (pc >= npieces) continue;
+    const size_t e0 = piece_elem0(pc >> 4, (int)(pc & 15));
+    uint4 piece;
+    uint32_t *pw = (uint32_t *)&piece;
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      if (nonfinite)  // uniform
+        *(float4 *)(xs + e0 + (size_t)sl * 32) =
+            make_float4(held[it][sl * 4], held[it][sl * 4 + 1], held[it][sl * 4 + 2], held[it][sl * 4 + 3]);
+      uint32_t packed = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        float x = held[it][sl * 4 + b];
+        if (!live) x = 0.0f;  // (a NaN or Inf times zero would not be zero)
+        float r = rintf(__fmul_rn(x, sl_));  // one multiply, ties to even
+        r = __builtin_fminf(__builtin_fmaxf(r, -128.0f), 127.0f);
+        const int q = (int)r;
+        sum += q;
+        packed |= ((uint32_t)q & 0xFFu) << (8 * b);
+      }
+      pw[sl] = packed;
+    }
+    rows[piece_offset(pc >> 4, (int)(pc & 15), R, 0) >> 4] = piece;
+  }
+  sum = block_sum(sum, shi);
+  if (lane == 0) {
+    ((int *)cst)[0] = sum;
+    ((float *)(cst + 256))[0] = gamma == 0.0f ? 0.0f : __fdiv_rn(gamma, 127.0f);
+    ((uint32_t *)(cst + 512))[0] = nonfinite ? 1u : 0u;
+    ((float *)(cst + 768))[0] = s;
+  }
+}
+
 __device__ __forceinline__ void fused_stage_rows(const TkProblem &pr, uint4 *rows, uint8_t *cst) {
   __shared__ float shf[4];
   __shared__ int shi[32];
+  if (pr.norm_kind) {  // (one token under the int8 contract: the host's rule)
+    if (pr.raw_dtype == TK_BF16) fused_token_a8_normed<2>(pr, rows, cst, shf, shi);
+    else fused_token_a8_normed<1>(pr, rows, cst, shf, shi);
+    __syncthreads();
+    return;
+  }
   const int M = pr.M;
   const size_t k = (size_t)pr.k, nb = (size_t)pr.nb, R = (size_t)pr.R;
   const void *act = pr.raw_act;
@@ -2937,6 +3020,26 @@ __device__ __forceinline__ void fused_stage_rows(const TkProblem &pr, uint4 *row
   __syncthreads();
 }
 
+// seq_dot_raw() under the int8 contract for a row of f32 values that lies in LDS (the normalized row of the fused
+// form): seq_dot_raw reads its activations with global loads, which an LDS address must never reach.
+__device__ __noinline__ float seq_dot_a8_lds(const uint8_t *codes, int nb, int kdim, const float *y, int n, float s,
+                                             int gamma_zero) {
+  float acc = 0.0f;
+  for (int k = 0; k < kdim; ++k) {
+    const int code = code_at(codes, nb, n, k);
+    if (code == 1) continue;
+    float a = y[k];
+    if (gamma_zero) {
+      a = 0.0f;
+    } else {
+      a = rintf(__fmul_rn(a, s));
+      a = a < -128.0f ? -128.0f : (a > 127.0f ? 127.0f : a);
+    }
+    acc = (code == 2) ? __fadd_rn(acc, a) : __fsub_rn(acc, a);
+  }
+  return acc;
+}
+
 // exact_rows() with the per-token constants of the fused form (in LDS, not in the problem's arrays)
 __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int rowbase, unsigned flag, const uint8_t *cst) {
   if (pr.out_dtype == TK_I32) return;
@@ -2948,7 +3051,10 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
     const float s = a8 ? ((const float *)(cst + 768))[m] : 0.0f;
     float f = 0.0f;
     for (int p = 0; p < pr.planes; ++p) {
-      float t = __fmul_rn(seq_dot_raw(pr.codes[p], pr.nb, pr.k, pr.raw_act, pr.raw_dtype, n, m, a8 ? 1 : 0, s, a8 && as == 0.0f), pr.scales[p][n]);
+      // behind an RMSNorm (one token) the row to re-quantize is the normalized one, left in LDS by the staging
+      const float dot = pr.norm_kind ? seq_dot_a8_lds(pr.codes[p], pr.nb, pr.k, (const float *)(cst + 1024), n, s, as == 0.0f)
+                                     : seq_dot_raw(pr.codes[p], pr.nb, pr.k, pr.raw_act, pr.raw_dtype, n, m, a8 ? 1 : 0, s, a8 && as == 0.0f);
+      float t = __fmul_rn(dot, pr.scales[p][n]);
       f = p == 0 ? t : __fadd_rn(f, t);
     }
     if (a8) f = __fmul_rn(f, as);
@@ -3153,8 +3259,8 @@ static hipError_t launch_skinny_p(hipStream_t s, const TkProblem *single, const 
   TkProblem dummy = {};
   const TkProblem &sg = single ? *single : dummy;
   dim3 grid(cfg.grid), block(TK_WG);
-  if (cfg.fused) {  // the operand rows are built inside the kernel: one problem, one row tile
-    if (table || cfg.rt != 1) return hipErrorInvalidValue;
+  if (cfg.fused) {  // the operand rows are built inside the kernel: one row tile
+    if (cfg.rt != 1) return hipErrorInvalidValue;
     hipLaunchKernelGGL((tk_skinny_kernel<P, 1, true>), grid, block, cfg.lds_bytes, s, sg, table, nprobs);
     return hipGetLastError();
   }
