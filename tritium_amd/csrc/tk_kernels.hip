@@ -79,11 +79,21 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
       __syncthreads();
     }
 
-    for (int kbl = wave; kbl < kcn; kbl += 4) {
-      uint4 w[P];
+    // the chunk of the next trip is requested before this trip's arithmetic (the last trip asks for its own chunk
+    // again: a cache hit), so that a wave's round trips to memory overlap with its matrix work
+    uint4 w[P], wn[P];
+    if (wave < kcn) {
 #pragma unroll
       for (int p = 0; p < P; ++p)
-        w[p] = *(const uint4 *)(pr.codes[p] + (((size_t)t * nb + kb0 + kbl) * 64 + lane) * 16);
+        wn[p] = *(const uint4 *)(pr.codes[p] + (((size_t)t * nb + kb0 + wave) * 64 + lane) * 16);
+    }
+    for (int kbl = wave; kbl < kcn; kbl += 4) {
+      const int kn = kbl + 4 < kcn ? kbl + 4 : kbl;
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        w[p] = wn[p];
+        wn[p] = *(const uint4 *)(pr.codes[p] + (((size_t)t * nb + kb0 + kn) * 64 + lane) * 16);
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         v4i a[RT];
