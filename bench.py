@@ -262,7 +262,8 @@ def bench_config1(T, be, rng, iters=200):
     (b) one device-resident call on a single 4.4 MB layer (one launch: the decode kernel splits the token's digits
         itself; beside it the same call as two launches -- cache resident and launch-bound, so latency figures,
         not bandwidth ones);
-    (c) the adapter call on host slices (upload, kernels, download, sync per call)."""
+    (c) the adapter call on host slices (through the context's pinned block: host memcpy, copy kernel, decode
+        launch, sync, host memcpy per call)."""
     n, k = 6912, 2560
     trits = [ternary(rng, n, k, 0.4) for _ in range(2)]
     packed = [T.pack_rows(w, n, k) for w in trits]

@@ -519,6 +519,12 @@ int tk_set_gemm_two_by_two(tk_ctx *ctx, int on);
  * workgroup instead of one wave (few tokens: the launch lasts as long as one token's chain of instructions).
  * Default 384 (the digit split of the float contract: 8/3 of it). Process-wide; identical bits either way. A tuning and test knob. */
 int tk_set_prep_team_rows(tk_ctx *ctx, int rows);
+/* Host-slice calls (tk_mpgemm, tk_mpgemm_with_act_quant) whose operands (activation, scales, output) total at most
+ * `bytes` go through a pinned host block that the context owns: one copy kernel brings activation and scales to the
+ * device, the kernels write the output into the block, the call synchronizes once -- in place of four transfers from
+ * and to pageable memory. Larger calls, and when no pinned memory can be had, take those transfers. Default 1 MiB;
+ * 0 = never; at most 64 MiB. Identical results. A tuning and test knob. */
+int tk_set_host_direct_bytes(tk_ctx *ctx, size_t bytes);
 /* Decode calls of very few tokens run as ONE launch: the decode kernel quantizes (or digit-splits) the tokens
  * itself, every workgroup for itself, instead of a prep launch in front of it. Single calls (tk_linear_a8,
  * tk_linear_float, tk_linear_a8_residual; tk_linear_rmsnorm_a8 for one token, norm included) and groups created

@@ -126,3 +126,38 @@ def test_determinism(backend, oracle):
     _, a = _run(backend, oracle, v, fused=True)
     _, b = _run(backend, oracle, v, fused=True)
     assert same_bits(a, b)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 6912, 2560), (3, 300, 700), (40, 520, 1280), (1, 33, 256), (300, 1100, 512)])
+def test_host_calls_through_the_pinned_block_agree_with_the_transfers(backend, oracle, m, n, k):
+    """Small host-slice calls go through the context's pinned block (one copy kernel in, the kernels write the output
+    into it); larger ones, and all of them with the knob at 0, take four transfers from and to pageable memory. Same
+    bits either way under both contracts, a NaN token included; the int8 contract equals the CPU oracle."""
+    print("case host-direct", m, n, k, flush=True)
+    from helpers import ternary, scales as mk_scales
+    from oracle_lib import FMT_TQ2_0
+    rng = np.random.default_rng(m + n + k)
+    w, sc = ternary(rng, n, k, 0.4), mk_scales(rng, n)
+    packed = T.pack_rows(w, n, k)
+    buf = backend.upload_weights(packed, T.GemmShape(0, n, k), T.TernaryFormat.Tq2_0)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    if m >= 3:
+        act[1, 3] = np.nan
+    got = {}
+    for direct in (1 << 20, 0):
+        backend.set_host_direct_bytes(direct)
+        for fused in (True, False):
+            out = np.zeros(m * n, np.float32)
+            p = T.MpGemm(act=act.reshape(-1), weights=buf, scales=sc, shape=T.GemmShape(m, n, k),
+                         format=T.TernaryFormat.Tq2_0, out=out)
+            (backend.mpgemm_with_act_quant if fused else backend.mpgemm)(p)
+            got[(direct, fused)] = out
+    backend.set_host_direct_bytes(1 << 20)
+    for fused in (True, False):
+        a, b = got[(1 << 20, fused)], got[(0, fused)]
+        fin = ~np.isnan(a)
+        assert (np.isnan(b) == ~fin).all() and same_bits(a[fin], b[fin]), fused
+    rc, want = oracle.cpu_mpgemm_with_act_quant(packed, FMT_TQ2_0, act, sc, m, n, k)
+    fin = ~np.isnan(want.reshape(-1))
+    assert same_bits(got[(1 << 20, True)][fin], want.reshape(-1)[fin])
+    buf.free()

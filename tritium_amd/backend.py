@@ -585,6 +585,11 @@ class Mi355xBackend:
         """Grouped launches of two kernels (flow part + prefill-kernel part): side by side (default) or in turn."""
         _check(self._lib.tk_set_group_overlap(self._ctx, 1 if on else 0))
 
+    def set_host_direct_bytes(self, nbytes):
+        """Host-slice calls (`mpgemm`, `mpgemm_with_act_quant`) of up to `nbytes` of operands go through the context's
+        pinned host block instead of four pageable transfers (default 1 MiB, 0 = never)."""
+        _check(self._lib.tk_set_host_direct_bytes(self._ctx, nbytes))
+
     def set_fuse_tokens(self, tokens):
         """Decode calls (and groups created afterwards) of up to `tokens` tokens (1..4) build their operand rows inside
         the decode kernel: one launch instead of two. 0 = always the separate prep launch, -1 (default) = chosen per

@@ -85,6 +85,12 @@ struct tk_ctx {
   int gemm_two_by_two = 0;  // one-plane prefill kernel, 64 x 128 form: 0 = four waves side by side, 1 = two by two
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
   unsigned long long fused_calls = 0;  // calls that ran as one launch (tk_get_fused_calls)
+  // Host-slice calls (tk_mpgemm, tk_mpgemm_with_act_quant) of up to host_direct_bytes of operands: the kernels read
+  // the activation and the scales from this pinned host block and write the output into it, so the call is two memcpy
+  // on the host, the launches and one synchronization -- no copy-engine transfers (grow-only; freed with the context)
+  void *pin = nullptr;
+  size_t pin_cap = 0;
+  size_t host_direct_bytes = (size_t)1 << 20;
   int fuse_tokens = -1;    // single decode calls of up to this many tokens build their operand rows inside the decode kernel (-1 = chosen per call, 0 = never)
   int gemm_rows = 0;       // one-plane int8-contract prefill, single launches: 0 = tile rows chosen per launch, 64 / 128 = force
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
@@ -279,6 +285,9 @@ extern "C" void tk_destroy(tk_ctx *ctx) {
     }
     if (ctx->d_invalid) (void)hipFree(ctx->d_invalid);
     ctx->d_invalid = nullptr;
+    if (ctx->pin) (void)hipHostFree(ctx->pin);
+    ctx->pin = nullptr;
+    ctx->pin_cap = 0;
   }
   ctx_release(ctx);
 }
@@ -354,6 +363,14 @@ extern "C" int tk_set_group_overlap(tk_ctx *ctx, int on) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_group_overlap: null context");
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->group_overlap = on ? 1 : 0;
+  return TK_OK;
+}
+
+extern "C" int tk_set_host_direct_bytes(tk_ctx *ctx, size_t bytes) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_host_direct_bytes: null context");
+  if (bytes > ((size_t)64 << 20)) return tk_fail(TK_ERR_INVALID_INPUT, "host_direct_bytes=%zu - use at most 64 MiB (0 = never)", bytes);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->host_direct_bytes = bytes;
   return TK_OK;
 }
 
@@ -1697,6 +1714,43 @@ static int host_call(tk_ctx *ctx, bool a8, const float *act, size_t act_len, con
 
   std::lock_guard<std::mutex> lk(ctx->mu);
   HIPCHK(hipSetDevice(ctx->device));
+  size_t macs;
+  const bool tiny = !__builtin_mul_overflow(m * n, k, &macs) && macs <= ctx->exact_max_macs;
+  // Small calls (decode): the operands go through one pinned host block. A copy kernel brings the activation and the
+  // scales to the device in one launch (so whatever reads them more than once reads device memory) and the kernels
+  // write the output into the block themselves: two memcpy on the host, the launches and one synchronization in place
+  // of four copy-engine transfers from and to pageable memory, which cost ~10 us each whatever their size.
+  auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+  const size_t a_b = al(act_len * 4), s_b = al(n * 4), o_b = al(out_len * 4);
+  if (a_b + s_b + o_b <= ctx->host_direct_bytes && (a8 || !tiny)) {
+    if (a_b + s_b + o_b > ctx->pin_cap) {
+      if (ctx->pin) {
+        HIPCHK(hipStreamSynchronize(ctx->stream));
+        (void)hipHostFree(ctx->pin);
+        ctx->pin = nullptr;
+        ctx->pin_cap = 0;
+      }
+      const size_t want = a_b + s_b + o_b + (a_b + s_b + o_b) / 4 + 4096;
+      if (hipHostMalloc(&ctx->pin, want, hipHostMallocDefault) == hipSuccess) ctx->pin_cap = want;
+      else { (void)hipGetLastError(); ctx->pin = nullptr; }  // no pinned memory to be had: the copies below
+    }
+    if (ctx->pin) {
+      uint8_t *pa = (uint8_t *)ctx->pin, *ps = pa + a_b, *po = ps + s_b;
+      memcpy(pa, act, act_len * 4);
+      memcpy(ps, scales, n * 4);
+      TKCHK(ensure(ctx, ctx->h_act, a_b + s_b));
+      HIPCHK(tk_launch_copy(ctx->stream, ctx->h_act.p, pa, a_b + s_b));
+      tk_linear_desc layer = {};
+      layer.planes[0] = weights;
+      layer.scales[0] = (const float *)((const uint8_t *)ctx->h_act.p + a_b);
+      layer.n_planes = 1;
+      TKCHK(run_linear(ctx, &layer, a8 ? TK_MODE_INT8 : TK_MODE_DIGITS, a8 ? TK_PREP_A8 : TK_PREP_DIGITS, ctx->h_act.p, TK_F32,
+                       nullptr, m, po, TK_F32));
+      HIPCHK(hipStreamSynchronize(ctx->stream));
+      memcpy(out, po, out_len * 4);
+      return TK_OK;
+    }
+  }
   TKCHK(ensure(ctx, ctx->h_act, act_len * 4));
   TKCHK(ensure(ctx, ctx->h_scales, n * 4));
   TKCHK(ensure(ctx, ctx->h_out, out_len * 4));
@@ -1706,8 +1760,6 @@ static int host_call(tk_ctx *ctx, bool a8, const float *act, size_t act_len, con
   layer.planes[0] = weights;
   layer.scales[0] = (const float *)ctx->h_scales.p;
   layer.n_planes = 1;
-  size_t macs;
-  const bool tiny = !__builtin_mul_overflow(m * n, k, &macs) && macs <= ctx->exact_max_macs;
   if (a8) {
     TKCHK(run_linear(ctx, &layer, TK_MODE_INT8, TK_PREP_A8, ctx->h_act.p, TK_F32, nullptr, m, ctx->h_out.p, TK_F32));
   } else if (tiny) {
