@@ -85,9 +85,9 @@ struct tk_ctx {
   int gemm_two_by_two = 0;  // one-plane prefill kernel, 64 x 128 form: 0 = four waves side by side, 1 = two by two
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
   unsigned long long fused_calls = 0;  // calls that ran as one launch (tk_get_fused_calls)
-  // Host-slice calls (tk_mpgemm, tk_mpgemm_with_act_quant) of up to host_direct_bytes of operands: the kernels read
-  // the activation and the scales from this pinned host block and write the output into it, so the call is two memcpy
-  // on the host, the launches and one synchronization -- no copy-engine transfers (grow-only; freed with the context)
+  // Host-slice calls (tk_mpgemm, tk_mpgemm_with_act_quant) of up to host_direct_bytes of operands go through this
+  // pinned host block: a copy kernel reads the activation and the scales from it, the kernels write the output into
+  // it -- no copy-engine transfers (see host_call; grow-only; freed with the context)
   void *pin = nullptr;
   size_t pin_cap = 0;
   size_t host_direct_bytes = (size_t)1 << 20;
