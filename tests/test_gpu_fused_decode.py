@@ -271,6 +271,40 @@ def test_group_of_single_tokens_is_one_launch(backend, oracle, kernel, m, normed
         a.free()
 
 
+def test_group_with_members_of_different_k_and_token_counts(backend, oracle, kernel):
+    """One launch for a group whose members differ in K, N, token count and norm: every workgroup sizes its rows, row
+    constants and norm scratch from its own member."""
+    if kernel != KSPLIT:
+        pytest.skip("groups take the form in the K-split kernel")
+    backend.set_decode_kernel(0)
+    backend.set_fuse_tokens(4)
+    rng = np.random.default_rng(21)
+    spec = [(1, 80, 512, True), (2, 48, 1280, False), (1, 200, 2560, True), (3, 33, 256, False), (1, 64, 6912, False)]
+    members, norms, keep = [], [], []
+    for m, n, k, normed in spec:
+        w, sc = ternary(rng, n, k, 0.4), scales(rng, n)
+        layer = backend.linear([T.pack_rows(w, n, k)], [sc], n, k)
+        x = _tokens(rng, m, k, "plain")
+        nw = rng.uniform(0.5, 1.5, k).astype(np.float32)
+        dx, dw, out = backend.to_device(x, "f32"), backend.to_device(nw, "f32"), backend.empty(m * n, "f32")
+        members.append((layer, dx, m, out))
+        norms.append((dw, 1e-5, False) if normed else None)
+        keep.append((layer, dx, dw, out, x, nw, w, sc, m, n, k, normed))
+    grp = backend.group(members, 1, "f32", "f32", norms=norms)
+    before = backend.fused_calls()
+    grp.launch()
+    assert backend.fused_calls() == before + 1
+    for layer, dx, dw, out, x, nw, w, sc, m, n, k, normed in keep:
+        y = np.stack([oracle.rmsnorm(x[r], nw, 1e-5) for r in range(m)]) if normed else x
+        want = oracle.cpu_linear_a8_planes([T.pack_rows(w, n, k)], FMT_TQ2_0, [sc], y, m, n, k)
+        assert same_bits(out.to_host(), want), (m, n, k, normed)
+    grp.destroy()
+    for layer, dx, dw, out, *_ in keep:
+        for a in (dx, dw, out):
+            a.free()
+        layer.free()
+
+
 def test_single_call_behind_a_norm_is_one_launch(backend, oracle, kernel):
     """tk_linear_rmsnorm_a8 on one token: norm, quantization and contraction in one launch, the oracle's bits (a row
     with an Inf goes through the exact fallback, which reads the normalized row from LDS)."""
