@@ -1033,6 +1033,21 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
       pl.skinny = false;
       plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units, ctx->gemm_tiles);
     }
+    // Narrow launches that would take the K-split kernel (one workgroup per 16 outputs, each staging every operand
+    // row): with its K split the prefill kernel is the faster one beyond 32 rows (the K-split kernel's four-row-tile
+    // form), at 32 rows of one plane under the int8 contract, and from 16-20 rows when the rows need more than one
+    // pass through LDS. Measured, call incl. prep, K-split -> prefill kernel, bf16 tokens: 2560 x 2560 one plane,
+    // 32 / 48 / 64 int8 rows 15.4 -> 13.9 / 18.9 -> 14.0 / 22.1 -> 13.9 us, float contract 12 / 16 tokens 18.1 -> 15.1 /
+    // 21.4 -> 15.1 (8 tokens 14.6 -> 15.1: left alone); 6912 x 2560 two planes 48 / 64 rows 21.1 -> 16.2 / 24.5 -> 16.1
+    // (32 rows 17.1 -> 16.0, float 8 tokens 16.1 -> 17.1: left alone); K = 6912 (two passes) one plane 16 / 32 / 64
+    // rows 18.5 -> 16.3 / 27.3 -> 16.6 / 43.8 -> 16.8, two planes 20 rows 23.6 -> 20.5 (16 rows 19.9 -> 20.4).
+    const bool passes = (size_t)pl.pr.kc < nb;
+    if (ctx->decode_force == DECODE_AUTO && pl.skinny && variant == DECODE_KSPLIT &&
+        (R > 32 || (R == 32 && pl.cfg.planes == 1 && mode == TK_MODE_INT8) ||
+         (passes && (R >= 20 || (R >= 16 && pl.cfg.planes == 1))))) {
+      pl.skinny = false;
+      plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units, ctx->gemm_tiles);
+    }
   }
   // A single decode call of few tokens is two short dependent launches, and the gap between them costs more than
   // either: the flow kernel then builds the operand rows itself, every workgroup for itself (256 threads, at most
