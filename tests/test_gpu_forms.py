@@ -362,3 +362,41 @@ def test_activation_prep_forms_agree(backend, oracle, mode, k, m, copies):
             fin = ~np.isnan(a)
             assert (np.isnan(b) == ~fin).all() and same_bits(a[fin], b[fin])
     layer.free()
+
+
+@pytest.mark.parametrize("m", [17, 20, 32, 64])
+def test_narrow_groups_of_several_row_tiles_take_the_prefill_kernel(backend, oracle, m):
+    """q,k,v and gate,up of a decode step of 17..64 tokens are narrow groups (a few hundred tiles) whose rows fit LDS;
+    left to the automatic dispatch they run through the grouped prefill kernel (the K-split kernel below 20 rows for the
+    small group). Whatever is picked: the CPU oracle's bits, with and without an RMSNorm in front."""
+    print("case narrow-group", m, flush=True)
+    rng = np.random.default_rng(900 + m)
+    h, f, kv = 512, 1536, 128
+    x = (rng.standard_normal((m, h)) * 2).astype(np.float32)
+    x[m // 2] = 0.0
+    dx = backend.to_device(x, "f32")
+    nw = rng.uniform(0.5, 1.5, h).astype(np.float32)
+    dw = backend.to_device(nw, "f32")
+    y = np.stack([oracle.rmsnorm(x[r], nw, 1e-5) for r in range(m)])
+    for names in ((h, kv, kv), (f, f)):
+        for normed in (True, False):
+            members, keep = [], []
+            for n in names:
+                w, sc = ternary(rng, n, h, 0.4), scales(rng, n)
+                packed = T.pack_rows(w, n, h)
+                layer = backend.linear([packed], [sc], n, h)
+                out = backend.empty(m * n, "f32")
+                members.append((layer, dx, m, out))
+                keep.append((layer, out, packed, sc, n))
+            grp = backend.group(members, 1, "f32", "f32", norms=[(dw, 1e-5, False)] * len(names) if normed else None)
+            grp.launch()
+            grp.launch()
+            for layer, out, packed, sc, n in keep:
+                want = oracle.cpu_linear_a8_planes([packed], FMT_TQ2_0, [sc], y if normed else x, m, n, h)
+                assert same_bits(out.to_host(), want), (m, n, normed)
+            grp.destroy()
+            for layer, out, *_ in keep:
+                out.free()
+                layer.free()
+    dx.free()
+    dw.free()

@@ -2049,6 +2049,18 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   // (operand rows streamed block by block, int8 MFMA over 64-row tiles) beats a decode kernel that
   // re-stages slices of K behind barriers.
   if (ctx->decode_force == DECODE_AUTO && !flow_ok && rt >= 2) variant = DECODE_GEMM;
+  // A narrow group that would take the K-split kernel with more than one row tile (q,k,v or gate,up of a step of 17+
+  // tokens): the prefill kernel, as for single launches (run_linear). Measured on hidden 2560, one plane, int8 contract
+  // behind an RMSNorm, K-split -> prefill kernel: gate,up (864 tiles) 17 / 24 / 32 / 64 tokens 19.2 -> 14.9 / 21.6 ->
+  // 14.9 / 23.7 -> 15.0 / 35.2 -> 15.3 us; q,k,v (240 tiles) 20 / 32 / 64 tokens 15.1 -> 14.8 / 16.6 -> 14.8 / 23.6 ->
+  // 15.1 (17 tokens 13.7 -> 14.8: left alone). More planes and the float contract from 33 rows on, as single launches.
+  const bool narrow_to_gemm = (planes == 1 && kmode == TK_MODE_INT8) ? (rows_max >= 20 || tiles > 2u * (unsigned)ctx->info.compute_units)
+                                                                       : rows_max > 32;
+  if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && rt >= 2 && narrow_to_gemm) {
+    variant = DECODE_GEMM;
+    flow_ok = false;
+    for (size_t i = 0; i < count; ++i) plans[i].flow_ok = false;
+  }
   std::vector<int> wg_prob;
   int group_gemm_nt = 0;
   unsigned groups_total = 0;
