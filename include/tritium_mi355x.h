@@ -532,8 +532,8 @@ int tk_set_host_direct_bytes(tk_ctx *ctx, size_t bytes);
  * of 256 up to 8192, 16-byte aligned f32 or bf16 rows (and norm weights), operand rows within 62 KiB of LDS in the
  * flow kernel or 48 KiB in the K-split kernel of narrow launches, and there at most two workgroups per CU (beyond
  * that the repeated quantization costs more than the launch saved). tokens: -1 (default) = one token, or two under
- * the int8 contract in the K-split kernel (single calls); 0 = never; 1..4 = up to that many. Identical bits either
- * way. A tuning and test knob. */
+ * the int8 contract in the K-split kernel; 0 = never; 1..4 = up to that many. Identical bits either way. A tuning
+ * and test knob. */
 int tk_set_fuse_tokens(tk_ctx *ctx, int tokens);
 /* Calls of this context so far that ran in that single-launch form (for tests of the dispatch). */
 int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count);
