@@ -1019,7 +1019,10 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R);
     const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
-    variant = choose_decode(ctx, pl.flow_ok, flow_groups, pl.stream_groups);
+    // (an eight-wave workgroup of the flow kernel fills a CU alone: it counts as two. 17408 x 5120 x 3 planes, 16 / 24 /
+    // 32 int8 rows, 136 such workgroups: 36.8 / 32.0 / 32.1 us through the K-split or prefill kernel, 21.2 / 26.3 / 27.5
+    // through the flow kernel)
+    variant = choose_decode(ctx, pl.flow_ok, flow_groups * (unsigned)(fw >= 8 ? 2 : 1), pl.stream_groups);
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
     // Operand rows that do not fit in LDS: the prefill kernel (rows streamed from L2 block by block)
     // beats the decode kernels that re-stage slices of K behind barriers, beyond 32 rows always and
@@ -1035,16 +1038,21 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     }
     // Narrow launches that would take the K-split kernel (one workgroup per 16 outputs, each staging every operand
     // row): with its K split the prefill kernel is the faster one beyond 32 rows (the K-split kernel's four-row-tile
-    // form), at 32 rows of one plane under the int8 contract, and from 16-20 rows when the rows need more than one
-    // pass through LDS. Measured, call incl. prep, K-split -> prefill kernel, bf16 tokens: 2560 x 2560 one plane,
+    // form), beyond 16 rows of one plane under the int8 contract (16384 x 2048, 24 rows: 18.4 -> 12.6 us; a tie on
+    // layers of 2560 outputs), and from 16 rows when the rows need more than one pass through LDS (5120 x 17408 x 3
+    // planes, 16 rows: 42.6 -> 38.8). Measured, call incl. prep, K-split -> prefill kernel, bf16 tokens: 2560 x 2560 one plane,
     // 32 / 48 / 64 int8 rows 15.4 -> 13.9 / 18.9 -> 14.0 / 22.1 -> 13.9 us, float contract 12 / 16 tokens 18.1 -> 15.1 /
     // 21.4 -> 15.1 (8 tokens 14.6 -> 15.1: left alone); 6912 x 2560 two planes 48 / 64 rows 21.1 -> 16.2 / 24.5 -> 16.1
     // (32 rows 17.1 -> 16.0, float 8 tokens 16.1 -> 17.1: left alone); K = 6912 (two passes) one plane 16 / 32 / 64
     // rows 18.5 -> 16.3 / 27.3 -> 16.6 / 43.8 -> 16.8, two planes 20 rows 23.6 -> 20.5 (16 rows 19.9 -> 20.4).
-    const bool passes = (size_t)pl.pr.kc < nb;
+    const size_t n_passes = (nb + (size_t)pl.pr.kc - 1) / (size_t)(pl.pr.kc ? pl.pr.kc : 1);
+    const bool one_a8 = pl.cfg.planes == 1 && mode == TK_MODE_INT8;
+    // (two passes stay: 5120 x 5120 x 3 planes, 16 rows 18.8 vs 22.7 us; float contract 5 tokens of K = 2560, one plane
+    // 13.2 vs 15.1. Three passes at 16 rows only for one plane of int8 rows: 2560 x 6912 18.6 -> 16.8, two planes
+    // 19.8 -> 20.4, float contract 4 tokens x two planes 19.5 -> 21.9)
+    const bool passes = (n_passes >= 3 && (R >= 20 || one_a8)) || n_passes >= 4;
     if (ctx->decode_force == DECODE_AUTO && pl.skinny && variant == DECODE_KSPLIT &&
-        (R > 32 || (R == 32 && pl.cfg.planes == 1 && mode == TK_MODE_INT8) ||
-         (passes && (R >= 20 || (R >= 16 && pl.cfg.planes == 1))))) {
+        (R > 32 || (R > 16 && one_a8) || (passes && R >= 16))) {
       pl.skinny = false;
       plan_gemm(&pl, 4u * (unsigned)ctx->info.compute_units, ctx->gemm_tiles);
     }
