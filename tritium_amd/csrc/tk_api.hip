@@ -2061,9 +2061,12 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   // tokens): the prefill kernel, as for single launches (run_linear). Measured on hidden 2560, one plane, int8 contract
   // behind an RMSNorm, K-split -> prefill kernel: gate,up (864 tiles) 17 / 24 / 32 / 64 tokens 19.2 -> 14.9 / 21.6 ->
   // 14.9 / 23.7 -> 15.0 / 35.2 -> 15.3 us; q,k,v (240 tiles) 20 / 32 / 64 tokens 15.1 -> 14.8 / 16.6 -> 14.8 / 23.6 ->
-  // 15.1 (17 tokens 13.7 -> 14.8: left alone). More planes and the float contract from 33 rows on, as single launches.
-  const bool narrow_to_gemm = (planes == 1 && kmode == TK_MODE_INT8) ? (rows_max >= 20 || tiles > 2u * (unsigned)ctx->info.compute_units)
-                                                                       : rows_max > 32;
+  // 15.1 (17 tokens 13.7 -> 14.8: left alone). More planes and the float contract from 33 rows on, as single launches;
+  // groups of more than two tiles per CU whatever their planes and contract.
+  // (gate,up, float contract 5 / 8 tokens, one plane 18.2 / 20.3 us through the K-split kernel, 14.7 through the prefill
+  // kernel; two planes of int8 rows, 17 / 32 tokens 20.0 / 24.3 against 16.8)
+  const bool many_tiles = tiles > 2u * (unsigned)ctx->info.compute_units;
+  const bool narrow_to_gemm = many_tiles || ((planes == 1 && kmode == TK_MODE_INT8) ? rows_max >= 20 : rows_max > 32);
   if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && rt >= 2 && narrow_to_gemm) {
     variant = DECODE_GEMM;
     flow_ok = false;
