@@ -530,8 +530,8 @@ int tk_set_host_direct_bytes(tk_ctx *ctx, size_t bytes);
  * tk_linear_float, tk_linear_a8_residual; tk_linear_rmsnorm_a8 for one token, norm included) and groups created
  * after the call (every member within the limits; a member behind an RMSNorm holds one token). Limits: K a multiple
  * of 256 up to 8192, 16-byte aligned f32 or bf16 rows (and norm weights), operand rows within 62 KiB of LDS in the
- * flow kernel or 48 KiB in the K-split kernel of narrow launches, and there at most two workgroups per CU (beyond
- * that the repeated quantization costs more than the launch saved). tokens: -1 (default) = one token, or two under
+ * flow kernel or 48 KiB in the K-split kernel of narrow launches, and there at most eight output tiles per CU (a
+ * workgroup takes up to four behind one quantization). tokens: -1 (default) = one token, or two under
  * the int8 contract in the K-split kernel; 0 = never; 1..4 = up to that many. Identical bits either way. A tuning
  * and test knob. */
 int tk_set_fuse_tokens(tk_ctx *ctx, int tokens);

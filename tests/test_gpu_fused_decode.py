@@ -305,6 +305,52 @@ def test_group_with_members_of_different_k_and_token_counts(backend, oracle, ker
         layer.free()
 
 
+@pytest.mark.parametrize("n", [8208, 16384, 20000])
+def test_wide_launches_take_several_tiles_per_workgroup(backend, oracle, kernel, n):
+    """Beyond two output tiles per CU a workgroup of the K-split form stages its rows once and takes up to four
+    consecutive tiles (513 tiles: the last workgroup has one; 1250 tiles: three per workgroup, the last has two).
+    Single calls and a group of two members behind a norm, against the oracle's bits."""
+    if kernel != KSPLIT:
+        pytest.skip("the K-split kernel's form")
+    print("case fused-wide", n, flush=True)
+    rng = np.random.default_rng(n)
+    k = 1024
+    w, sc = ternary(rng, n, k, 0.4), scales(rng, n)
+    packed = T.pack_rows(w, n, k)
+    layer = backend.linear([packed], [sc], n, k)
+    for m in (1, 2):
+        x = _tokens(rng, m, k, "nan" if m == 2 else "plain")
+        dx, out = backend.to_device(x, "f32"), backend.empty(m * n, "f32")
+        before = backend.fused_calls()
+        backend.linear_a8(layer, dx, m, out)
+        assert backend.fused_calls() == before + 1
+        assert _same(oracle.cpu_linear_a8_planes([packed], FMT_TQ2_0, [sc], x, m, n, k).reshape(-1), out.to_host())
+        backend.linear_float(layer, dx, m, out)
+        got = out.to_host().copy()
+        backend.set_fuse_tokens(0)
+        backend.linear_float(layer, dx, m, out)
+        backend.set_fuse_tokens(4)
+        assert _same(out.to_host(), got)
+        for a in (dx, out):
+            a.free()
+    x = _tokens(rng, 1, k, "plain")
+    nw = rng.uniform(0.5, 1.5, k).astype(np.float32)
+    dx, dw = backend.to_device(x, "f32"), backend.to_device(nw, "f32")
+    outs = [backend.empty(n, "f32") for _ in range(2)]
+    grp = backend.group([(layer, dx, 1, o) for o in outs], 1, "f32", "f32", norms=[(dw, 1e-5, True)] * 2)
+    before = backend.fused_calls()
+    grp.launch()
+    assert backend.fused_calls() == before + (1 if 2 * ((n + 15) // 16) <= 2048 else 0)
+    y = oracle.rmsnorm(x[0], nw, 1e-5, True).reshape(1, k)
+    want = oracle.cpu_linear_a8_planes([packed], FMT_TQ2_0, [sc], y, 1, n, k).reshape(-1)
+    for o in outs:
+        assert same_bits(o.to_host(), want)
+    grp.destroy()
+    for a in [dx, dw] + outs:
+        a.free()
+    layer.free()
+
+
 def test_single_call_behind_a_norm_is_one_launch(backend, oracle, kernel):
     """tk_linear_rmsnorm_a8 on one token: norm, quantization and contraction in one launch, the oracle's bits (a row
     with an Inf goes through the exact fallback, which reads the normalized row from LDS)."""

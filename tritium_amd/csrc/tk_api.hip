@@ -1078,11 +1078,14 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
                          (act_dtype == TK_F32 || act_dtype == TK_BF16) &&
                          (!norm || (m == 1 && fuse_limit >= 1 && ((uintptr_t)norm->weight & 15) == 0));
   const bool fused_flow = fuse_rows && variant == DECODE_FLOW && !wide && !b3 && flow_lds + fuse_lds + 1024 <= 64 * 1024;
-  // (the K-split kernel has one workgroup per output tile, each repeating the tokens' prep: beyond two workgroups per
-  // CU they queue up behind each other and the repeats cost more than the launch saved -- gate,up of hidden 2560,
-  // 864 tiles: 8.4 -> 10.4 us, 10.1 -> 13.1 us behind a norm; q,k,v, 240 tiles: 8.0 -> 5.6 and 9.6 -> 7.0 us)
-  const bool fused_ksplit = fuse_rows && variant == DECODE_KSPLIT && (size_t)pl.pr.kc >= nb && pl.cfg.lds_bytes + fuse_lds + 1024 <= 64 * 1024 &&
-                            pl.cfg.grid <= 2u * (unsigned)ctx->info.compute_units;
+  // (the K-split kernel has one workgroup per output tile; in this form each repeats the tokens' prep, and beyond two
+  // workgroups per CU they queue up behind each other and the repeats cost more than the launch saved -- gate,up of
+  // hidden 2560, 864 tiles: 8.4 -> 10.4 us, 10.1 -> 13.1 us behind a norm; q,k,v, 240 tiles: 8.0 -> 5.6 and 9.6 -> 7.0
+  // us. Larger launches therefore give a workgroup up to four consecutive tiles behind one prep.)
+  const size_t fused_ksplit_lds = nb * 256 * R + fuse_lds + (size_t)4096 * pl.cfg.planes;  // rows, constants (+ norm scratch), reduction
+  const unsigned fuse_tpw = (pl.cfg.grid + 2u * (unsigned)ctx->info.compute_units - 1) / (2u * (unsigned)ctx->info.compute_units);
+  const bool fused_ksplit = fuse_rows && variant == DECODE_KSPLIT && (size_t)pl.pr.kc >= nb && fused_ksplit_lds + 1024 <= 64 * 1024 &&
+                            fuse_tpw <= 4;
   const bool fused = fused_flow || fused_ksplit;
   Workspace ws;
   TKCHK(take_workspace(ctx, static_ws, (size_t)pl.pr.rs * nb * 256, R, m, norm ? m * k * 4 : 0, &ws));
@@ -1165,7 +1168,9 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else if (pl.skinny) {
     if (fused) {
       pl.cfg.fused = 1;
-      pl.cfg.lds_bytes += fuse_lds;
+      pl.cfg.lds_bytes = fused_ksplit_lds;
+      pr.run_tiles = (int)(fuse_tpw ? fuse_tpw : 1);
+      pl.cfg.grid = (pl.cfg.grid + (unsigned)pr.run_tiles - 1) / (unsigned)pr.run_tiles;
       ctx->fused_calls++;
     }
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
@@ -2183,7 +2188,8 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   // hidden 2560 behind a norm, one token: prep 4.8 us + kernel 4.2 us as two dependent launches.
   bool gfused = variant == DECODE_KSPLIT && rt == 1 && (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) &&
                 (act_dtype == TK_F32 || act_dtype == TK_BF16);
-  size_t fuse_lds = 1024;
+  size_t fuse_lds = 0;  // LDS of the fused form: the largest member's rows + constants (+ norm scratch) + reduction
+  unsigned fuse_tpw = 1;
   {
     // (q,k,v of hidden 2560 without a norm, two tokens: int8 contract 8.6 -> 7.3 us, float contract 9.7 -> 9.2; three
     // tokens 9.0 -> 9.0 and 10.5 -> 11.2)
@@ -2194,9 +2200,21 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       gfused = (size_t)members[i].m <= glimit && nb * 16 <= 512 && k % 256 == 0 && ((uintptr_t)members[i].act & 15) == 0 &&
                (size_t)plans[i].pr.kc >= nb &&
                (!pp.norm_kind || (members[i].m == 1 && ((uintptr_t)pp.norm_w & 15) == 0));
-      if (pp.norm_kind && 2048 + k * 4 > fuse_lds) fuse_lds = 2048 + k * 4;
+      const size_t need = nb * 256 * (size_t)plans[i].pr.R + 1024 + (pp.norm_kind ? k * 4 + 1024 : 0) + (size_t)4096 * planes;
+      if (need > fuse_lds) fuse_lds = need;
     }
-    gfused = gfused && lds + fuse_lds + 1024 <= 64 * 1024 && tiles <= 2u * (unsigned)ctx->info.compute_units;  // (as for single calls)
+    fuse_tpw = (tiles + 2u * (unsigned)ctx->info.compute_units - 1) / (2u * (unsigned)ctx->info.compute_units);
+    if (!fuse_tpw) fuse_tpw = 1;
+    gfused = gfused && fuse_lds + 1024 <= 64 * 1024 && fuse_tpw <= 4;  // (as for single calls)
+    if (gfused) {  // workgroups take fuse_tpw consecutive tiles of one member: tile_begin counts workgroups
+      unsigned wgs = 0;
+      for (size_t i = 0; i < count; ++i) {
+        plans[i].pr.tile_begin = (int)wgs;
+        plans[i].pr.run_tiles = (int)fuse_tpw;
+        wgs += ((unsigned)plans[i].pr.n_tiles + fuse_tpw - 1) / fuse_tpw;
+      }
+      tiles = wgs;
+    }
   }
   tk_group *g = new (std::nothrow) tk_group();
   if (!g) return tk_fail(TK_ERR_BACKEND, "tk_group_create: host allocation failed");
@@ -2318,7 +2336,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max);
   if (gfused) {
     g->cfg.fused = 1;
-    g->cfg.lds_bytes += fuse_lds;
+    g->cfg.lds_bytes = fuse_lds;
   }
   ctx->refs.fetch_add(1);
   *out = g;

@@ -31,7 +31,7 @@
 
 // FUSED (one row tile, a single problem whose operand rows fit LDS in one pass): the kernel builds the operand rows
 // of its one to four tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of
-// two; the row constants sit in LDS behind the rows (and behind the reduction's buffer).
+// two; the row constants sit in LDS behind the rows.
 __device__ __forceinline__ void fused_stage_rows(const TkProblem &pr, uint4 *rows, uint8_t *cst);
 __device__ __forceinline__ RowConst row_const_from_lds(const uint8_t *cst, int mode, int R, int M, int rowbase);
 __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int rowbase, unsigned flag, const uint8_t *cst);
@@ -65,19 +65,75 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
   const uint4 *ap4 = (const uint4 *)pr.ap;
   uint4 *lds4 = (uint4 *)smem;
 
-  const size_t rows_bytes = (size_t)nb * 256 * R, red_bytes = (size_t)4 * P * RT * 1024;
-  uint8_t *const cst = smem + (rows_bytes > red_bytes ? rows_bytes : red_bytes);  // fused form only
+  if constexpr (FUSED) {
+    // The rows fit LDS in one pass (kc >= nb). A workgroup stages them once and then takes pr.run_tiles consecutive
+    // output tiles (its index counts workgroups, not tiles: tile_begin is in those units), so that launches of more
+    // than two tiles per CU do not repeat the tokens' prep in every tile; the reduction's buffer lies behind the rows,
+    // the row constants and the norm's scratch, which all stay in place for the next tile.
+    const size_t rows_bytes = (size_t)nb * 256 * R;
+    uint8_t *const cst = smem + rows_bytes;
+    v4i *const red = (v4i *)(cst + 1024 + (pr.norm_kind ? (size_t)pr.k * 4 + 1024 : 0));
+    fused_stage_rows(pr, lds4, cst);
+    const int tpw = pr.run_tiles > 0 ? pr.run_tiles : 1;
+    for (int tt = 0; tt < tpw; ++tt) {
+      const int tf = t * tpw + tt;
+      if (tf >= pr.n_tiles) break;  // (uniform over the workgroup)
+#pragma unroll
+      for (int p = 0; p < P; ++p) acc[p][0] = v4i{0, 0, 0, 0};
+      uint4 w[P], wn[P];
+      if (wave < nb) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) wn[p] = *(const uint4 *)(pr.codes[p] + (((size_t)tf * nb + wave) * 64 + lane) * 16);
+      }
+      for (int kbl = wave; kbl < nb; kbl += 4) {
+        const int kn = kbl + 4 < nb ? kbl + 4 : kbl;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          w[p] = wn[p];
+          wn[p] = *(const uint4 *)(pr.codes[p] + (((size_t)tf * nb + kn) * 64 + lane) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint4 q = make_uint4(0, 0, 0, 0);
+          if (i < R) q = lds4[((kbl * 4 + j) * 4 + g) * R + i];
+          const v4i a = v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
+#pragma unroll
+          for (int p = 0; p < P; ++p) {
+            const uint32_t wj = j == 0 ? w[p].x : (j == 1 ? w[p].y : (j == 2 ? w[p].z : w[p].w));
+            acc[p][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, expand_codes(wj), acc[p][0], 0, 0, 0);
+          }
+        }
+      }
+      __syncthreads();  // (the first wave has finished the previous tile's epilogue, which reads `red`)
+#pragma unroll
+      for (int p = 0; p < P; ++p) red[(wave * P + p) * 64 + lane] = acc[p][0];
+      __syncthreads();
+      const int n = tf * 16 + i;
+      if (wave == 0 && n < pr.n) {
+        const int rowbase = 4 * g;
+        v4i sum[P];
+        float sc[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          sum[p] = red[(0 * P + p) * 64 + lane];
+#pragma unroll
+          for (int w2 = 1; w2 < 4; ++w2) sum[p] += red[(w2 * P + p) * 64 + lane];
+          sc[p] = pr.scales[p][n];
+        }
+        const RowConst rc = row_const_from_lds(cst, pr.mode, R, pr.M, rowbase);
+        flow_epilogue<P>(pr, n, rowbase, sum, sc, rc);
+        if (rc.flag) exact_rows_fused(pr, n, rowbase, rc.flag, cst);
+      }
+    }
+    return;
+  }
   for (int kb0 = 0; kb0 < nb; kb0 += kc) {
     const int kcn = min(kc, nb - kb0);
-    if constexpr (FUSED) {  // (kc >= nb: one pass)
-      fused_stage_rows(pr, lds4, cst);
-    } else {
-      __syncthreads();
-      const int cnt = kcn * 16 * R;  // 16-byte pieces in this K chunk
-      const uint4 *src = ap4 + (size_t)kb0 * 16 * R;
-      for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4[idx] = src[idx];
-      __syncthreads();
-    }
+    __syncthreads();
+    const int cnt = kcn * 16 * R;  // 16-byte pieces in this K chunk
+    const uint4 *src = ap4 + (size_t)kb0 * 16 * R;
+    for (int idx = threadIdx.x; idx < cnt; idx += TK_WG) lds4[idx] = src[idx];
+    __syncthreads();
 
     // the chunk of the next trip is requested before this trip's arithmetic (the last trip asks for its own chunk
     // again: a cache hit), so that a wave's round trips to memory overlap with its matrix work
@@ -126,24 +182,6 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
   __syncthreads();
 
   const int n = t * 16 + i;
-  if constexpr (FUSED) {
-    if (wave == 0 && n < pr.n) {
-      const int rowbase = 4 * g;
-      v4i sum[P];
-      float sc[P];
-#pragma unroll
-      for (int p = 0; p < P; ++p) {
-        sum[p] = red[(0 * P + p) * 64 + lane];
-#pragma unroll
-        for (int w2 = 1; w2 < 4; ++w2) sum[p] += red[(w2 * P + p) * 64 + lane];
-        sc[p] = pr.scales[p][n];
-      }
-      const RowConst rc = row_const_from_lds(cst, pr.mode, R, pr.M, rowbase);
-      flow_epilogue<P>(pr, n, rowbase, sum, sc, rc);
-      if (rc.flag) exact_rows_fused(pr, n, rowbase, rc.flag, cst);
-    }
-    return;
-  }
   for (int rt = wave; rt < RT; rt += 4) {
     const int rowbase = rt * 16 + 4 * g;
     float out[4] = {0.f, 0.f, 0.f, 0.f};
