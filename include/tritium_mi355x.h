@@ -303,15 +303,18 @@ int tk_linear_float(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, i
 int tk_linear_a8(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
                  size_t m, void *out, int out_dtype);
 
-/* tk_linear_a8 for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same arguments,
- * same kernels and same bits as tk_linear_a8; the workspace of the call (operand rows, row sums,
- * per-token scales and flags) lives in a static device array of TK_NOALLOC_SCRATCH_BYTES that every
- * GPU the library runs on holds until the process ends, and the call makes no hipMalloc, hipFree or
- * other allocating call. A shape whose workspace does not fit (about (m + 16) * ceil(k/256) * 256
- * bytes: e.g. 64 tokens at k = 17408, or 2048 tokens at k = 3584) is answered with
- * TK_ERR_INVALID_INPUT. Every call on one GPU shares that GPU's array: calls that overlap on one GPU
- * (two contexts of a device, two threads) race and must be serialised by the caller. */
+/* tk_linear_a8 for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc, code that must not allocate while another thread captures a HIP graph). No counterpart in the
+ * reference. Same arguments and same bits as tk_linear_a8 (the same kernels, except that a narrow prefill
+ * launch which tk_linear_a8 would split over K runs unsplit here: the split needs a workspace that grows with
+ * the launch); the workspace of the call (operand rows, row sums, per-token scales and flags) lives in a
+ * static device array of TK_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process
+ * ends, and the call makes no hipMalloc, hipFree or other allocating call. The launches go to the context's
+ * own stream, as those of every other entry point do. The workspace takes about (m + 16) * ceil(k/256) * 256
+ * bytes: 64 tokens at k = 17408 (1.4 MB) and 2048 tokens at k = 3584 (7.4 MB) are about the largest shapes
+ * that fit; one that does not (e.g. 2048 tokens at k = 8192, 16.9 MB) is answered with TK_ERR_INVALID_INPUT.
+ * Every call on one GPU shares that GPU's array: calls that overlap on one GPU (two contexts of a device, two
+ * threads) race and must be serialised by the caller. */
 #define TK_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
 int tk_linear_a8_noalloc(tk_ctx *ctx, const tk_linear_desc *layer, const void *act, int act_dtype,
                          size_t m, void *out, int out_dtype);
@@ -537,6 +540,10 @@ int tk_set_host_direct_bytes(tk_ctx *ctx, size_t bytes);
 int tk_set_fuse_tokens(tk_ctx *ctx, int tokens);
 /* Calls of this context so far that ran in that single-launch form (for tests of the dispatch). */
 int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count);
+/* Name of the contraction kernel the last single call of this context (tk_linear_*, tk_mpgemm*) took:
+ * "flow", "flow32", "flow3", "stream", "ksplit_decode", "gemm64", "gemm64_ksplit", "gemm128", "gemm256";
+ * "" before the first call. A static string. For tests of the dispatch; no counterpart in the reference. */
+const char *tk_last_kernel(tk_ctx *ctx);
 /* Row count of the workgroup tile for single launches of one plane under the int8 contract (f32 or bf16
  * rows of whole 16-byte pieces at a 16-byte aligned address, no residual): 0 = chosen per launch, 64 = the
  * 64-row kernels, 128 = the 128 x 256 kernel, which shares both operands through LDS. Other launches take

@@ -112,3 +112,21 @@ amdhsa.kernels:
     bad = check_isa.check_budgets(meta, budgets)
     assert ("_Z4betaILi2EEvv", 169, 168) in bad and ("_Z5gammaILi3EEvv", 10100, 128) in bad and ("deltaILi4E", None, 64) in bad
     assert not any("alpha" in b[0] for b in bad) and len(bad) == 3
+
+
+def test_static_lds_rule():
+    """A listed kernel with static LDS in front of its dynamic array, and a listed kernel missing from the
+    assembly, are reported; one with an empty fixed segment is not."""
+    meta = """
+amdhsa.kernels:
+  - .agpr_count:     0
+    .group_segment_fixed_size: 0
+    .name:           _Z5alphaILi1EEvv
+    .vgpr_count:     100
+  - .agpr_count:     0
+    .group_segment_fixed_size: 144
+    .name:           _Z4betaILi2EEvv
+    .vgpr_count:     100
+"""
+    bad = check_isa.check_static_lds(meta, ("alpha", "beta", "gamma"))
+    assert bad == [("_Z4betaILi2EEvv", 144), ("gamma", None)]

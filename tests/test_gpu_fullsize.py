@@ -215,3 +215,64 @@ def test_config2_sweep_full_layer(backend, oracle, m):
         d.free()
         o.free()
     layer.free()
+
+
+def test_config3_prefill_bf16_automatic_kernel(backend, oracle):
+    """configs[2] exactly as the benchmark times it: 2048 bf16 tokens x 2560 -> 6912, one plane, W1.58A8,
+    bf16 out, one tk_linear_a8 call with the automatic kernel choice -- which must be one of the wide-tile
+    prefill kernels, not the 64-row form. Every output against the exact composition, sampled tokens of it
+    against the C oracle (crates/tritium-cuda/src/cuda/tests.rs:2100-2190 holds the reference's GPU GEMM to
+    its CPU backend the same way)."""
+    rng = np.random.default_rng(33)
+    m, n, k = 2048, 6912, 2560
+    w, sc = ternary(rng, n, k, 0.4), scales(rng, n)
+    packed = T.pack_rows(w, n, k)
+    layer = backend.linear([packed], [sc], n, k)
+    bits, act = _bf16(rng.standard_normal((m, k)).astype(np.float32))
+    dact, dout = backend.to_device(bits, "bf16"), backend.empty(m * n, "bf16")
+    print("case config3-bf16-auto", flush=True)
+    backend.linear_a8(layer, dact, m, dout)
+    took = backend.last_kernel()
+    assert took in ("gemm128", "gemm256"), took
+    want = a8_expected(oracle, [w], [sc], act)
+    assert (dout.to_host().reshape(m, n) == f32_to_bf16_bits(want).reshape(m, n)).all()
+    tok = [0, 1, 63, 64, 777, 1023, 1024, 2047]
+    rc, ref = oracle.cpu_mpgemm_with_act_quant(packed, FMT_TQ2_0, act[tok], sc, len(tok), n, k)
+    assert rc == 0 and same_bits(want[tok], ref)
+    # f32 out through the same kernel: the oracle's bits themselves
+    dout32 = backend.empty(m * n, "f32")
+    backend.linear_a8(layer, dact, m, dout32)
+    assert backend.last_kernel() == took
+    got32 = dout32.to_host().reshape(m, n)
+    assert same_bits(got32, want) and same_bits(got32[tok], ref)
+    for b in (dact, dout, dout32):
+        b.free()
+    layer.free()
+
+
+def test_config5_attention_projections_batch64_ksplit(backend, oracle):
+    """configs[4]'s attention projections as single 64-token calls: q / o 5120 x 5120 and k / v 1024 x 5120,
+    three planes (P(0)=0.4/0.7/0.85), bf16 in and out. 20 and 4 workgroups of the prefill kernel: the automatic
+    K split. Every output against the C oracle's plane composition."""
+    h, m = 5120, 64
+    rng = np.random.default_rng(55)
+    bits, act = _bf16(rng.standard_normal((m, h)).astype(np.float32))
+    dact = backend.to_device(bits, "bf16")
+    for name, n in (("q", 5120), ("k", 1024)):
+        print("case config5-attn", name, flush=True)
+        ws = [ternary(rng, n, h, p0) for p0 in (0.4, 0.7, 0.85)]
+        scs = [scales(rng, n) for _ in range(3)]
+        packed = [T.pack_rows(w, n, h) for w in ws]
+        layer = backend.linear(packed, scs, n, h)
+        o = backend.empty(m * n, "bf16")
+        backend.linear_a8(layer, dact, m, o)
+        assert backend.last_kernel() == "gemm64_ksplit", backend.last_kernel()
+        ref = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, h)
+        assert (o.to_host().reshape(m, n) == f32_to_bf16_bits(ref).reshape(m, n)).all()
+        o32 = backend.empty(m * n, "f32")
+        backend.linear_a8(layer, dact, m, o32)
+        assert same_bits(o32.to_host(), ref)
+        o.free()
+        o32.free()
+        layer.free()
+    dact.free()

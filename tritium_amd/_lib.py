@@ -142,6 +142,7 @@ SIGNATURES = {
     "tk_set_fuse_tokens": (C.c_int, [vp, C.c_int]),
     "tk_set_host_direct_bytes": (C.c_int, [vp, C.c_size_t]),
     "tk_get_fused_calls": (C.c_int, [vp, C.POINTER(C.c_ulonglong)]),
+    "tk_last_kernel": (C.c_char_p, [vp]),
     "tk_set_group_overlap": (C.c_int, [vp, C.c_int]),
     "tk_set_stream_min_groups": (C.c_int, [vp, C.c_int]),
     "tk_get_stream_min_groups": (C.c_int, [vp]),

@@ -602,6 +602,10 @@ class Mi355xBackend:
         _check(self._lib.tk_get_fused_calls(self._ctx, C.byref(c)))
         return int(c.value)
 
+    def last_kernel(self):
+        """Name of the contraction kernel the last single call took ("flow", "gemm64_ksplit", "gemm128", ...)."""
+        return self._lib.tk_last_kernel(self._ctx).decode()
+
     def set_gemm_rows(self, rows):
         """0 = automatic, 64 / 128 = rows of the workgroup tile for one-plane int8-contract prefill launches."""
         _check(self._lib.tk_set_gemm_rows(self._ctx, rows))

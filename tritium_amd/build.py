@@ -26,24 +26,25 @@ def hipcc():
     return "hipcc"
 
 
+# Translation units whose device assembly is emitted and checked before linking: in-flight registers of the
+# hand-issued loads (the prefill kernels), register budgets, and kernels that need an empty static LDS segment.
+ASM_SOURCES = ["tk_kernels.hip", "tk_gemm128.hip", "tk_base3.hip"]
+HAZARD_SOURCES = ["tk_kernels.hip"]
+
+
 def build_library(verbose=True):
     """Compile every translation unit and link the shared library. Always rebuilds. The device
-    assembly of the kernel file is produced alongside and checked (check_isa) before linking."""
+    assembly of the kernel files is produced alongside and checked (check_isa) before linking."""
     objs = []
     procs = []
-    asm_file = tempfile.NamedTemporaryFile(suffix=".s", delete=False)
-    asm_file.close()
-    asm_cmd = [hipcc(), *FLAGS, "--offload-device-only", "-S", "-x", "hip", os.path.join(CSRC, "tk_kernels.hip"),
-               "-o", asm_file.name]
-    if verbose:
-        print(" ".join(asm_cmd), flush=True)
-    asm_proc = subprocess.Popen(asm_cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    # (the 128-row prefill kernel has a register budget too; its file compiles in seconds)
-    asm128_file = tempfile.NamedTemporaryFile(suffix=".s", delete=False)
-    asm128_file.close()
-    asm128_proc = subprocess.Popen([hipcc(), *FLAGS, "--offload-device-only", "-S", "-x", "hip",
-                                    os.path.join(CSRC, "tk_gemm128.hip"), "-o", asm128_file.name],
-                                   stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    asm = []
+    for src in ASM_SOURCES:
+        f = tempfile.NamedTemporaryFile(suffix=".s", delete=False)
+        f.close()
+        cmd = [hipcc(), *FLAGS, "--offload-device-only", "-S", "-x", "hip", os.path.join(CSRC, src), "-o", f.name]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        asm.append((src, f.name, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     for src in SOURCES:
         obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
         cmd = [hipcc(), *FLAGS, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
@@ -59,32 +60,37 @@ def build_library(verbose=True):
         if out.strip() and (verbose or p.returncode):
             print(out, flush=True)
         failed |= p.returncode != 0
-    asm_out, _ = asm_proc.communicate()
     try:
-        if asm_proc.returncode:
-            print(asm_out, flush=True)
-            failed = True
+        texts = {}
+        for src, path, p in asm:
+            out, _ = p.communicate()
+            if p.returncode:
+                print(out, flush=True)
+                failed = True
+            else:
+                with open(path) as f:
+                    texts[src] = f.read()
         if failed:
             raise RuntimeError("hipcc failed")
         from . import check_isa
-        with open(asm_file.name) as f:
-            bad = check_isa.check_text(f.read())
-        if bad:
-            raise RuntimeError("generated code reads registers of loads still in flight:\n" + check_isa.report(bad))
-        asm128_out, _ = asm128_proc.communicate()
-        if asm128_proc.returncode:
-            print(asm128_out, flush=True)
-            raise RuntimeError("hipcc failed")
-        with open(asm_file.name) as f, open(asm128_file.name) as f128:
-            over = check_isa.check_budgets(f.read() + "\n" + f128.read())
+        for src in HAZARD_SOURCES:
+            bad = check_isa.check_text(texts[src])
+            if bad:
+                raise RuntimeError("generated code reads registers of loads still in flight:\n" + check_isa.report(bad))
+        everything = "\n".join(texts.values())
+        over = check_isa.check_budgets(everything)
         if over:
             raise RuntimeError("kernels over their register budget (kernel, registers [+10000 = spills], budget):\n" +
                                "\n".join(str(x) for x in over))
+        lds = check_isa.check_static_lds(everything)
+        if lds:
+            raise RuntimeError("kernels that address their dynamic LDS from 0 have static LDS in front of it "
+                               "(kernel, bytes; None = kernel not found):\n" + "\n".join(str(x) for x in lds))
     finally:
-        os.unlink(asm_file.name)
-        if asm128_proc.poll() is None:
-            asm128_proc.kill()
-        os.unlink(asm128_file.name)
+        for _, path, p in asm:
+            if p.poll() is None:
+                p.kill()
+            os.unlink(path)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -171,6 +171,36 @@ def check_budgets(text, budgets=REGISTER_BUDGETS):
     return bad
 
 
+# Kernels that build raw LDS addresses from offsets into their dynamic array and therefore need that array to
+# start at LDS address 0: no static LDS in front of it (the base-3 flow kernel's decode-table lookup is one
+# v_perm_b32 of the byte and the lane offset, with no add of a base).
+NO_STATIC_LDS = ("tk_flow3_kernel",)
+
+
+def check_static_lds(text, kernels=NO_STATIC_LDS):
+    """[(kernel, static LDS bytes)] for every listed kernel whose fixed LDS segment is not empty, and
+    (key, None) for a listed kernel the assembly does not contain."""
+    # one metadata entry per kernel ("  - .agpr_count: ..." starts it); its keys come in alphabetical order, so
+    # the fixed LDS size precedes the name
+    fixed, size = {}, None
+    for line in text.splitlines():
+        if re.match(r"\s+- \.\w+:", line):
+            size = None
+        m = re.match(r"[\s-]+\.group_segment_fixed_size:\s+(\d+)", line)
+        if m:
+            size = int(m.group(1))
+        m = re.match(r"[\s-]+\.name:\s+(\S+)", line)
+        if m and size is not None:
+            fixed[m.group(1)] = size
+    bad = []
+    for key in kernels:
+        names = [n for n in fixed if key in n]
+        if not names:
+            bad.append((key, None))
+        bad += [(n, fixed[n]) for n in names if fixed[n]]
+    return bad
+
+
 def report(found):
     out = []
     for name, hz in found.items():

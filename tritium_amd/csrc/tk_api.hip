@@ -85,6 +85,7 @@ struct tk_ctx {
   int gemm_two_by_two = 0;  // one-plane prefill kernel, 64 x 128 form: 0 = four waves side by side, 1 = two by two
   int gemm_ksplit = 0;     // prefill kernel, single launches: 0 = K slices chosen per launch, 1 = never split, n = n slices
   unsigned long long fused_calls = 0;  // calls that ran as one launch (tk_get_fused_calls)
+  const char *last_kernel = "";        // contraction kernel of the last single call (tk_last_kernel)
   // Host-slice calls (tk_mpgemm, tk_mpgemm_with_act_quant) of up to host_direct_bytes of operands go through this
   // pinned host block: a copy kernel reads the activation and the scales from it, the kernels write the output into
   // it -- no copy-engine transfers (see host_call; grow-only; freed with the context)
@@ -99,6 +100,7 @@ struct tk_ctx {
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum, kpart, kcount;
   int *d_invalid = nullptr;
+  bool kcount_stale = false;  // a K-split launch failed: its arrival counters are cleared before the next one
   // The context itself plus every weight buffer and group created on it: tk_destroy gives up the
   // context's own reference, the stream and this record live until the last of them is released, so
   // buffers and groups may be freed after tk_destroy.
@@ -275,6 +277,7 @@ extern "C" void tk_destroy(tk_ctx *ctx) {
     std::lock_guard<std::mutex> lk(ctx->mu);
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->stream2) (void)hipStreamSynchronize(ctx->stream2);
     DevBuf *bufs[] = {&ctx->ap, &ctx->rowsum, &ctx->fscale, &ctx->aux, &ctx->exps,
                       &ctx->flags, &ctx->h_act, &ctx->h_out, &ctx->h_scales, &ctx->tmp,
                       &ctx->ynorm, &ctx->blocksum, &ctx->kpart, &ctx->kcount};
@@ -387,6 +390,12 @@ extern "C" int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count) {
   std::lock_guard<std::mutex> lk(ctx->mu);
   *count = ctx->fused_calls;
   return TK_OK;
+}
+
+extern "C" const char *tk_last_kernel(tk_ctx *ctx) {
+  if (!ctx) return "";
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  return ctx->last_kernel;
 }
 
 extern "C" int tk_set_gemm_rows(tk_ctx *ctx, int rows) {
@@ -506,7 +515,7 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
   hipError_t e = hipMemsetAsync((uint8_t *)codes + code_bytes, 0x55, TK_CHUNK_BYTES, ctx->stream);
   if (e == hipSuccess && zmap) e = hipMemsetAsync(zmap, 0, map_words * 4, ctx->stream);
   if (e == hipSuccess && zmap) e = hipMemsetAsync(ctx->d_count, 0, sizeof(unsigned), ctx->stream);
-  if (packed_len) e = hipMemcpyAsync(raw, packed, packed_len, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess && packed_len) e = hipMemcpyAsync(raw, packed, packed_len, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) e = hipMemcpyAsync(ctx->d_invalid, &invalid, sizeof invalid, hipMemcpyHostToDevice, ctx->stream);
   if (e == hipSuccess) {
     if (format == TK_FORMAT_TQ2_0)
@@ -1156,6 +1165,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     }
     pr.run_tiles = run_tiles;
     pr.group_begin = 0;
+    ctx->last_kernel = b3 ? "flow3" : (wide ? "flow32" : "flow");
     if (b3) HIPCHK(tk_launch_flow3(ctx->stream, &pr, nullptr, nullptr, cfg));
     else HIPCHK(tk_launch_flow(ctx->stream, &pr, nullptr, nullptr, cfg));
   } else if (pl.skinny && variant == DECODE_STREAM) {
@@ -1164,6 +1174,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.lds_bytes = pl.stream_lds;
     pr.kc = pl.stream_kc;
     pr.group_begin = 0;
+    ctx->last_kernel = "stream";
     HIPCHK(tk_launch_stream(ctx->stream, &pr, nullptr, nullptr, cfg));
   } else if (pl.skinny) {
     if (fused) {
@@ -1173,6 +1184,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
       pl.cfg.grid = (pl.cfg.grid + (unsigned)pr.run_tiles - 1) / (unsigned)pr.run_tiles;
       ctx->fused_calls++;
     }
+    ctx->last_kernel = "ksplit_decode";
     HIPCHK(tk_launch_skinny(ctx->stream, &pr, nullptr, 0, pl.cfg));
   } else {
     // One plane under the int8 contract with whole 16-byte output pieces: the 128 x 256 kernel moves a third
@@ -1184,6 +1196,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     const bool want128 = ctx->gemm_rows == 128 || (ctx->gemm_rows == 0 && gemm128_pays(ctx, R, blocks128));
     if (can128 && want128) {
       plan_gemm128(&pl);
+      ctx->last_kernel = "gemm128";
       HIPCHK(tk_launch_gemm128(ctx->stream, &pr));
       return TK_OK;
     }
@@ -1210,13 +1223,19 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
       const bool fresh = tiles * 4 > ctx->kcount.cap;
       TKCHK(ensure(ctx, ctx->kpart, tiles * (size_t)ksn * regs * 256 * 4));
       TKCHK(ensure(ctx, ctx->kcount, tiles * 4));
-      if (fresh) HIPCHK(hipMemsetAsync(ctx->kcount.p, 0, ctx->kcount.cap, ctx->stream));  // the kernel leaves it zero
+      if (fresh || ctx->kcount_stale) HIPCHK(hipMemsetAsync(ctx->kcount.p, 0, ctx->kcount.cap, ctx->stream));  // the kernel leaves it zero
+      ctx->kcount_stale = false;
       pr.ksplit = ksn;
       pr.kpart = (int32_t *)ctx->kpart.p;
       pr.kcount = (int *)ctx->kcount.p;
     }
     pl.cfg.gemm_two_by_two = ctx->gemm_two_by_two;
-    HIPCHK(tk_launch_gemm(ctx->stream, &pr, nullptr, nullptr, pl.cfg));
+    ctx->last_kernel = ksn > 1 ? "gemm64_ksplit" : "gemm64";
+    const hipError_t le = tk_launch_gemm(ctx->stream, &pr, nullptr, nullptr, pl.cfg);
+    if (le != hipSuccess) {
+      if (ksn > 1) ctx->kcount_stale = true;  // counters of a launch that did not complete may be non-zero
+      return tk_fail(TK_ERR_BACKEND, "prefill kernel launch: %s", hipGetErrorString(le));
+    }
   }
   return TK_OK;
 }
@@ -2361,22 +2380,48 @@ extern "C" int tk_group_launch_parts(tk_ctx *ctx, tk_group *g, int do_prep, int 
   const bool both = do_main && g->has_flow_part && g->variant == DECODE_GEMM && g->cfg.grid > 0;
   bool forked = false;
   if (both && ctx->group_overlap) {
-    if (!ctx->stream2) {
-      HIPCHK(hipStreamCreateWithFlags(&ctx->stream2, hipStreamNonBlocking));
-      HIPCHK(hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming));
-      HIPCHK(hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming));
+    if (!ctx->stream2 || !ctx->ev_fork || !ctx->ev_join) {  // all three or none
+      hipStream_t s2 = nullptr;
+      hipEvent_t ef = nullptr, ej = nullptr;
+      hipError_t ce = hipStreamCreateWithFlags(&s2, hipStreamNonBlocking);
+      if (ce == hipSuccess) ce = hipEventCreateWithFlags(&ef, hipEventDisableTiming);
+      if (ce == hipSuccess) ce = hipEventCreateWithFlags(&ej, hipEventDisableTiming);
+      if (ce != hipSuccess) {
+        if (ej) (void)hipEventDestroy(ej);
+        if (ef) (void)hipEventDestroy(ef);
+        if (s2) (void)hipStreamDestroy(s2);
+        return tk_fail(TK_ERR_BACKEND, "second stream of the context: %s", hipGetErrorString(ce));
+      }
+      ctx->stream2 = s2;
+      ctx->ev_fork = ef;
+      ctx->ev_join = ej;
     }
     HIPCHK(hipEventRecord(ctx->ev_fork, ctx->stream));
     HIPCHK(hipStreamWaitEvent(ctx->stream2, ctx->ev_fork, 0));
-    HIPCHK(tk_launch_gemm(ctx->stream2, nullptr, probs, wg_prob, g->cfg));
-    HIPCHK(hipEventRecord(ctx->ev_join, ctx->stream2));
+    // From here on the second stream may hold work: whatever fails below, the first stream is ordered behind it
+    // before the call returns (join_error), so that nothing enqueued later, and no tk_sync, overtakes it.
+    hipError_t fe = tk_launch_gemm(ctx->stream2, nullptr, probs, wg_prob, g->cfg);
+    if (fe == hipSuccess) fe = hipEventRecord(ctx->ev_join, ctx->stream2);
+    if (fe != hipSuccess) {
+      (void)hipStreamSynchronize(ctx->stream2);
+      return tk_fail(TK_ERR_BACKEND, "grouped prefill launch on the second stream: %s", hipGetErrorString(fe));
+    }
     forked = true;
   }
-  if (do_main && g->has_flow_part)
-    HIPCHK(tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),
-                          g->flow_cfg));
-  if (forked)
-    HIPCHK(hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0));
+  if (do_main && g->has_flow_part) {
+    const hipError_t fe = tk_launch_flow(ctx->stream, nullptr, probs, (const int *)((const uint8_t *)g->tables + g->flow_wg_prob_off),
+                                         g->flow_cfg);
+    if (fe != hipSuccess) {
+      if (forked && hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0) != hipSuccess) (void)hipStreamSynchronize(ctx->stream2);
+      return tk_fail(TK_ERR_BACKEND, "grouped flow launch: %s", hipGetErrorString(fe));
+    }
+  }
+  if (forked) {
+    if (hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0) != hipSuccess) {
+      (void)hipStreamSynchronize(ctx->stream2);
+      return tk_fail(TK_ERR_BACKEND, "joining the second stream failed");
+    }
+  }
   else if (do_main && g->variant == DECODE_GEMM)
     HIPCHK(tk_launch_gemm(ctx->stream, nullptr, probs, wg_prob, g->cfg));
   else if (do_main && g->variant == DECODE_FLOW && g->cfg.base3)
@@ -2399,6 +2444,7 @@ extern "C" void tk_group_destroy(tk_group *g) {
     std::lock_guard<std::mutex> lk(ctx->mu);
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->stream2) (void)hipStreamSynchronize(ctx->stream2);
     if (g->ws) (void)hipFree(g->ws);
     if (g->tables) (void)hipFree(g->tables);
   }

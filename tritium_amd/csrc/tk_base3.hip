@@ -79,7 +79,8 @@ struct TkB3Piece {
 #define TK_LDS __attribute__((address_space(3)))
 
 // digits 1..4 of byte k of w, as four int8 codes: the table entry of that byte in this lane's bank
-// (the table starts at LDS address 0: the kernel has no static LDS in front of its dynamic array)
+// (the table starts at LDS address 0: the kernel has no static LDS in front of its dynamic array, which the
+// build verifies from the kernel's metadata: check_isa.NO_STATIC_LDS)
 __device__ __forceinline__ int b3_table(uint32_t w, uint32_t lane4, int k) {
   // v_perm_b32: selector bytes 0..3 pick from the second operand, 4..7 from the first, 0x0c is zero
   const uint32_t addr = __builtin_amdgcn_perm(w, lane4, 0x0C0C0400u | ((uint32_t)k << 8));

@@ -1545,11 +1545,22 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
         for (int c = 0; c < 16; ++c)
           __hip_atomic_store(mine + ((rt2 * NP + y) * 16 + c) * TK_GEMM_THREADS, acc[rt2][y][c], __ATOMIC_RELAXED,
                              __HIP_MEMORY_SCOPE_AGENT);
-    // The partial sums and the counter are accessed with device-scope (cache-coherent) stores, loads and
-    // atomics of their own, so no fence has to write back or invalidate a whole L2 (a device-scope
-    // fence per workgroup costs several times the kernel). Order: all of this workgroup's stores are
-    // acknowledged (vmcnt 0, every thread, then the barrier) before thread 0 counts the arrival; the
-    // last workgroup reads the others' sums only after it has seen every arrival.
+    // Hand-off between workgroups without a fence. What it relies on, instruction by instruction (gfx950 follows
+    // the gfx942 memory model of the LLVM AMDGPU backend):
+    //  * every access to the partial sums and to the counter is an agent-scope atomic, i.e. carries sc1: such a
+    //    store is written through the XCD's L2 to the memory side (where the XCDs' L2s meet), such a load never
+    //    hits a line another XCD made stale, and the counter's read-modify-write executes at that same level;
+    //  * vmcnt counts a store until it is acknowledged at the level its scope names, so `s_waitcnt vmcnt(0)` in
+    //    EVERY thread followed by the workgroup barrier means all 256 threads' partial sums are visible device-wide
+    //    before thread 0 issues the counter's increment -- the instruction pair a release at agent scope expands
+    //    to, minus its `buffer_wbl2 sc1` write-back of the whole L2, which only earlier NON-sc1 stores would need
+    //    (there are none whose values another workgroup reads);
+    //  * the workgroup that reads ksn-1 from the counter is by construction the last to arrive; its loads of the
+    //    others' sums are issued after the counter's value has come back (the value travels through LDS, a
+    //    barrier and a branch, and a wave issues in order), and being sc1 loads they need no `buffer_inv sc1`,
+    //    the other half of an acquire.
+    // A device-scope fence per workgroup was measured at several times the kernel; the forced-slice tests cover
+    // the result, tests/test_ksplit_protocol.py the counting protocol over every interleaving of arrivals.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     int *arrived = (int *)smem;  // the A slots are free after the main loop's last barrier
