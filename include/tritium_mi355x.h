@@ -546,9 +546,15 @@ int tk_get_fused_calls(tk_ctx *ctx, unsigned long long *count);
 const char *tk_last_kernel(tk_ctx *ctx);
 /* Row count of the workgroup tile for single launches of one plane under the int8 contract (f32 or bf16
  * rows of whole 16-byte pieces at a 16-byte aligned address, no residual): 0 = chosen per launch, 64 = the
- * 64-row kernels, 128 = the 128 x 256 kernel, which shares both operands through LDS. Other launches take
- * the 64-row kernels whatever this says. A tuning and test knob: identical bits. */
+ * 64-row kernels, 128 = the 128 x 256 kernel, which shares both operands through LDS, 256 = the 256-row kernel,
+ * which expands the weight tile to int8 once per workgroup, in LDS. Other launches take the 64-row kernels
+ * whatever this says. A tuning and test knob: identical bits. */
 int tk_set_gemm_rows(tk_ctx *ctx, int rows);
+/* Form of the 256-row kernel: 0 = four waves of 64 rows over a column block of 224 outputs, one workgroup per CU; 1 =
+ * eight waves of 32 rows; 2 = four waves over a part of the column block (128 or 96 outputs), two workgroups per CU;
+ * -1 (the state of a new context) = form 1, the one the automatic dispatch uses (for launches of 0.7 .. 1 workgroups per
+ * CU). A measurement and test knob: identical bits. */
+int tk_set_gemm256_form(tk_ctx *ctx, int form);
 /* A grouped launch whose members partly fit LDS runs two kernels (the flow kernel for those that fit, the prefill
  * kernel for the others). on != 0 (default): side by side on two streams of the context, joined before
  * anything enqueued later; 0: one after the other. A measurement knob: identical results. */

@@ -26,6 +26,7 @@ def automatic_dispatch(backend):
     backend.set_gemm_tiles(0)
     backend.set_gemm_two_by_two(False)
     backend.set_gemm_rows(0)
+    backend.set_gemm256_form(-1)
     backend.set_stream_min_groups(backend.info.compute_units)
 
 
@@ -123,6 +124,53 @@ def test_prefill_kernel_128_rows(backend, oracle, m, n, k):
     backend.linear_i8(layer, dq, None, m, do)
     assert same_bits(do.to_host().reshape(m, n), acc * scs[0][None, :])
     for a in (dact, dq, dsc, do):
+        a.free()
+    layer.free()
+
+
+@pytest.mark.parametrize("form", [0, 1, 2])
+@pytest.mark.parametrize("m,n,k", [(65, 8, 256), (257, 232, 512), (300, 456, 300), (256, 1040, 2560), (520, 2104, 768),
+                                   (1030, 4104, 256), (640, 520, 1280), (700, 240, 4096)])
+def test_prefill_kernel_256_rows(backend, oracle, m, n, k, form):
+    """tk_gemm256_kernel (the weight tile expanded to int8 once per workgroup, in LDS) forced at small sizes, in its three
+    forms (four waves of 64 rows, eight waves of 32, and column blocks split over two workgroups): partial row blocks and column blocks (224 outputs each), one and
+    several K blocks (odd and even counts: both LDS buffers end a launch), a ragged K, one to several workgroups per
+    XCD; f32 and bf16 outputs from float rows (with an all-zero token and two tokens that hold NaN / Inf and take
+    the reference-order path) and from int8 rows; against the CPU oracle, bit for bit."""
+    print("case gemm-256", m, n, k, form, flush=True)
+    rng = np.random.default_rng(256000 + m + n + k)
+    ws, scs, packed = _planes(rng, n, k, 1)
+    layer = backend.linear(packed, scs, n, k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[m // 2] = 0.0
+    act[1, k // 3] = np.nan
+    act[m - 1, 0] = np.inf
+    dact = backend.to_device(act, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    nan = np.isnan(want)
+    backend.set_gemm_rows(256)
+    backend.set_gemm256_form(form)
+    dout = backend.empty(m * n, "f32")
+    backend.linear_a8(layer, dact, m, dout)
+    assert backend.last_kernel() == "gemm256"
+    got = dout.to_host().reshape(m, n)
+    assert (np.isnan(got) == nan).all()
+    assert same_bits(got[~nan], want[~nan])
+    dob = backend.empty(m * n, "bf16")
+    backend.linear_a8(layer, dact, m, dob)
+    gb = dob.to_host().reshape(m, n)
+    assert (gb[~nan] == f32_to_bf16_bits(want)[~nan]).all()
+    # int8 rows in, with and without per-token scales
+    q = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    asc = rng.uniform(0.01, 0.2, m).astype(np.float32)
+    dq, dsc, do = backend.to_device(q, "i8"), backend.to_device(asc, "f32"), backend.empty(m * n, "f32")
+    acc = oracle.int8_accumulators(packed[0], FMT_TQ2_0, q, m, n, k).astype(np.float32)
+    backend.linear_i8(layer, dq, dsc, m, do)
+    assert backend.last_kernel() == "gemm256"
+    assert same_bits(do.to_host().reshape(m, n), (acc * scs[0][None, :]) * asc[:, None])
+    backend.linear_i8(layer, dq, None, m, do)
+    assert same_bits(do.to_host().reshape(m, n), acc * scs[0][None, :])
+    for a in (dact, dout, dob, dq, dsc, do):
         a.free()
     layer.free()
 

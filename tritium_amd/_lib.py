@@ -139,6 +139,7 @@ SIGNATURES = {
     "tk_set_gemm_tiles": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_ksplit": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_rows": (C.c_int, [vp, C.c_int]),
+    "tk_set_gemm256_form": (C.c_int, [vp, C.c_int]),
     "tk_set_fuse_tokens": (C.c_int, [vp, C.c_int]),
     "tk_set_host_direct_bytes": (C.c_int, [vp, C.c_size_t]),
     "tk_get_fused_calls": (C.c_int, [vp, C.POINTER(C.c_ulonglong)]),

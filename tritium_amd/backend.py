@@ -607,8 +607,13 @@ class Mi355xBackend:
         return self._lib.tk_last_kernel(self._ctx).decode()
 
     def set_gemm_rows(self, rows):
-        """0 = automatic, 64 / 128 = rows of the workgroup tile for one-plane int8-contract prefill launches."""
+        """0 = automatic, 64 / 128 / 256 = rows of the workgroup tile for one-plane int8-contract prefill launches."""
         _check(self._lib.tk_set_gemm_rows(self._ctx, rows))
+
+    def set_gemm256_form(self, form):
+        """The 256-row prefill kernel: 0 = 4 waves x 224 outputs, 1 = 8 waves x 224, 2 = 4 waves x (128 | 96) outputs with
+        two workgroups per CU, -1 = chosen per launch (same bits)."""
+        _check(self._lib.tk_set_gemm256_form(self._ctx, form))
 
     def set_gemm_ksplit(self, slices):
         """0 automatic, 1 off, 2..64 K slices of the prefill kernel in single launches."""

@@ -143,6 +143,9 @@ REGISTER_BUDGETS = (
     ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
     ("tk_gemm32_kernelILi3ELi2ELb0ELb0E", 256),     # prefill, three planes (two waves per SIMD)
     ("tk_gemm128_kernel", 128),                     # prefill, 128 x 256 form (four waves per SIMD)
+    ("tk_gemm256_kernelILi0E", 512),                # prefill, 256 x 224 form, four waves (one per SIMD)
+    ("tk_gemm256_kernelILi1E", 256),                # ... eight waves (two per SIMD)
+    ("tk_gemm256_kernelILi2E", 256),                # ... four waves over 128 | 96 outputs, two workgroups per CU
 )
 
 

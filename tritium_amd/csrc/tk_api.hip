@@ -93,10 +93,13 @@ struct tk_ctx {
   size_t pin_cap = 0;
   size_t host_direct_bytes = (size_t)1 << 20;
   int fuse_tokens = -1;    // single decode calls of up to this many tokens build their operand rows inside the decode kernel (-1 = chosen per call, 0 = never)
-  int gemm_rows = 0;       // one-plane int8-contract prefill, single launches: 0 = tile rows chosen per launch, 64 / 128 = force
+  int gemm_rows = 0;       // one-plane int8-contract prefill, single launches: 0 = tile rows chosen per launch, 64 / 128 / 256 = force
+  bool gemm256_form_forced = false;  // tk_set_gemm256_form was called: automatic launches keep that form
+  int gemm256_form = 0;    // the 256-row kernel: 0 = 4 waves x 224 outputs, 1 = 8 waves x 224, 2 = 4 waves x (128 | 96), two workgroups per CU
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
   int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
   unsigned *d_count = nullptr;  // a device counter for the uploads
+
   uint8_t *static_scratch = nullptr;  // this device's copy of `scratch` (below), resolved at tk_init
   DevBuf ap, rowsum, fscale, aux, exps, flags, h_act, h_out, h_scales, tmp, ynorm, blocksum, kpart, kcount;
   int *d_invalid = nullptr;
@@ -400,9 +403,19 @@ extern "C" const char *tk_last_kernel(tk_ctx *ctx) {
 
 extern "C" int tk_set_gemm_rows(tk_ctx *ctx, int rows) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm_rows: null context");
-  if (rows != 0 && rows != 64 && rows != 128) return tk_fail(TK_ERR_INVALID_INPUT, "gemm_rows=%d - use 0 (automatic), 64 or 128", rows);
+  if (rows != 0 && rows != 64 && rows != 128 && rows != 256)
+    return tk_fail(TK_ERR_INVALID_INPUT, "gemm_rows=%d - use 0 (automatic), 64, 128 or 256", rows);
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->gemm_rows = rows;
+  return TK_OK;
+}
+
+extern "C" int tk_set_gemm256_form(tk_ctx *ctx, int form) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_gemm256_form: null context");
+  if (form < -1 || form > 2) return tk_fail(TK_ERR_INVALID_INPUT, "gemm256_form=%d - use -1 (chosen per launch), 0, 1 or 2", form);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->gemm256_form = form < 0 ? 0 : form;
+  ctx->gemm256_form_forced = form >= 0;
   return TK_OK;
 }
 
@@ -883,6 +896,32 @@ static void plan_gemm128(Plan *pl) {
   }
 }
 
+// The 256 x 224 kernel's grid: row blocks of 256 operand rows, column blocks of 14 tiles, split over the XCDs
+// (the operand-row stride plan_gemm chose stays). An XCD reads, per unit of K, 256 bytes of operand rows per row
+// block it owns and 56 bytes of codes per column block.
+static void plan_gemm256(Plan *pl) {
+  TkProblem &pr = pl->pr;
+  pl->grid_m = (unsigned)(((size_t)pr.R + 255) / 256);
+  pl->grid_n = ((unsigned)pr.n_tiles + 13u) / 14u;
+  pr.grid_m = (int)pl->grid_m;
+  pr.grid_n = (int)pl->grid_n;
+  pr.ksplit = 0;
+  size_t best = (size_t)-1;
+  for (int xr = 1; xr <= 8; xr *= 2) {
+    const int xc = 8 / xr;
+    const int sm = ((int)pl->grid_m + xr - 1) / xr, sn = ((int)pl->grid_n + xc - 1) / xc;
+    const size_t cost = (size_t)256 * sm + (size_t)56 * sn;
+    const size_t waste = (size_t)8 * sm * sn;
+    const size_t score = cost * 1024 + waste;
+    if (score < best) {
+      best = score;
+      pr.xr = xr;
+      pr.sub_m = sm;
+      pr.sub_n = sn;
+    }
+  }
+}
+
 // Where the 128 x 256 kernel is chosen over the 64-row forms: launches it finishes in one round of its 512
 // resident workgroups (two per CU) and that still give most CUs one. A/B on one box, int8 rows in, bf16 out,
 // call incl. the operand re-ordering launch, 64-row kernels -> 128 x 256: 2048 x 2560 -> 6912 (432 blocks)
@@ -893,6 +932,21 @@ static void plan_gemm128(Plan *pl) {
 static bool gemm128_pays(const tk_ctx *ctx, size_t rows, size_t blocks128) {
   const size_t cus = (size_t)ctx->info.compute_units;
   return rows >= 1024 && blocks128 * 4 >= cus * 3 && blocks128 <= 2 * cus;
+}
+
+// Where the 256-row kernel (weight tile expanded once per workgroup) is chosen: launches of 1024 rows or more that give
+// 0.7 .. 1 workgroups per CU, as eight waves of 32 rows over whole 224-output column blocks. A/B on one box, bf16 rows
+// in and out, call incl. quantization, best of the 64-row / 128-row kernels -> this form: 2048 x 2560 -> 6912 (248
+// blocks) 45.6 -> 41.6 us; 1536 x 2560 -> 6912 (186) 40.4 -> 38.9; 2048 x 5120 -> 5120 (184) 62.6 -> 59.8; 4096 x 2560 ->
+// 2560 (192) 42.2 -> 40.8. Outside that window it loses -- one workgroup per CU leaves every round's prologue and
+// epilogue in the open: 1024 x 2048 -> 8192 (148 blocks) 26.7 -> 31.2; 3072 x 2560 -> 6912 (372) 61.8 -> 64.5; 4096 x 17408
+// -> 5120 320 -> 360 -- and the form with two workgroups per CU over 128 | 96 outputs is within 1-2% of the 64-row
+// kernels either way (e.g. 4096 x 5120 -> 17408 282 -> 276, 1024 x 2048 -> 8192 26.7 -> 30.9): not chosen by itself.
+static bool gemm256_pays(const tk_ctx *ctx, size_t rows, size_t n_tiles, int *form) {
+  const size_t cus = (size_t)ctx->info.compute_units;
+  const size_t blocks = ((rows + 255) / 256) * ((n_tiles + 13) / 14);
+  *form = ctx->gemm256_form_forced ? ctx->gemm256_form : 1;
+  return rows >= 1024 && blocks <= cus && blocks * 10 >= cus * 7;
 }
 
 static void plan_shape(tk_ctx *ctx, const tk_linear_desc *layer, size_t n, size_t k, size_t m, int mode,
@@ -1096,6 +1150,14 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   const bool fused_ksplit = fuse_rows && variant == DECODE_KSPLIT && (size_t)pl.pr.kc >= nb && fused_ksplit_lds + 1024 <= 64 * 1024 &&
                             fuse_tpw <= 4;
   const bool fused = fused_flow || fused_ksplit;
+  // One plane under the int8 contract with whole 16-byte output pieces: the wide-tile prefill kernels.
+  const size_t out_esz = out_dtype == TK_BF16 ? 2 : 4;
+  const bool can_wide = !pl.skinny && pl.pr.planes == 1 && mode == TK_MODE_INT8 && (out_dtype == TK_F32 || out_dtype == TK_BF16) &&
+                        !residual && (n * out_esz) % 16 == 0 && ((uintptr_t)out & 15) == 0;
+  int form256 = 0;
+  const bool pays256 = gemm256_pays(ctx, R, (size_t)pl.pr.n_tiles, &form256);
+  const bool use256 = can_wide && (ctx->gemm_rows == 256 || (ctx->gemm_rows == 0 && pays256));
+  if (use256) plan_gemm256(&pl);
   Workspace ws;
   TKCHK(take_workspace(ctx, static_ws, (size_t)pl.pr.rs * nb * 256, R, m, norm ? m * k * 4 : 0, &ws));
 
@@ -1189,9 +1251,15 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   } else {
     // One plane under the int8 contract with whole 16-byte output pieces: the 128 x 256 kernel moves a third
     // of the bytes per op through the CU's memory path (both operands shared through LDS).
-    const size_t esz = out_dtype == TK_BF16 ? 2 : 4;
-    const bool can128 = pr.planes == 1 && mode == TK_MODE_INT8 && (out_dtype == TK_F32 || out_dtype == TK_BF16) && !residual &&
-                        (n * esz) % 16 == 0 && ((uintptr_t)out & 15) == 0;
+    const bool can128 = can_wide;
+    if (use256) {
+      ctx->last_kernel = "gemm256";
+      const hipError_t le = tk_launch_gemm256(ctx->stream, &pr, form256);
+      if (le != hipSuccess) {
+        return tk_fail(TK_ERR_BACKEND, "prefill kernel launch: %s", hipGetErrorString(le));
+      }
+      return TK_OK;
+    }
     const size_t blocks128 = ((R + 127) / 128) * (((size_t)pr.n_tiles + 15) / 16);
     const bool want128 = ctx->gemm_rows == 128 || (ctx->gemm_rows == 0 && gemm128_pays(ctx, R, blocks128));
     if (can128 && want128) {

@@ -186,6 +186,12 @@ hipError_t tk_launch_gemm(hipStream_t s, const TkProblem *single, const TkProble
 // no residual; grid from the problem's XCD split over 128-row x 16-tile blocks
 int tk_gemm128_lds_bytes(void);
 hipError_t tk_launch_gemm128(hipStream_t s, const TkProblem *single);
+// 256 x 224 prefill kernel (tk_gemm256.hip): the same launches as the 128 x 256 kernel; the weight tile is expanded to
+// int8 once per workgroup, in LDS. form 0: four waves of 64 rows over the whole column block (224 outputs); 1: eight
+// waves of 32 rows; 2: four waves over a part of the column block (128 or 96 outputs), two workgroups per CU. Grid from
+// the problem's XCD split over 256-row x 14-tile blocks.
+int tk_gemm256_lds_bytes(int form);
+hipError_t tk_launch_gemm256(hipStream_t s, const TkProblem *single, int form);
 hipError_t tk_launch_seq(hipStream_t s, const TkProblem *single);
 // The three gradients of one packed mpGEMM (tk_vjp.hip); a null output is skipped.
 hipError_t tk_launch_projected_vjp(hipStream_t s, const uint8_t *codes, size_t nb, size_t n, size_t k, size_t m,

@@ -2047,19 +2047,6 @@ __device__ void row_absmax(const void *act, int dtype, size_t base, size_t k, bo
   nonfinite = nf != 0;
 }
 
-// A thread of the prep kernels builds whole 16-byte pieces of the operand layout. Piece q of K block
-// kb (q = c*8 + h*4 + j, lane group g = 2c + h) holds the elements kb*256 + c*128 + s*32 + h*16 + j*4
-// + b for s, b = 0..3: consecutive q walk 32 consecutive elements for each s, so the four loads of
-// a wave are contiguous runs.
-__device__ __forceinline__ size_t piece_elem0(size_t kb, int q) {
-  const int c = q >> 3, h = (q >> 2) & 1, j = q & 3;
-  return kb * 256 + (size_t)c * 128 + (size_t)h * 16 + (size_t)j * 4;
-}
-__device__ __forceinline__ size_t piece_offset(size_t kb, int q, size_t R, size_t row) {
-  const int c = q >> 3, h = (q >> 2) & 1, j = q & 3, g = c * 2 + h;
-  return (((kb * 4 + j) * 4 + g) * R + row) * 16;
-}
-
 // uniform_m > 0: every tensor of the table has that many tokens, so the entry follows from the
 // workgroup index without the chain of dependent loads the search costs.
 __device__ __forceinline__ const TkPrep &find_prep(const TkPrep &single, const TkPrep *table, int nprep, int uniform_m,
@@ -2475,36 +2462,10 @@ __device__ __forceinline__ const TkPrep &find_prep_wave(const TkPrep &single, co
   return table[lo];
 }
 
-__device__ __forceinline__ int wave_sum(int v) {
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
-}
-
 // FAST != 0: the launch's rows are whole K blocks (k a multiple of 256), 16-byte aligned, of one element type
 // (1 = f32, 2 = bf16) and only the operand rows are wanted: no bound, alignment or type is tested per
 // element, which is most of what the general form executes (a wave works through its token alone, one
 // dependent instruction after the other: the instruction count is the launch's time).
-template <int FAST>
-__device__ __forceinline__ void load_piece_fast(const void *act, size_t base, size_t e0, float (&v)[16]) {
-#pragma unroll
-  for (int sl = 0; sl < 4; ++sl) {
-    if constexpr (FAST == 2) {
-      typedef unsigned v2u __attribute__((ext_vector_type(2)));
-      const v2u u = *(const TK_GLOBAL v2u *)((const uint16_t *)act + base + e0 + sl * 32);
-      v[sl * 4 + 0] = __uint_as_float(u.x << 16);
-      v[sl * 4 + 1] = __uint_as_float(u.x & 0xFFFF0000u);
-      v[sl * 4 + 2] = __uint_as_float(u.y << 16);
-      v[sl * 4 + 3] = __uint_as_float(u.y & 0xFFFF0000u);
-    } else {
-      const v4u u = *(const TK_GLOBAL v4u *)((const float *)act + base + e0 + sl * 32);
-      v[sl * 4 + 0] = __uint_as_float(u.x);
-      v[sl * 4 + 1] = __uint_as_float(u.y);
-      v[sl * 4 + 2] = __uint_as_float(u.z);
-      v[sl * 4 + 3] = __uint_as_float(u.w);
-    }
-  }
-}
-
 template <int HELD, int FAST = 0, int TEAM = 64>
 __device__ __forceinline__ void wave_absmax_held(const void *act, int dtype, size_t base, size_t k, size_t npieces, bool vec,
                                                  int lane, float (&held)[HELD][16], float &gamma, int &nonfinite,
