@@ -237,6 +237,7 @@ def bench_prefill(T, be, rng, m, k, n, planes=1, iters=100):
     verified = check_a8(f"prefill M={m} K={k} N={n}", out.to_host().reshape(m, n)[tok], hostw[1][0], hostw[1][1],
                         bf16_to_f32(abits).reshape(m, k)[tok], "bf16")
     ms = time_calls(be, lambda i: be.linear_a8(layers[i % 2], act, m, out), iters)
+    kernel = be.last_kernel()
     # the contraction alone: the same call on already-quantized int8 rows (their re-ordering launch stays in)
     q = be.to_device(rng.integers(-127, 128, (m, k)).astype(np.int8), "i8")
     qs = be.to_device(rng.uniform(0.01, 0.05, m).astype(np.float32), "f32")
@@ -248,7 +249,7 @@ def bench_prefill(T, be, rng, m, k, n, planes=1, iters=100):
         x.free()
     return {"workload": f"prefill GEMM M={m} K={k} N={n} {planes} plane(s), bf16 act -> int8 per token -> int32 acc -> bf16",
             "ms_per_call_incl_quant": round(ms, 4), "TOPS": round(ops / ms / 1e9, 1),
-            "frac_of_int8_peak": round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4),
+            "frac_of_int8_peak": round(ops / ms / 1e9 / INT8_PEAK_TOPS, 4), "kernel": kernel,
             "int8_input_call": {"ms_per_call": round(ms_i8, 4), "TOPS": round(ops / ms_i8 / 1e9, 1),
                                 "frac_of_int8_peak": round(ops / ms_i8 / 1e9 / INT8_PEAK_TOPS, 4),
                                 "note": "activations already int8 (no absmax pass; the operand re-ordering launch included)"},
@@ -746,7 +747,7 @@ def cpu_baseline(rng):
         bits = f32_to_bf16_bits(rng.standard_normal((m, K2)).astype(np.float32))
         acts.append((bits.astype(np.uint32) << 16).view(np.float32).reshape(m, K2))
     t0 = time.perf_counter()
-    while passes < 60 and time.perf_counter() - t0 < 12.0:  # a bounded sample: about 12 s of CPU work
+    while passes < 60 and time.perf_counter() - t0 < 9.0:  # a bounded sample: about 9 s of CPU work
         for m, act in zip(SWEEP, acts):
             out = None
             for p in range(PLANES2):
@@ -756,10 +757,94 @@ def cpu_baseline(rng):
             total_bytes += algorithmic_bytes(m, N2, K2, PLANES2, 2, 4)
         passes += 1
     dt = time.perf_counter() - t0
-    return {"value": round(total_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": used_max, "kind": "port",
-            "sample": f"{passes} passes of the sweep (batch {','.join(map(str, SWEEP))}) over ONE layer copy, "
-                      f"{dt:.1f} s; C restatement of tritium-cpu (unpack per call, AVX-512 k-order f32 fold, rows "
-                      f"chunked over threads: batch 1 gets a single worker, batch 16 gets {used_max})"}
+    res = {"value": round(total_bytes / dt / 1e9, 4), "unit": "GB/s", "cores": used_max, "kind": "port",
+           "sample": f"{passes} passes of the sweep (batch {','.join(map(str, SWEEP))}) over ONE layer copy, "
+                     f"{dt:.1f} s; C restatement of tritium-cpu (unpack per call, AVX-512 k-order f32 fold, rows "
+                     f"chunked over threads: batch 1 gets a single worker, batch 16 gets {used_max})"}
+    kernels = {0: "scalar", 1: "AVX2 f32 fold", 2: "AVX-512 f32 fold", 3: "AVX2 maddubs int8", 4: "AVX-VNNI dpbusd int8"}
+    # configs[2]: what TernaryLinear::forward asks of tritium-cpu -- tokens quantized per token to int8 values, then
+    # mpgemm, whose dispatch takes the integer kernel for such activations (crates/tritium-cpu/src/kernel.rs:577-664)
+    m, k, n = 2048, 2560, 6912
+    packed = orc.pack_matrix(ternary(rng, n, k, 0.4), n, k, oracle_lib.FMT_TQ2_0)
+    sc = rng.uniform(0.01, 0.1, n).astype(np.float32)
+    bits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    act = (bits.astype(np.uint32) << 16).view(np.float32).reshape(m, k)
+    t0 = time.perf_counter()
+    calls, used, kern = 0, 0, 0
+    while calls < 20 and time.perf_counter() - t0 < 6.0:
+        q, _ = orc.quantize_act_int8(act, m, k)
+        _, used, kern = orc.cpu_mpgemm_fast(packed, oracle_lib.FMT_TQ2_0, np.ascontiguousarray(q, np.float32), sc, m, n, k, threads)
+        calls += 1
+    dt = time.perf_counter() - t0
+    res["prefill_gemm"] = {"value": round(2.0 * m * n * k * calls / dt / 1e12, 4), "unit": "TOPS", "cores": used,
+                           "kind": "port", "kernel": kernels.get(kern, str(kern)),
+                           "sample": f"{calls} whole calls of M={m} K={k} N={n} (quantization, unpack and contraction), {dt:.1f} s"}
+    # configs[3], batch 1: one token through q,k,v,o,gate,up,down of a layer; M = 1 gives the reference a single worker
+    h, f, kv, sample_layers = 2560, 6912, 640, 2
+    shapes = [(h, h), (kv, h), (kv, h), (h, h), (f, h), (f, h), (h, f)]
+    layer = [(orc.pack_matrix(ternary(rng, nn, kk, 0.4), nn, kk, oracle_lib.FMT_TQ2_0), rng.uniform(0.01, 0.1, nn).astype(np.float32),
+              nn, kk) for nn, kk in shapes]
+    toks = {kk: np.ascontiguousarray(orc.quantize_act_int8(rng.standard_normal((1, kk)).astype(np.float32), 1, kk)[0], np.float32)
+            for kk in (h, f)}
+    t0 = time.perf_counter()
+    done = 0
+    while done < sample_layers or (time.perf_counter() - t0 < 4.0 and done < 30):
+        for pk, scl, nn, kk in layer:
+            _, used, kern = orc.cpu_mpgemm_fast(pk, oracle_lib.FMT_TQ2_0, toks[kk], scl, 1, nn, kk, threads)
+        done += 1
+    dt = time.perf_counter() - t0
+    res["projection_stack_batch1"] = {"value": round(done / dt / 30.0, 3), "unit": "tokens/s", "cores": used, "kind": "port",
+                                      "kernel": kernels.get(kern, str(kern)),
+                                      "sample": f"{done} of the 30 layers' seven projections (tokens already int8-valued), {dt:.1f} s; "
+                                                f"tokens/s = layers per second / 30"}
+    return res
+
+
+def summarize(out):
+    """The five configurations in a few lines, as the LAST key of the record (a reader that keeps only the end of the
+    line still has every headline figure): value, unit, fraction of the roofline that bounds it, kernel."""
+    ex = out.get("extra", {})
+    s = {"config2_decode_sweep_bf16": {"value": out["value"], "unit": "GB/s", "kernel_frac_of_hbm_peak": out["roofline"]["frac"],
+                                       "kernel": "tk_flow_kernel / tk_flow32_kernel"}}
+    c1 = ex.get("config1_f32_batch1")
+    if c1:
+        s["config1_batch1_f32"] = {"value": c1["step_GB/s_incl_digit_split"], "unit": "GB/s", "frac_of_hbm_peak": c1["step_frac_of_hbm_peak"],
+                                   "kernel_frac_of_hbm_peak": c1["kernel_frac_of_hbm_peak"], "kernel": "tk_flow_kernel<1,1,1,4>"}
+    a8 = ex.get("decode_sweep_int8_activations")
+    if a8:
+        s["config2_decode_sweep_int8_contract"] = {"value": a8["step_sweep_GB/s_incl_quant"], "unit": "GB/s",
+                                                   "frac_of_hbm_peak": a8["step_frac_of_hbm_peak"],
+                                                   "kernel_frac_of_hbm_peak": a8["kernel_frac_of_hbm_peak"]}
+    pf = ex.get("prefill_gemm")
+    if pf:
+        s["config3_prefill"] = {"value": pf["TOPS"], "unit": "TOPS", "frac_of_int8_peak": pf["frac_of_int8_peak"],
+                                "us_per_call_incl_quant": round(pf["ms_per_call_incl_quant"] * 1e3, 1), "kernel": pf.get("kernel")}
+    st = ex.get("projection_stack")
+    if st:
+        s["config4_stack"] = {b: {"value": st[b]["tokens_per_s"], "unit": "tokens/s", "frac_of_hbm_peak": st[b]["frac_of_hbm_peak"]}
+                              for b in ("batch1", "batch32") if b in st}
+        for b in ("batch1", "batch32"):
+            key = f"{b}_layer_by_layer"
+            if key in st:
+                s["config4_stack"][key] = {"value": st[key]["tokens_per_s"], "unit": "tokens/s"}
+    c5 = ex.get("config5_three_planes")
+    if c5:
+        d = c5["decode_batch64"]
+        s["config5"] = {"decode_batch64": {"value": d["GB/s"], "unit": "GB/s", "frac_of_hbm_peak": d["frac_of_hbm_peak"],
+                                           "TOPS": d["kernels_only"]["TOPS"], "tokens_per_s": d["tokens_per_s"]}}
+        for leg in ("prefill_4096_up", "prefill_4096_down"):
+            if leg in c5:
+                s["config5"][leg] = {"value": c5[leg]["TOPS"], "unit": "TOPS", "frac_of_int8_peak": c5[leg]["frac_of_int8_peak"]}
+    cpu = out.get("cpu_baseline")
+    if cpu:
+        s["cpu_port"] = {"decode_sweep_GB/s": cpu["value"], "cores": cpu["cores"]}
+        if "prefill_gemm" in cpu:
+            s["cpu_port"]["prefill_TOPS"] = cpu["prefill_gemm"]["value"]
+            s["cpu_port"]["prefill_cores"] = cpu["prefill_gemm"]["cores"]
+        if "projection_stack_batch1" in cpu:
+            s["cpu_port"]["stack_batch1_tokens_per_s"] = cpu["projection_stack_batch1"]["value"]
+            s["cpu_port"]["stack_batch1_cores"] = cpu["projection_stack_batch1"]["cores"]
+    return s
 
 
 def main():
@@ -837,6 +922,7 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np.random.default_rng(1))
     be.close()
+    out["summary"] = summarize(out)
     print(json.dumps(out))
 
 
