@@ -785,8 +785,13 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
 // rows at 8 (16x, eight-wave workgroups, one per CU). Re-measured with the ring at 4 positions: 4-8
 // operand rows (8-16 KiB staged) are 5-8% faster with runs of ONE tile (64 KiB per workgroup), 16
 // rows stay at 2.
+// Re-measured with the weight stream read through non-temporal loads (same shape; sweep of run length x ring size): one
+// row tile of two or more TOKENS now peaks at 2 tiles per run -- float contract 2 / 4 tokens 5.85 -> 6.33 / 5.58 -> 5.95
+// TB/s, int8 contract 4 / 8 / 16 tokens 5.44 -> 6.16 / 4.99 -> 5.92 / 5.35 -> 5.76 -- and a single token stays at one
+// (6.45 / 6.66 TB/s; 6.52 / 6.55 with two): what separates the two is the output a run writes when it ends. Tiles of
+// less than 16 KiB of codes (one plane, K = 2560) take two per run at every token count (one int8 token 6.03 -> 6.47).
 static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, int rt, int waves, size_t lds_bytes,
-                          size_t nb, bool wide, bool b3, size_t rows) {
+                          size_t nb, bool wide, bool b3, size_t rows, size_t tokens) {
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * (b3 ? TK_B3_CHUNK_BYTES : TK_CHUNK_BYTES);
@@ -794,6 +799,7 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   if (target < 64 * 1024) target = 64 * 1024;
   size_t s = 1;
   while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
+  if (!wide && !b3 && rt == 1 && s < 2 && (tokens >= 2 || tile_bytes < 16 * 1024)) s = 2;
   // keep every CU supplied: two four-wave workgroups each, or one eight-wave workgroup (those fill
   // the LDS of a CU alone, and a single round of them has no change-over in the middle of the launch)
   const unsigned per_cu = waves >= 8 ? 1u : 2u;
@@ -1079,7 +1085,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
     if (b3) flow_lds += TK_B3_TABLE_BYTES;
     const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds);
-    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R);
+    run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R, m);
     const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
     // (an eight-wave workgroup of the flow kernel fills a CU alone: it counts as two. 17408 x 5120 x 3 planes, 16 / 24 /
@@ -2120,10 +2126,11 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     if (plans[i].flow_lds > flds) flds = plans[i].flow_lds;
     flow_ok = flow_ok && plans[i].flow_ok;
   }
-  size_t nb_max = 1, rows_max = 1;
+  size_t nb_max = 1, rows_max = 1, tokens_max = 1;
   for (size_t i = 0; i < count; ++i) {
     if ((size_t)plans[i].pr.nb > nb_max) nb_max = plans[i].pr.nb;
     if ((size_t)plans[i].pr.R > rows_max) rows_max = plans[i].pr.R;
+    if ((size_t)plans[i].pr.M > tokens_max) tokens_max = plans[i].pr.M;
   }
   bool b3 = flow_ok;
   for (size_t i = 0; i < count && b3; ++i) b3 = flow_base3(plans[i].pr, planes, rt, flds);
@@ -2131,7 +2138,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   if (wide) flds = flow_wide_lds(rt, nb_max);
   if (b3) flds += TK_B3_TABLE_BYTES;
   const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds);
-  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, b3, rows_max);
+  int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, b3, rows_max, tokens_max);
   {
     std::vector<unsigned> member_tiles(count);
     for (size_t i = 0; i < count; ++i) member_tiles[i] = (unsigned)plans[i].pr.n_tiles;
@@ -2201,7 +2208,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds);
-    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max) : 1;
+    int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max, tokens_max) : 1;
     {
       std::vector<unsigned> member_tiles;
       for (size_t i = 0; i < count; ++i)

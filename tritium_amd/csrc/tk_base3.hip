@@ -143,11 +143,18 @@ __global__ __launch_bounds__(TK_B3_WAVES * 64) void tk_flow3_kernel(const TkProb
 #pragma unroll
       for (int p = 0; p < P; ++p) {
         const uint8_t *base = codes[p] + (size_t)off;
+        // (non-temporal, like the 2-bit stream: every byte is read once per launch)
+#if TK_STREAM_NT
+        const tk_v3u d = __builtin_nontemporal_load((const TK_GLOBAL tk_v3u_a4 *)(base + lane12));
+        const uint8_t hb = __builtin_nontemporal_load((const TK_GLOBAL uint8_t *)(base + lane_h));
+#else
         const tk_v3u d = *(const TK_GLOBAL tk_v3u_a4 *)(base + lane12);
+        const uint8_t hb = *(const TK_GLOBAL uint8_t *)(base + lane_h);
+#endif
         ring[slot][tw][p].q[0] = d.x;
         ring[slot][tw][p].q[1] = d.y;
         ring[slot][tw][p].q[2] = d.z;
-        ring[slot][tw][p].h = (uint32_t) * (const TK_GLOBAL uint8_t *)(base + lane_h);
+        ring[slot][tw][p].h = (uint32_t)hb;
       }
       roff[tw] += real ? CB : 0u;
     }

@@ -56,6 +56,20 @@ __device__ __forceinline__ uint4 gload16(const void *p) {
   const v4u v = *(const TK_GLOBAL v4u *)p;
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+// The same load for bytes that are read once per launch (the weight stream of the decode kernels): the non-temporal
+// bit. A plain read probe on one MI355X streams 6.1-6.4 TB/s with ordinary 16-byte loads and 6.9-7.15 TB/s with the
+// bit set, whatever the run length and the number of loads in flight (sc0 / sc1 alone change nothing).
+#ifndef TK_STREAM_NT
+#define TK_STREAM_NT 1
+#endif
+__device__ __forceinline__ uint4 gload16_stream(const void *p) {
+#if TK_STREAM_NT
+  const v4u v = __builtin_nontemporal_load((const TK_GLOBAL v4u *)p);
+#else
+  const v4u v = *(const TK_GLOBAL v4u *)p;
+#endif
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 __device__ __forceinline__ float load_act(const void *p, int dtype, size_t idx) {
   return dtype == TK_BF16 ? bf16_to_f32(gload((const uint16_t *)p + idx)) : gload((const float *)p + idx);

@@ -141,14 +141,14 @@ __global__ __launch_bounds__(TK_WG) void tk_skinny_kernel(TkProblem single, cons
     if (wave < kcn) {
 #pragma unroll
       for (int p = 0; p < P; ++p)
-        wn[p] = *(const uint4 *)(pr.codes[p] + (((size_t)t * nb + kb0 + wave) * 64 + lane) * 16);
+        wn[p] = gload16(pr.codes[p] + (((size_t)t * nb + kb0 + wave) * 64 + lane) * 16);
     }
     for (int kbl = wave; kbl < kcn; kbl += 4) {
       const int kn = kbl + 4 < kcn ? kbl + 4 : kbl;
 #pragma unroll
       for (int p = 0; p < P; ++p) {
         w[p] = wn[p];
-        wn[p] = *(const uint4 *)(pr.codes[p] + (((size_t)t * nb + kb0 + kn) * 64 + lane) * 16);
+        wn[p] = gload16(pr.codes[p] + (((size_t)t * nb + kb0 + kn) * 64 + lane) * 16);
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -414,7 +414,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
           }
           if ((word >> (chunk & 31u)) & 1u) o = zero_off;
         }
-        ring[slot][tw][p] = gload16(codes[p] + (size_t)o);
+        ring[slot][tw][p] = gload16_stream(codes[p] + (size_t)o);
       }
       roff[tw] += real ? 1024u : 0u;
     }
@@ -645,7 +645,7 @@ __global__ __launch_bounds__(512) void tk_salt_flow_kernel(const TkProblem singl
     const unsigned off = min(roff, last_off);
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      ring[slot][p] = gload16(codes[p] + (size_t)off);
+      ring[slot][p] = gload16_stream(codes[p] + (size_t)off);
       ring_s[slot][p] = gload(bscale[p] + (size_t)(off >> 10) * 16 + i);  // chunk index * 16 + column
     }
     roff += real ? 1024u : 0u;
@@ -805,8 +805,8 @@ __global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, 
     const unsigned off = min(roff, last_off);
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      ring[slot][p][0] = gload16(codes[p] + (size_t)off);
-      ring[slot][p][1] = gload16(codes[p] + (size_t)off + 512);
+      ring[slot][p][0] = gload16_stream(codes[p] + (size_t)off);
+      ring[slot][p][1] = gload16_stream(codes[p] + (size_t)off + 512);
     }
     roff += real ? 1024u : 0u;
   };
@@ -1436,12 +1436,22 @@ tk_gemm32_kernel(const TkProblem single, const TkProblem *__restrict__ table, co
 #pragma unroll
     for (int rt2 = 0; rt2 < RT2W; ++rt2) asm volatile("" : "+v"(a[rt2]));
   };
+  // Grouped launches (decode batches: one row block per member) and K-split launches (few workgroups) read every weight
+  // byte once: their loads carry the non-temporal bit, like the decode kernels' weight stream. A prefill launch reads a
+  // chunk again in every row block and leaves it to the caches. (Chosen per instantiation: a branch around two forms
+  // of the load would put both into the instruction stream the build's in-flight check walks.)
+  constexpr bool W_ONCE = TABLE || KSPLIT;
   auto load_w = [&](v4i (&w)[NP][2], int kb) {
 #pragma unroll
     for (int y = 0; y < NP; ++y) {
       const uint8_t *ptr = wptr[y] + (size_t)kb * TK_CHUNK_BYTES;
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(w[y][0]) : "v"(ptr));
-      asm volatile("global_load_dwordx4 %0, %1, off offset:512" : "=v"(w[y][1]) : "v"(ptr));
+      if constexpr (W_ONCE) {
+        asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(w[y][0]) : "v"(ptr));
+        asm volatile("global_load_dwordx4 %0, %1, off offset:512 nt" : "=v"(w[y][1]) : "v"(ptr));
+      } else {
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(w[y][0]) : "v"(ptr));
+        asm volatile("global_load_dwordx4 %0, %1, off offset:512" : "=v"(w[y][1]) : "v"(ptr));
+      }
     }
   };
   auto tie_w = [&](v4i (&w)[NP][2]) {
@@ -3482,12 +3492,14 @@ int tk_flow32_runs_per_wave(void) { return 2; }
 // row tiles) of the positions, weighted by each problem's chunk count; if all do, the one that
 // pads least.
 int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int rows, int tw) {
-  // one row tile: 4 positions with runs of one tile (up to 8 rows), 5 with runs of two (9..16 rows)
-  const int pref1a[4] = {4, 5, 3, 2}, pref1b[4] = {5, 4, 3, 2}, pref2[4] = {4, 5, 3, 2}, pref4[4] = {2, 3, 4, 5};
-  const int *pref1 = rows <= 8 ? pref1a : pref1b;  // (one plane with two runs per wave: 4 positions at every row count; see the caller)
-  // one row tile with two runs per wave: 4 positions measured best even where they pad K (K = 2560, ten
-  // blocks: 4 positions 97.9 us, 3: 98.6, 5: 99.1; 16 int8 rows: 128.5 / 131 / 130.5)
-  const double limit = (rt == 1 && tw < 2) ? 0.10 : 0.25;
+  // one row tile: 4 positions, and 2 where 4 would pad the K block count by more than a tenth. Re-measured with the
+  // weight stream on non-temporal loads, 128 layer copies per launch: ten K blocks (K = 2560, one plane) on 2 positions
+  // against 4 padded to 12 -- 6912 outputs, one f32 token 5.90 -> 6.27 TB/s, 4 / 16 int8 tokens 5.31 -> 5.61 / 4.96 ->
+  // 5.16; 2560 outputs 5.55 -> 6.12, 5.29 -> 5.68, 4.61 -> 4.90 -- and 5 positions, the choice before, lose 5-14% to 2;
+  // eight K blocks are within 1.5% either way (two planes, K = 2048: 2 positions +2.6% for one float token, -1% for two).
+  const int pref1a[4] = {4, 2, 3, 5}, pref1b[4] = {5, 4, 3, 2}, pref2[4] = {4, 2, 3, 5}, pref4[4] = {2, 3, 4, 5};
+  const int *pref1 = rows <= 8 ? pref1a : pref1b;  // (one plane with two runs per wave: the first list at every row count; see the caller)
+  const double limit = rt == 1 ? 0.10 : 0.25;
   const int *cand = rt == 1 ? (tw >= 2 ? pref2 : pref1) : (rt == 2 ? pref2 : pref4);
   int best = cand[0];
   double best_waste = -1.0;
