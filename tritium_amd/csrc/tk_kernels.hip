@@ -3499,7 +3499,9 @@ int tk_flow_ring(const int *nbs, const double *weights, int count, int rt, int r
   // eight K blocks are within 1.5% either way (two planes, K = 2048: 2 positions +2.6% for one float token, -1% for two).
   const int pref1a[4] = {4, 2, 3, 5}, pref1b[4] = {5, 4, 3, 2}, pref2[4] = {4, 2, 3, 5}, pref4[4] = {2, 3, 4, 5};
   const int *pref1 = rows <= 8 ? pref1a : pref1b;  // (one plane with two runs per wave: the first list at every row count; see the caller)
-  const double limit = rt == 1 ? 0.10 : 0.25;
+  // two row tiles likewise: 32 int8 rows, K = 2560, one plane, 2 positions against 4 padded to 12: 6912 outputs 4.16 ->
+  // 4.35 TB/s, 2560 outputs 3.91 -> 4.35, 640 outputs 2.31 -> 3.17
+  const double limit = rt <= 2 ? 0.10 : 0.25;
   const int *cand = rt == 1 ? (tw >= 2 ? pref2 : pref1) : (rt == 2 ? pref2 : pref4);
   int best = cand[0];
   double best_waste = -1.0;
