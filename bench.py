@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel (sweep average), from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration against a 1 GiB copy kernel):
 # profiles/decode_flow_c2_sweep_traffic.txt
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_142_447_431
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_180_451_472
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 FP32_PEAK_TFLOPS = 157.3  # MI355X fp32, published
 
@@ -430,12 +430,13 @@ def bench_config5(T, be, rng):
 
 
 def bench_zero_skip(T, be, rng, iters=60):
-    """Zero-chunk skip on the headline shape (two planes, K=2048, N=8192, W1.58A8, batch 1 and 4, 128 layer
-    copies per launch). Plane 2 has P(0)=0.85 in two forms: block-structured (75% of its 16-row x 256-trit
-    chunks all zero, the rest i.i.d. with P(0)=0.4) and i.i.d. Each is timed with the map the upload keeps
-    by the 0.5% rule and with maps disabled; for the i.i.d. plane also with a map forced on (it has no
-    zero chunk: the rule keeps none, so the default costs nothing). GB/s are the dense algorithmic bytes
-    over time, so a skip shows as a figure above what the memory could deliver for the full planes."""
+    """Zero-chunk skip on the headline shape (two planes, K=2048, N=8192, W1.58A8, batch 1, 4, 16, 32 and 64, 128
+    layer copies per launch). Plane 2 has P(0)=0.85 in two forms: block-structured (75% of its 16-row x
+    256-trit chunks all zero, the rest i.i.d. with P(0)=0.4) and i.i.d. Each is timed with the map the upload
+    keeps by the 0.5% rule and with maps disabled; for the i.i.d. plane also with a map forced on (it has no
+    zero chunk: the rule keeps none, so the default costs nothing). Batch 32 takes the 32x32x32 form of the
+    kernel, the others the 16x16x64 form. GB/s are the dense algorithmic bytes over time, so a skip shows as a
+    figure above what the memory could deliver for the full planes."""
     nt, nb = N2 // 16, K2 // 256
     p1 = ternary(rng, N2, K2, 0.4)
     structured = ternary(rng, N2, K2, 0.4)
@@ -447,8 +448,9 @@ def bench_zero_skip(T, be, rng, iters=60):
                        f"W1.58A8, {COPIES} layer copies per launch, decode kernel alone",
            "zero_fraction_of_plane2": {"structured": round(float((structured == 0).mean()), 3), "iid": round(float((iid == 0).mean()), 3)}}
     packed1 = T.pack_rows(p1, N2, K2)
-    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((4, K2)).astype(np.float32)), "bf16") for _ in range(COPIES)]
-    outs = [be.empty(4 * N2, "f32") for _ in range(COPIES)]
+    batches = (1, 4, 16, 32, 64)
+    acts = [be.to_device(f32_to_bf16_bits(rng.standard_normal((max(batches), K2)).astype(np.float32)), "bf16") for _ in range(COPIES)]
+    outs = [be.empty(max(batches) * N2, "f32") for _ in range(COPIES)]
     ref_out = {}
     for name, plane2, modes in (("structured", structured, (0, 1)), ("iid", iid, (0, 1, 2))):
         packed2 = T.pack_rows(plane2, N2, K2)
@@ -458,7 +460,7 @@ def bench_zero_skip(T, be, rng, iters=60):
             kept = layers[0].planes[1].zero_chunks()
             tag = f"{name}_{('by_rule', 'maps_off', 'map_forced')[mode]}"
             res[tag] = {"plane2_zero_chunks": kept[0], "chunks": kept[1], "map_kept": kept[2]}
-            for m in (1, 4):
+            for m in batches:
                 g = be.group([(layers[i], acts[i], m, outs[i]) for i in range(COPIES)], 1, "bf16", "f32")
                 g.launch()
                 be.sync()

@@ -111,3 +111,59 @@ def test_bits_identical_with_and_without_the_map(backend, oracle, m, planes, run
         a.free()
     with_map.free()
     without.free()
+
+
+@pytest.mark.parametrize("m", [5, 8, 20, 28, 32, 48, 64])
+@pytest.mark.parametrize("planes", [1, 2])
+@pytest.mark.parametrize("mfma", [0, 32])
+def test_the_32x32x32_form_consults_the_maps_too(backend, oracle, m, planes, mfma):
+    """The 32x32x32 form of the flow kernel (automatic at 25..32 operand rows, forced here beyond) with mapped
+    planes, single launches and groups: the bits of the unmapped planes and of the CPU. A wave of that form walks a
+    pair of tiles, so pairs with one marked chunk, with both and with none all occur."""
+    print("case zero-skip 32x32x32", m, planes, mfma, flush=True)
+    rng = np.random.default_rng(7000 + m * 100 + planes * 10 + mfma)
+    n, k = 16 * 37 + 5, 256 * 7 - 13  # (an odd tile count: the last pair has one tile)
+    ws = [structured(rng, n, k, pz, p0)[0] for pz, p0 in ((0.5, 0.4), (0.75, 0.7))[:planes]]
+    ws[-1][16:48, :] = 0  # a pair of tiles whose every chunk is marked
+    ws[-1][-5:, :256] = 0
+    ws[-1][-21:-5, :256] = 0  # ... and the first chunks of the last two tiles
+    scs = [scales(rng, n) for _ in range(planes)]
+    packed = [T.pack_rows(w, n, k) for w in ws]
+    backend.set_zero_skip(2)
+    with_map = backend.linear(packed, scs, n, k)
+    backend.set_zero_skip(1)
+    without = backend.linear(packed, scs, n, k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    bits = f32_to_bf16_bits(act)
+    actb = bf16_bits_to_f32(bits).reshape(m, k)
+    dact = backend.to_device(bits, "bf16")
+    o = [backend.empty(m * n, "f32") for _ in range(2)]
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, actb, m, n, k)
+    backend.set_flow_mfma(mfma)
+    try:
+        backend.linear_a8(with_map, dact, m, o[0])
+        took = backend.last_kernel()
+        backend.linear_a8(without, dact, m, o[1])
+        if mfma == 32 and m > 16 or 24 < m <= 32:
+            assert took == "flow32", (took, m, planes, mfma)
+        assert same_bits(o[0].to_host(), want) and same_bits(o[1].to_host(), want)
+        if m <= 16:
+            backend.linear_float(with_map, dact, m, o[0])
+            tookf = backend.last_kernel()
+            backend.linear_float(without, dact, m, o[1])
+            if mfma == 32 or m == 8:
+                assert tookf == "flow32", (tookf, m, planes, mfma)
+            assert same_bits(o[0].to_host(), o[1].to_host())
+            wantf = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, actb, m, n, k)
+            assert accepts(o[0].to_host().reshape(m, n), wantf, rel=1e-4, floor=1.0).all()
+        # a group of a mapped and an unmapped member through the table forms
+        grp = backend.group([(with_map, dact, m, o[0]), (without, dact, m, o[1])], 1, "bf16", "f32")
+        grp.launch()
+        assert same_bits(o[0].to_host(), want) and same_bits(o[1].to_host(), want)
+        grp.destroy()
+    finally:
+        backend.set_flow_mfma(0)
+    for a in [dact] + o:
+        a.free()
+    with_map.free()
+    without.free()

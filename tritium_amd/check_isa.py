@@ -137,7 +137,7 @@ REGISTER_BUDGETS = (
     ("tk_flow_kernelILi1ELi1ELi2ELi4ELb1E", 128),   # one plane, two runs per wave: 2..16 rows
     ("tk_flow_kernelILi2ELi1ELi1ELi4ELb1E", 128),   # two planes, up to 8 rows
     ("tk_flow_kernelILi2ELi1ELi2ELi4ELb1E", 168),   # two planes, 9..16 rows
-    ("tk_flow32_kernelILi2ELi1ELi4ELb1E", 168),     # two planes, 25..32 rows
+    ("tk_flow32_kernelILi2ELi1ELi4ELb1ELb0E", 168),     # two planes, 25..32 rows
     ("tk_flow_kernelILi2ELi4ELi2ELi2ELb1E", 256),   # two planes, 33..64 rows
     ("tk_gemm32_kernelILi1ELi2ELb0ELb0E", 168),     # prefill, one plane (three waves per SIMD by design)
     ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
@@ -146,6 +146,8 @@ REGISTER_BUDGETS = (
     ("tk_gemm256_kernelILi0E", 512),                # prefill, 256 x 224 form, four waves (one per SIMD)
     ("tk_gemm256_kernelILi1E", 256),                # ... eight waves (two per SIMD)
     ("tk_gemm256_kernelILi2E", 256),                # ... four waves over 128 | 96 outputs, two workgroups per CU
+) + tuple(  # the 32x32x32 flow forms that consult the zero-chunk maps (last argument true): present, no spills
+    (f"tk_flow32_kernelILi{p}ELi{rt2}ELi{dr}ELb{t}ELb1E", 256) for p in (1, 2) for rt2 in (1, 2) for dr in (2, 3, 4) for t in (0, 1)
 )
 
 

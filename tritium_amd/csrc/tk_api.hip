@@ -511,7 +511,7 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
   const size_t map_words = (n_chunks + 31) / 32;
   void *codes = nullptr, *raw = nullptr, *bscales = nullptr, *zmap = nullptr, *codes3 = nullptr;
   const bool want3 = n_chunks && !keep_block_scales && (ctx->base3 == 2 || (ctx->base3 == 1 && format == TK_FORMAT_TQ1_0));
-  TKCHK(dev_malloc(code_bytes + TK_CHUNK_BYTES, &codes));  // + the resident all-zero chunk
+  TKCHK(dev_malloc(code_bytes + TK_ZERO_CHUNKS * TK_CHUNK_BYTES, &codes));  // + the resident all-zero chunks
   int rc = dev_malloc(packed_len, &raw);
   if (!rc && want3) rc = dev_malloc(n_chunks * TK_B3_CHUNK_BYTES, &codes3);
   if (!rc && keep_block_scales) rc = dev_malloc(n_tiles * nb * 16 * sizeof(float), &bscales);
@@ -525,7 +525,7 @@ static int upload_weights(tk_ctx *ctx, const uint8_t *packed, size_t packed_len,
   }
   int invalid = INT32_MAX;
   unsigned zero_chunks = 0;
-  hipError_t e = hipMemsetAsync((uint8_t *)codes + code_bytes, 0x55, TK_CHUNK_BYTES, ctx->stream);
+  hipError_t e = hipMemsetAsync((uint8_t *)codes + code_bytes, 0x55, TK_ZERO_CHUNKS * TK_CHUNK_BYTES, ctx->stream);
   if (e == hipSuccess && zmap) e = hipMemsetAsync(zmap, 0, map_words * 4, ctx->stream);
   if (e == hipSuccess && zmap) e = hipMemsetAsync(ctx->d_count, 0, sizeof(unsigned), ctx->stream);
   if (e == hipSuccess && packed_len) e = hipMemcpyAsync(raw, packed, packed_len, hipMemcpyHostToDevice, ctx->stream);
@@ -763,8 +763,15 @@ static bool flow_base3(const TkProblem &pr, int planes, int rt, size_t rows_lds)
     if (!pr.codes3[p]) return false;
   return true;
 }
-// zmap_tiles > 0: some plane of the launch carries a zero-chunk map; a workgroup of that many tiles stages
-// the words of its chunks behind the operand rows (16x16x64 form only; the other kernels ignore the maps)
+// Room for the zero-chunk maps of a flow launch: the tiles per workgroup whose map words are staged behind the operand
+// rows (behind the row constants in the 32x32x32 form), or 0 when they do not fit or the form ignores the maps
+// (base-3 stream; the fused single-launch form keeps its row constants there) -- plain loads then.
+static size_t flow_zero_plan(bool wide, bool b3, bool fused, int planes, size_t flow_lds, size_t tiles_per_wg, size_t nb) {
+  if (b3 || fused || !tiles_per_wg) return 0;
+  const size_t words = (size_t)planes * tk_flow_zmap_words(tiles_per_wg, nb) * 4;
+  return flow_lds + (wide ? kFlowWideExtraLds : 0) + words <= kLdsFlowMax ? tiles_per_wg : 0;
+}
+// zmap_tiles > 0: some plane of the launch carries a zero-chunk map (flow_zero_plan)
 // (b3: flow_lds includes the decode table; ring and runs per wave are the base-3 kernel's own)
 static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds, size_t rows, size_t zmap_tiles = 0,
                           size_t zmap_nb = 0) {
@@ -773,8 +780,9 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
   if (b3) cfg->ring = 4;
   cfg->tw = flow_runs_per_wave(wide, b3, cfg->planes, cfg->rt, rows);
   cfg->lds_bytes = flow_lds + (wide ? kFlowWideExtraLds : 0);
-  if (!wide && zmap_tiles) cfg->lds_bytes += (size_t)cfg->planes * tk_flow_zmap_words(zmap_tiles, zmap_nb) * 4;
+  if (zmap_tiles) cfg->lds_bytes += (size_t)cfg->planes * tk_flow_zmap_words(zmap_tiles, zmap_nb) * 4;
   if (wide && cfg->ring > 4) cfg->ring = 4;
+  cfg->zmap32 = wide && zmap_tiles ? 1 : 0;
 }
 
 // Consecutive tiles per run of the flow kernel. A workgroup pays for staging its operand rows
@@ -1221,9 +1229,8 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.lds_bytes = flow_lds;
     cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds);
     cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R));
-    size_t ztiles = pr.zskip && !wide && !b3 ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0;
-    if (ztiles && flow_lds + (size_t)cfg.planes * tk_flow_zmap_words(ztiles, nb) * 4 > kLdsFlowMax) ztiles = 0;
-    if (fused) ztiles = 0;      // the row constants take the maps' place behind the rows
+    const size_t ztiles = flow_zero_plan(wide, b3, fused, cfg.planes, flow_lds,
+                                         pr.zskip ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0, nb);
     if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or another form of the kernel): plain loads
     flow_cfg_form(&cfg, wide, b3, flow_lds, R, ztiles, nb);
     if (fused) {
@@ -2246,8 +2253,8 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, false, planes, rt, prows_max));
       size_t ztiles = 0;
       for (size_t i = 0; i < count; ++i)
-        if (plans[i].flow_ok && plans[i].pr.zskip && !pwide) ztiles = pper;
-      if (ztiles && pflds + (size_t)planes * tk_flow_zmap_words(ztiles, pnb_max) * 4 > kLdsFlowMax) ztiles = 0;
+        if (plans[i].flow_ok && plans[i].pr.zskip) ztiles = pper;
+      ztiles = flow_zero_plan(pwide, false, false, planes, pflds, ztiles, pnb_max);
       if (!ztiles)
         for (size_t i = 0; i < count; ++i)
           if (plans[i].flow_ok) plans[i].pr.zskip = 0;
@@ -2272,8 +2279,8 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   size_t group_ztiles = 0;
   if (variant == DECODE_FLOW) {
     for (size_t i = 0; i < count; ++i)
-      if (plans[i].pr.zskip && !wide && !b3) group_ztiles = fper;
-    if (group_ztiles && flds + (size_t)planes * tk_flow_zmap_words(group_ztiles, nb_max) * 4 > kLdsFlowMax) group_ztiles = 0;
+      if (plans[i].pr.zskip) group_ztiles = fper;
+    group_ztiles = flow_zero_plan(wide, b3, false, planes, flds, group_ztiles, nb_max);
     if (!group_ztiles)
       for (size_t i = 0; i < count; ++i) plans[i].pr.zskip = 0;
   }

@@ -16,6 +16,13 @@
 // Rows past n are filled with 0x55 (all-zero trits). Block scales are dropped.
 #define TK_TILE_ROWS 16
 #define TK_CHUNK_BYTES 1024
+// all-zero chunks kept behind a plane's last chunk (a power of two): a request for a chunk the zero-chunk map marks
+// reads copy (chunk index mod this). One copy: spreading the redirected requests over 16 copies (in case they crowded
+// a cache channel) measured 2-6% slower on a plane with 75% marked chunks (two planes K=2048 N=8192, 1 / 4 / 16 int8
+// tokens: 151 / 148 / 164 -> 155 / 152 / 174 us per 128 layers).
+#ifndef TK_ZERO_CHUNKS
+#define TK_ZERO_CHUNKS 1
+#endif
 
 // ---- base-3 weight stream ("T16B3"), an optional second copy of a plane ----------------------
 // The same tiles and K blocks, 832 bytes per chunk instead of 1024: lane l = g*16 + r keeps its 64
@@ -125,6 +132,7 @@ struct TkLaunchCfg {
   int tw;       // flow kernel, 16x16x64 form: runs per wave (tk_flow_runs_per_wave)
   int base3;    // flow kernel: stream the planes' base-3 copies (tk_launch_flow3)
   int fused;    // flow kernel, one row tile, one problem: build the operand rows in the kernel (no prep launch)
+  int zmap32;   // flow kernel, 32x32x32 form: the instantiations that consult the zero-chunk maps (tk_zskip.hip)
 };
 
 #ifdef __cplusplus
@@ -138,6 +146,10 @@ hipError_t tk_launch_relayout_tq1(hipStream_t s, const uint8_t *raw, uint8_t *co
 hipError_t tk_launch_zero_chunk_map(hipStream_t s, const uint8_t *codes, size_t chunks, uint32_t *map, unsigned *count);
 // LDS bytes the flow kernel needs for the maps of one workgroup: planes * this many words
 size_t tk_flow_zmap_words(size_t tiles_per_wg, size_t nb);
+// the 32x32x32 flow kernel's forms that consult the zero-chunk maps (tk_zskip.hip; tk_launch_flow goes there when
+// cfg.zmap32 is set): same arguments as tk_launch_flow
+hipError_t tk_launch_flow32_zmap(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                                 const TkLaunchCfg &cfg);
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
                                   int8_t *trits);
 // uniform_m > 0 says that entry j of the table starts at token j * uniform_m (all tensors equally long).
