@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel (sweep average), from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration against a 1 GiB copy kernel):
 # profiles/decode_flow_c2_sweep_traffic.txt
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_180_451_472
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_174_508_790
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 FP32_PEAK_TFLOPS = 157.3  # MI355X fp32, published
 
@@ -889,7 +889,7 @@ def main():
                    "copies": COPIES, "bytes_per_step": int(dec["bytes_per_launch_avg"] * len(SWEEP))},
         "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "tk_flow_kernel<2,1,1,4> (batch 1,2), tk_flow_kernel<2,1,2,4> (batch 4), tk_flow32_kernel<2,1,4> (batch 8), tk_flow_kernel<2,4,2,2> (batch 16)", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
+                     "kernel": "tk_flow_kernel<2,1,1,4> (batch 1,2), tk_flow_kernel<2,1,2,4> (batch 4), tk_flow32_kernel<2,1,2> (batch 8), tk_flow_kernel<2,4,2,2> (batch 16)", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
                      "algorithmic_bytes_per_launch": int(dec["bytes_per_launch_avg"])},
         "per_batch": dec["per_batch"],
         "verified": dec["verified"],

@@ -729,7 +729,17 @@ struct Plan {
 enum { DECODE_AUTO = 0, DECODE_KSPLIT = 1, DECODE_STREAM = 2, DECODE_FLOW = 3, DECODE_GEMM = 4 };
 
 static const size_t kLdsFlowMax = 160 * 1024;
-static int flow_waves(size_t lds) { return lds > 64 * 1024 ? 8 : 4; }
+// Waves per workgroup of the flow kernels: four up to 64 KiB of operand rows, eight beyond; with two row tiles and
+// more, eight as soon as a CU has room for at most two workgroups' rows (more than a third of the 160 KiB; one row
+// tile keeps the 64 KiB limit: not measured there, and its single-launch form that builds the rows itself is a
+// four-wave kernel). What counts is waves per CU: two four-wave workgroups are eight
+// waves, two eight-wave workgroups sixteen where the registers allow it (the one-plane forms of two row tiles on a
+// ring of two: 126), and where they do not a single eight-wave workgroup stages the rows once instead of twice.
+// Measured, 96-128 layer copies per launch, four -> eight waves between 53 and 64 KiB of rows: one plane K=2560,
+// 22 / 24 int8 rows x 6912 outputs 3.35 -> 4.36 / 3.30 -> 4.32 TB/s, 2560 outputs 3.39 -> 4.20, six float tokens
+// 3.74 -> 4.83; the 32x32x32 form at 64 KiB (two planes K=2048, eight float tokens) 5.32 -> 5.70 with runs of four
+// pairs on a ring of two.
+static int flow_waves(size_t lds, int rt) { return lds > (rt >= 2 ? kLdsFlowMax / 3 : 64 * 1024) ? 8 : 4; }
 // widest row stride any kernel asks of the staged operand rows of an R-row problem
 static size_t kPrepRowsMax(size_t R) { return R + 16 > 64 ? R + 16 : 64; }
 
@@ -785,6 +795,16 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
   cfg->zmap32 = wide && zmap_tiles ? 1 : 0;
 }
 
+// Ring size of a flow launch: the kernels' own rule (tk_flow_ring), except that the 32x32x32 form in eight-wave
+// workgroups of up to 64 KiB of rows takes two positions (two planes K=2048, eight float tokens: 5.54 -> 5.70 TB/s; one
+// plane, 28 int8 rows: 3.65 -> 4.24: on two positions its one-plane forms stay within 128 registers, four waves per SIMD).
+static int pick_flow_ring(const tk_ctx *ctx, const int *nbs, const double *wts, int count, int rt, int rows, int tw,
+                          bool wide, int waves, size_t lds) {
+  if (ctx->flow_ring) return ctx->flow_ring;
+  if (wide && waves >= 8 && lds <= 64 * 1024) return 2;
+  return tk_flow_ring(nbs, wts, count, rt, rows, tw);
+}
+
 // Consecutive tiles per run of the flow kernel. A workgroup pays for staging its operand rows
 // (lds_bytes) once, so it should stream several times that in weights; beyond that, shorter runs
 // win (more, shorter-lived workgroups keep more loads in flight and balance the tail). Measured on
@@ -803,7 +823,7 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * (b3 ? TK_B3_CHUNK_BYTES : TK_CHUNK_BYTES);
-  size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 ? 2 : 4);
+  size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 && lds_bytes > 64 * 1024 ? 2 : 4);
   if (target < 64 * 1024) target = 64 * 1024;
   size_t s = 1;
   while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
@@ -1092,7 +1112,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     wide = !b3 && pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R);
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
     if (b3) flow_lds += TK_B3_TABLE_BYTES;
-    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds);
+    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt);
     run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R, m);
     const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
@@ -1227,8 +1247,8 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
-    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds);
-    cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(&pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R));
+    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt);
+    cfg.ring = pick_flow_ring(ctx, &pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R), wide, cfg.waves, flow_lds);
     const size_t ztiles = flow_zero_plan(wide, b3, fused, cfg.planes, flow_lds,
                                          pr.zskip ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0, nb);
     if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or another form of the kernel): plain loads
@@ -1464,7 +1484,7 @@ static int run_salt(tk_ctx *ctx, const tk_salt_desc *layer, const void *act, int
   cfg.planes = layer->n_planes;
   cfg.rt = R <= 16 ? 1 : (R <= 32 ? 2 : 4);
   cfg.lds_bytes = lds;
-  cfg.waves = flow_waves(lds);
+  cfg.waves = flow_waves(lds, 1);  // (the 64 KiB limit at every row count: this kernel was tuned with it)
   // tiles per run: as the plain flow kernel (2 / 4 / 8 for one / two / four row tiles), fewer when
   // the launch would not give every CU its workgroups
   int s_tiles = cfg.rt == 1 ? 2 : (cfg.rt == 2 ? 4 : 8);
@@ -2144,7 +2164,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   const bool wide = !b3 && flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
   if (wide) flds = flow_wide_lds(rt, nb_max);
   if (b3) flds += TK_B3_TABLE_BYTES;
-  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds);
+  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds, rt);
   int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, b3, rows_max, tokens_max);
   {
     std::vector<unsigned> member_tiles(count);
@@ -2214,7 +2234,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     group_gemm_nt = gemm_nt2 ? 2 : 0;
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
-    const int pfw = flow_waves(pflds);
+    const int pfw = flow_waves(pflds, rt);
     int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max, tokens_max) : 1;
     {
       std::vector<unsigned> member_tiles;
@@ -2250,7 +2270,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.lds_bytes = pflds;
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
-      flow_cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, false, planes, rt, prows_max));
+      flow_cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, false, planes, rt, prows_max), pwide, pfw, pflds);
       size_t ztiles = 0;
       for (size_t i = 0; i < count; ++i)
         if (plans[i].flow_ok && plans[i].pr.zskip) ztiles = pper;
@@ -2432,7 +2452,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       nbs[i] = plans[i].pr.nb;
       wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
     }
-    g->cfg.ring = ctx->flow_ring ? ctx->flow_ring : tk_flow_ring(nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max));
+    g->cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max), wide, fw, flds);
   }
   if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max);
   if (gfused) {
