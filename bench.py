@@ -811,7 +811,7 @@ def summarize(out):
     c1 = ex.get("config1_f32_batch1")
     if c1:
         s["config1_batch1_f32"] = {"value": c1["step_GB/s_incl_digit_split"], "unit": "GB/s", "frac_of_hbm_peak": c1["step_frac_of_hbm_peak"],
-                                   "kernel_frac_of_hbm_peak": c1["kernel_frac_of_hbm_peak"], "kernel": "tk_flow_kernel<1,1,1,4>"}
+                                   "kernel_frac_of_hbm_peak": c1["kernel_frac_of_hbm_peak"], "kernel": "tk_flow_kernel<1,1,2,2>"}
     a8 = ex.get("decode_sweep_int8_activations")
     if a8:
         s["config2_decode_sweep_int8_contract"] = {"value": a8["step_sweep_GB/s_incl_quant"], "unit": "GB/s",
@@ -889,7 +889,7 @@ def main():
                    "copies": COPIES, "bytes_per_step": int(dec["bytes_per_launch_avg"] * len(SWEEP))},
         "roofline": {"bound": "hbm", "achieved": round(dec["kernel_gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dec["kernel_gbs"] / HBM_PEAK_GBS, 4), "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "tk_flow_kernel<2,1,1,4> (batch 1,2), tk_flow_kernel<2,1,2,4> (batch 4), tk_flow32_kernel<2,1,2> (batch 8), tk_flow_kernel<2,4,2,2> (batch 16)", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
+                     "kernel": "tk_flow_kernel<2,1,1,2> (batch 1), tk_flow_kernel<2,1,1,4> (batch 2), tk_flow_kernel<2,1,2,2> (batch 4), tk_flow32_kernel<2,1,2> (batch 8), tk_flow_kernel<2,4,2,2> (batch 16)", "avg_launch_ms": round(dec["kernel_avg_ms"], 4),
                      "algorithmic_bytes_per_launch": int(dec["bytes_per_launch_avg"])},
         "per_batch": dec["per_batch"],
         "verified": dec["verified"],

@@ -136,6 +136,8 @@ REGISTER_BUDGETS = (
     ("tk_flow_kernelILi1ELi1ELi1ELi4ELb1E", 128),   # one plane, one run per wave: a single operand row
     ("tk_flow_kernelILi1ELi1ELi2ELi4ELb1E", 128),   # one plane, two runs per wave: 2..16 rows
     ("tk_flow_kernelILi2ELi1ELi1ELi4ELb1E", 128),   # two planes, up to 8 rows
+    ("tk_flow_kernelILi2ELi1ELi1ELi2ELb1E", 96),    # ... on a ring of two (eight K blocks or fewer, 4 rows): five waves per SIMD
+    ("tk_flow_kernelILi2ELi1ELi2ELi2ELb1E", 128),   # two planes, 9..16 rows on a ring of two: four waves per SIMD
     ("tk_flow_kernelILi2ELi1ELi2ELi4ELb1E", 168),   # two planes, 9..16 rows
     ("tk_flow32_kernelILi2ELi1ELi4ELb1ELb0E", 168),     # two planes, 25..32 rows, four-wave workgroups
     ("tk_flow32_kernelILi2ELi1ELi2ELb1ELb0E", 168),     # ... eight-wave workgroups (from 53 KiB of rows on) on a ring of two

@@ -798,10 +798,18 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
 // Ring size of a flow launch: the kernels' own rule (tk_flow_ring), except that the 32x32x32 form in eight-wave
 // workgroups of up to 64 KiB of rows takes two positions (two planes K=2048, eight float tokens: 5.54 -> 5.70 TB/s; one
 // plane, 28 int8 rows: 3.65 -> 4.24: on two positions its one-plane forms stay within 128 registers, four waves per SIMD).
+// One row tile of two or more planes over at most eight K blocks also takes two positions, at 4 rows (one float token)
+// and from 9 rows on: K=2048 N=8192, 128 layer copies, four -> two positions, two planes, float contract 1 / 3 / 4 tokens
+// 6.43 -> 6.61 / 5.96 -> 6.09 / 5.90 -> 5.99 TB/s, int8 contract 9 / 12 / 16 tokens 5.77 -> 5.85 / 5.73 -> 5.83 / 5.74 -> 5.81
+// (3 int8 tokens 6.21 -> 6.14: left on four); three planes, one float token 6.33 -> 6.56. Sixteen K blocks (K=4096) show
+// no difference either way.
 static int pick_flow_ring(const tk_ctx *ctx, const int *nbs, const double *wts, int count, int rt, int rows, int tw,
-                          bool wide, int waves, size_t lds) {
+                          bool wide, int waves, size_t lds, int planes) {
   if (ctx->flow_ring) return ctx->flow_ring;
   if (wide && waves >= 8 && lds <= 64 * 1024) return 2;
+  int nb_max = 0;
+  for (int i = 0; i < count; ++i) nb_max = nbs[i] > nb_max ? nbs[i] : nb_max;
+  if (!wide && rt == 1 && planes >= 2 && nb_max <= 8 && (rows == 4 || rows >= 9)) return 2;
   return tk_flow_ring(nbs, wts, count, rt, rows, tw);
 }
 
@@ -1248,7 +1256,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
     cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt);
-    cfg.ring = pick_flow_ring(ctx, &pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R), wide, cfg.waves, flow_lds);
+    cfg.ring = pick_flow_ring(ctx, &pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R), wide, cfg.waves, flow_lds, pl.cfg.planes);
     const size_t ztiles = flow_zero_plan(wide, b3, fused, cfg.planes, flow_lds,
                                          pr.zskip ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0, nb);
     if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or another form of the kernel): plain loads
@@ -2270,7 +2278,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       flow_cfg.lds_bytes = pflds;
       flow_cfg.grid = flow_total;
       flow_cfg.waves = pfw;
-      flow_cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, false, planes, rt, prows_max), pwide, pfw, pflds);
+      flow_cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)nbs.size(), rt, (int)prows_max, flow_runs_per_wave(pwide, false, planes, rt, prows_max), pwide, pfw, pflds, planes);
       size_t ztiles = 0;
       for (size_t i = 0; i < count; ++i)
         if (plans[i].flow_ok && plans[i].pr.zskip) ztiles = pper;
@@ -2452,7 +2460,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       nbs[i] = plans[i].pr.nb;
       wts[i] = (double)plans[i].pr.n_tiles * (double)plans[i].pr.nb;  // chunks of the member
     }
-    g->cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max), wide, fw, flds);
+    g->cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max), wide, fw, flds, planes);
   }
   if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max);
   if (gfused) {
