@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel (sweep average), from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 after calibration against a 1 GiB copy kernel):
 # profiles/decode_flow_c2_sweep_traffic.txt
-DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_174_508_790
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1_166_242_550
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 FP32_PEAK_TFLOPS = 157.3  # MI355X fp32, published
 
