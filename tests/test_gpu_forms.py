@@ -287,6 +287,50 @@ def test_grouped_flow_kernel_wide_form_chosen_automatically(backend, oracle, mod
     db.free()
 
 
+@pytest.mark.parametrize("mode,m,planes,k", [(1, 22, 1, 2560), (1, 24, 2, 2560), (0, 6, 1, 2560), (1, 17, 1, 3328), (1, 28, 1, 2048), (0, 7, 2, 2048)])
+def test_two_row_tiles_in_eight_wave_workgroups(backend, oracle, mode, m, planes, k):
+    """17..32 operand rows whose copy in LDS takes between a third of the 160 KiB and 64 KiB: the flow kernels
+    run them in eight-wave workgroups (both matrix-instruction forms), single launches and groups. Bits of the
+    CPU under the int8 contract, its bounds under the float contract, and the same bits with the run length and
+    the ring forced to other values."""
+    print("case eight-wave rt2", mode, m, planes, k, flush=True)
+    backend.set_stream_min_groups(1)
+    rng = np.random.default_rng(mode * 1000 + m * 10 + planes + k)
+    n = 1029
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    dact = backend.to_device(f32_to_bf16_bits(act), "bf16")
+    act = bf16_bits_to_f32(f32_to_bf16_bits(act)).reshape(m, k)
+    ws, scs, packed = _planes(rng, n, k, planes)
+    layer = backend.linear(packed, scs, n, k)
+    out, out2 = backend.empty(m * n, "f32"), backend.empty(m * n, "f32")
+    call = backend.linear_a8 if mode == 1 else backend.linear_float
+    call(layer, dact, m, out)
+    assert backend.last_kernel() in ("flow", "flow32"), backend.last_kernel()
+    got = out.to_host().copy()
+    if mode == 1:
+        assert same_bits(got, oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k))
+    else:
+        want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+        assert rel_err(got.reshape(m, n), want) <= 1e-3
+        assert accepts(got.reshape(m, n), want, rel=1e-4, floor=1.0).all()
+    try:
+        for run_tiles, ring in ((1, 3), (3, 2), (2, 4)):
+            backend.set_flow_run_tiles(run_tiles)
+            backend.set_flow_ring(ring)
+            call(layer, dact, m, out2)
+            assert same_bits(out2.to_host(), got), (run_tiles, ring)
+            grp = backend.group([(layer, dact, m, out2), (layer, dact, m, out)], mode, "bf16", "f32")
+            grp.launch()
+            assert same_bits(out2.to_host(), got) and same_bits(out.to_host(), got), (run_tiles, ring)
+            grp.destroy()
+    finally:
+        backend.set_flow_run_tiles(0)
+        backend.set_flow_ring(0)
+    for x in (dact, out, out2):
+        x.free()
+    layer.free()
+
+
 def test_gemm_tiles_knob_rejects_other_values(backend):
     for bad in (1, 3, 8, -2):
         with pytest.raises(T.InvalidInput):
