@@ -331,6 +331,60 @@ def test_two_row_tiles_in_eight_wave_workgroups(backend, oracle, mode, m, planes
     layer.free()
 
 
+@pytest.mark.parametrize("m", [1, 3, 4, 9, 16, 20, 40, 64])
+@pytest.mark.parametrize("planes,n", [(1, 1029), (2, 520), (3, 134), (4, 48)])
+def test_both_operand_orders_of_the_decode_kernel(backend, oracle, m, planes, n):
+    """The decode kernel under the int8 contract with weights as the first operand of the matrix instruction (a lane
+    finishes four channels of one token: one wide store) and with activations first: the same bits, and the CPU's --
+    f32 and bf16 outputs, output rows whose stride does not allow the wide store, a residual, a token holding NaN
+    (recomputed in the reference's order), single launches and groups."""
+    print("case operand order", m, planes, n, flush=True)
+    backend.set_stream_min_groups(1)
+    backend.set_decode_kernel(3)  # the flow kernel also for launches that would go elsewhere
+    rng = np.random.default_rng(m * 100 + planes * 7 + n)
+    k = 1280 - 24
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    if m >= 3:
+        act[m // 2, 5] = np.nan
+    dact = backend.to_device(act, "f32")
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85, 0.9)[:planes]]
+    scs = [scales(rng, n) for _ in range(planes)]
+    packed = [T.pack_rows(w, n, k) for w in ws]
+    layer = backend.linear(packed, scs, n, k)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    dres = backend.to_device(res, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    outs = {}
+    try:
+        for order in (1, 0):
+            backend.set_flow_operand_order(order)
+            o32, o16, ores = backend.empty(m * n, "f32"), backend.empty(m * n, "bf16"), backend.empty(m * n, "f32")
+            backend.linear_a8(layer, dact, m, o32)
+            assert backend.last_kernel() == "flow", backend.last_kernel()
+            backend.linear_a8(layer, dact, m, o16)
+            backend.linear_a8_residual(layer, dact, m, dres, ores)
+            g32 = backend.empty(m * n, "f32")
+            grp = backend.group([(layer, dact, m, g32), (layer, dact, m, o32)], 1, "f32", "f32")
+            grp.launch()
+            outs[order] = [x.to_host().copy() for x in (o32, o16, ores, g32)]
+            grp.destroy()
+            for x in (o32, o16, ores, g32):
+                x.free()
+    finally:
+        backend.set_flow_operand_order(1)
+    for a, b in zip(outs[0], outs[1]):
+        assert same_bits(a, b)
+    def like_cpu(got, ref):  # (NaN where the CPU has NaN -- the payload may differ -- and its bits everywhere else)
+        got, ref = got.reshape(-1), np.asarray(ref, np.float32).reshape(-1)
+        fin = ~np.isnan(ref)
+        return bool((np.isnan(got) == np.isnan(ref)).all()) and same_bits(got[fin], ref[fin])
+    assert like_cpu(outs[1][0], want) and like_cpu(outs[1][3], want)
+    assert like_cpu(outs[1][2], (res + want.reshape(m, n)).astype(np.float32))
+    for x in (dact, dres):
+        x.free()
+    layer.free()
+
+
 def test_gemm_tiles_knob_rejects_other_values(backend):
     for bad in (1, 3, 8, -2):
         with pytest.raises(T.InvalidInput):

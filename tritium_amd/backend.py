@@ -623,6 +623,11 @@ class Mi355xBackend:
         """Later uploads: 0 keep a zero-chunk map by the 0.5% threshold, 1 never, 2 always."""
         _check(self._lib.tk_set_zero_skip(self._ctx, mode))
 
+    def set_flow_operand_order(self, weights_first):
+        """Decode kernel under the int8 contract: 1 weights as the first operand of the matrix instruction (one wide
+        store per lane), 0 activations first (same bits)."""
+        _check(self._lib.tk_set_flow_operand_order(self._ctx, weights_first))
+
     def set_base3_stream(self, mode):
         """Later uploads: 0 no base-3 copy, 1 TQ1_0 uploads keep one beside the 2-bit codes, 2 every upload."""
         _check(self._lib.tk_set_base3_stream(self._ctx, mode))

@@ -10,7 +10,7 @@ import tempfile
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtritium_mi355x.so")
-SOURCES = ["tk_kernels.hip", "tk_zskip.hip", "tk_gemm128.hip", "tk_gemm256.hip", "tk_base3.hip", "tk_salt_v2.hip", "tk_vjp.hip", "tk_api.hip", "tk_format.cpp", "tk_salt.cpp", "tk_gguf.cpp"]
+SOURCES = ["tk_kernels.hip", "tk_flow_a8.hip", "tk_zskip.hip", "tk_gemm128.hip", "tk_gemm256.hip", "tk_base3.hip", "tk_salt_v2.hip", "tk_vjp.hip", "tk_api.hip", "tk_format.cpp", "tk_salt.cpp", "tk_gguf.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     # packed-FP32 instructions are kept out of every kernel of this library
@@ -28,7 +28,7 @@ def hipcc():
 
 # Translation units whose device assembly is emitted and checked before linking: in-flight registers of the
 # hand-issued loads (the prefill kernels), register budgets, and kernels that need an empty static LDS segment.
-ASM_SOURCES = ["tk_kernels.hip", "tk_zskip.hip", "tk_gemm128.hip", "tk_gemm256.hip", "tk_base3.hip"]
+ASM_SOURCES = ["tk_kernels.hip", "tk_flow_a8.hip", "tk_zskip.hip", "tk_gemm128.hip", "tk_gemm256.hip", "tk_base3.hip"]
 HAZARD_SOURCES = ["tk_kernels.hip", "tk_gemm256.hip"]
 
 

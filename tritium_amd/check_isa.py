@@ -133,15 +133,15 @@ def check_text(text, only=("tk_gemm",)):
 # forms over its step (a few registers are enough) costs a third or a quarter of the rate without any test
 # noticing. The build fails instead.
 REGISTER_BUDGETS = (
-    ("tk_flow_kernelILi1ELi1ELi1ELi4ELb1E", 128),   # one plane, one run per wave: a single operand row
-    ("tk_flow_kernelILi1ELi1ELi2ELi4ELb1E", 128),   # one plane, two runs per wave: 2..16 rows
-    ("tk_flow_kernelILi2ELi1ELi1ELi4ELb1E", 128),   # two planes, up to 8 rows
-    ("tk_flow_kernelILi2ELi1ELi1ELi2ELb1E", 96),    # ... on a ring of two (eight K blocks or fewer, 4 rows): five waves per SIMD
-    ("tk_flow_kernelILi2ELi1ELi2ELi2ELb1E", 128),   # two planes, 9..16 rows on a ring of two: four waves per SIMD
-    ("tk_flow_kernelILi2ELi1ELi2ELi4ELb1E", 168),   # two planes, 9..16 rows
+    ("tk_flow_kernelILi1ELi1ELi1ELi4ELb1ELb0ELb0E", 128),   # one plane, one run per wave: a single operand row
+    ("tk_flow_kernelILi1ELi1ELi2ELi4ELb1ELb0ELb0E", 128),   # one plane, two runs per wave: 2..16 rows
+    ("tk_flow_kernelILi2ELi1ELi1ELi4ELb1ELb0ELb0E", 128),   # two planes, up to 8 rows
+    ("tk_flow_kernelILi2ELi1ELi1ELi2ELb1ELb0ELb0E", 96),    # ... on a ring of two (eight K blocks or fewer, 4 rows): five waves per SIMD
+    ("tk_flow_kernelILi2ELi1ELi2ELi2ELb1ELb0ELb0E", 128),   # two planes, 9..16 rows on a ring of two: four waves per SIMD
+    ("tk_flow_kernelILi2ELi1ELi2ELi4ELb1ELb0ELb0E", 168),   # two planes, 9..16 rows
     ("tk_flow32_kernelILi2ELi1ELi4ELb1ELb0E", 168),     # two planes, 25..32 rows, four-wave workgroups
     ("tk_flow32_kernelILi2ELi1ELi2ELb1ELb0E", 168),     # ... eight-wave workgroups (from 53 KiB of rows on) on a ring of two
-    ("tk_flow_kernelILi2ELi4ELi2ELi2ELb1E", 256),   # two planes, 33..64 rows
+    ("tk_flow_kernelILi2ELi4ELi2ELi2ELb1ELb0ELb0E", 256),   # two planes, 33..64 rows
     ("tk_gemm32_kernelILi1ELi2ELb0ELb0E", 168),     # prefill, one plane (three waves per SIMD by design)
     ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
     ("tk_gemm32_kernelILi3ELi2ELb0ELb0E", 256),     # prefill, three planes (two waves per SIMD)

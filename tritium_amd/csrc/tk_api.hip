@@ -97,6 +97,7 @@ struct tk_ctx {
   bool gemm256_form_forced = false;  // tk_set_gemm256_form was called: automatic launches keep that form
   int gemm256_form = 0;    // the 256-row kernel: 0 = 4 waves x 224 outputs, 1 = 8 waves x 224, 2 = 4 waves x (128 | 96), two workgroups per CU
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
+  int flow_swap = 1;       // flow kernel, int8 contract: 1 = weights as the first operand of the matrix instruction (one wide store per lane), 0 = activations first
   int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
   unsigned *d_count = nullptr;  // a device counter for the uploads
 
@@ -432,6 +433,14 @@ extern "C" int tk_set_zero_skip(tk_ctx *ctx, int mode) {
   if (mode < 0 || mode > 2) return tk_fail(TK_ERR_INVALID_INPUT, "zero_skip=%d - use 0 (by threshold), 1 (never) or 2 (always)", mode);
   std::lock_guard<std::mutex> lk(ctx->mu);
   ctx->zero_skip = mode;
+  return TK_OK;
+}
+
+extern "C" int tk_set_flow_operand_order(tk_ctx *ctx, int weights_first) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_operand_order: null context");
+  if (weights_first < 0 || weights_first > 1) return tk_fail(TK_ERR_INVALID_INPUT, "flow_operand_order=%d - use 0 (activations first) or 1 (weights first)", weights_first);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->flow_swap = weights_first;
   return TK_OK;
 }
 
@@ -783,8 +792,10 @@ static size_t flow_zero_plan(bool wide, bool b3, bool fused, int planes, size_t 
 }
 // zmap_tiles > 0: some plane of the launch carries a zero-chunk map (flow_zero_plan)
 // (b3: flow_lds includes the decode table; ring and runs per wave are the base-3 kernel's own)
+// swap: the launch runs under the int8 contract and the context asks for the second operand order where a form exists
+// (the 16x16x64 kernel from a prepared set of operand rows)
 static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds, size_t rows, size_t zmap_tiles = 0,
-                          size_t zmap_nb = 0) {
+                          size_t zmap_nb = 0, bool swap = false) {
   cfg->wide_mfma = wide ? 1 : 0;
   cfg->base3 = b3 ? 1 : 0;
   if (b3) cfg->ring = 4;
@@ -793,6 +804,7 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
   if (zmap_tiles) cfg->lds_bytes += (size_t)cfg->planes * tk_flow_zmap_words(zmap_tiles, zmap_nb) * 4;
   if (wide && cfg->ring > 4) cfg->ring = 4;
   cfg->zmap32 = wide && zmap_tiles ? 1 : 0;
+  cfg->swap = swap && !wide && !b3 ? 1 : 0;
 }
 
 // Ring size of a flow launch: the kernels' own rule (tk_flow_ring), except that the 32x32x32 form in eight-wave
@@ -1260,7 +1272,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     const size_t ztiles = flow_zero_plan(wide, b3, fused, cfg.planes, flow_lds,
                                          pr.zskip ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0, nb);
     if (!ztiles) pr.zskip = 0;  // no room for the maps behind the rows (or another form of the kernel): plain loads
-    flow_cfg_form(&cfg, wide, b3, flow_lds, R, ztiles, nb);
+    flow_cfg_form(&cfg, wide, b3, flow_lds, R, ztiles, nb, mode == TK_MODE_INT8 && ctx->flow_swap && !fused);
     if (fused) {
       cfg.fused = 1;
       cfg.lds_bytes += fuse_lds;
@@ -2286,7 +2298,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       if (!ztiles)
         for (size_t i = 0; i < count; ++i)
           if (plans[i].flow_ok) plans[i].pr.zskip = 0;
-      flow_cfg_form(&flow_cfg, pwide, false, pflds, prows_max, ztiles, pnb_max);
+      flow_cfg_form(&flow_cfg, pwide, false, pflds, prows_max, ztiles, pnb_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
     }
   } else if (variant != DECODE_KSPLIT) {
     const unsigned per = variant == DECODE_FLOW ? fper : tpw;
@@ -2462,7 +2474,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     }
     g->cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max), wide, fw, flds, planes);
   }
-  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max);
+  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max, kmode == TK_MODE_INT8 && ctx->flow_swap && !gfused);
   if (gfused) {
     g->cfg.fused = 1;
     g->cfg.lds_bytes = fuse_lds;

@@ -367,6 +367,67 @@ __device__ __forceinline__ void flow_epilogue(const PR &pr, int n, int rowbase, 
   }
 }
 
+// The epilogue of the decode kernels' second operand order (int8 contract): the lane holds token m and the four output
+// channels n0 .. n0+3 in the four accumulator registers of every plane. The arithmetic per output is int8_value's, so the
+// bits are those of flow_epilogue; the four results leave as one 8-byte (bf16) or 16-byte (f32) store when the row
+// stride and the base address allow it and there is no residual to add. A flagged token (NaN/Inf in its activations) is
+// recomputed per output in the reference's order, like exact_rows does.
+template <int P, typename PR>
+__device__ __forceinline__ void flow_epilogue_swapped(const PR &hot, const TkProblem &pr, int m, int n0, const v4i (&acc)[P],
+                                                      const float (&sc4)[P][4], int rs, float as, unsigned flagged) {
+  if (m >= hot.R) return;
+  const size_t idx = (size_t)m * (size_t)hot.n + (size_t)n0;
+  if (hot.out_dtype == TK_I32) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n0 + r < hot.n) gstore((int32_t *)hot.out + idx + r, acc[0][r] - rs);
+    return;
+  }
+  if (flagged) {
+    for (int r = 0; r < 4; ++r) {
+      if (n0 + r >= hot.n) break;
+      float f = 0.0f;
+      for (int p = 0; p < pr.planes; ++p) {
+        const float t = __fmul_rn(seq_dot(pr, p, n0 + r, m, 1), pr.scales[p][n0 + r]);
+        f = p == 0 ? t : __fadd_rn(f, t);
+      }
+      if (pr.act_scale) f = __fmul_rn(f, pr.act_scale[m]);
+      store_out(hot.out, hot.out_dtype, idx + r, with_residual(hot.residual, hot.out_dtype, idx + r, f));
+    }
+    return;
+  }
+  const bool has_as = hot.act_scale != nullptr;
+  float f[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    f[r] = 0.0f;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      const float t = __fmul_rn((float)(acc[p][r] - rs), sc4[p][r]);
+      f[r] = p == 0 ? t : __fadd_rn(f[r], t);
+    }
+    if (has_as) f[r] = __fmul_rn(f[r], as);
+  }
+  const bool bf16 = hot.out_dtype == TK_BF16;
+  const unsigned esz = bf16 ? 2u : 4u;
+  const bool wide = !hot.residual && n0 + 3 < hot.n && (((uintptr_t)hot.out + idx * esz) & (bf16 ? 7u : 15u)) == 0;
+  if (wide) {
+    if (bf16) {
+      const uint32_t lo = (uint32_t)f32_to_bf16_rne(f[0]) | ((uint32_t)f32_to_bf16_rne(f[1]) << 16);
+      const uint32_t hi = (uint32_t)f32_to_bf16_rne(f[2]) | ((uint32_t)f32_to_bf16_rne(f[3]) << 16);
+      typedef unsigned v2u_ __attribute__((ext_vector_type(2)));
+      *(TK_GLOBAL v2u_ *)((uint16_t *)hot.out + idx) = v2u_{lo, hi};
+    } else {
+      typedef float v4f_ __attribute__((ext_vector_type(4)));
+      *(TK_GLOBAL v4f_ *)((float *)hot.out + idx) = v4f_{f[0], f[1], f[2], f[3]};
+    }
+    return;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (n0 + r < hot.n) store_out(hot.out, hot.out_dtype, idx + r, with_residual(hot.residual, hot.out_dtype, idx + r, f[r]));
+}
+
 // The rows of one lane that hold NaN/Inf: recomputed in the reference's order (needs no accumulator).
 __device__ __forceinline__ void exact_rows(const TkProblem &pr, int n, int rowbase, unsigned flag) {
   if (pr.out_dtype == TK_I32) return;

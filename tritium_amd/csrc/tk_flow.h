@@ -25,13 +25,20 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
 // eight waves); the form with two planes and two runs per wave on a ring of four sits at the edge of
 // three (168 registers) -- left alone it takes 169, which costs a third of the waves in flight and 8% of
 // the rate at 9..16 operand rows.
-#define TK_FLOW_MIN_WAVES(P, RT, TW, DR) (((P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
+#define TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP) ((!(SWAP) && (P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
 // FUSED (one row tile, a single problem, 256 threads): the kernel builds the operand rows of its one to four
 // tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of two.
-template <int P, int RT, int TW, int DR, bool TABLE, bool FUSED = false>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+// SWAP (int8 contract only; instantiated in tk_flow_a8.hip): the two operands of the matrix instruction change places --
+// weights first, activations second -- so that an accumulator register holds four consecutive OUTPUT CHANNELS of one
+// token (lane (g, i): token rt*16 + i, channels 16*tile + 4g .. 4g+3) instead of four tokens of one channel. The integers
+// are the same; what changes is the epilogue: a lane writes its four values with ONE 8- or 16-byte store instead of
+// four 2- or 4-byte stores to four output rows, and a decode launch of 8..64 tokens is held back by the number of
+// store instructions it issues, not by their bytes.
+template <int P, int RT, int TW, int DR, bool TABLE, bool FUSED = false, bool SWAP = false>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                       const int *__restrict__ wg_prob) {
   static_assert(!FUSED || (RT == 1 && !TABLE), "the fused form: one row tile, one problem");
+  static_assert(!(FUSED && SWAP), "the fused form keeps the first operand order");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : *single_problem();
   const int NW = (int)(blockDim.x >> 6);  // 4 or 8 waves
@@ -137,11 +144,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
   }
   RowConst rc[RT];
   unsigned any_flag = 0;
+  // SWAP: the constants of this lane's one token per row tile (row rt*16 + i)
+  int tok_rs[RT];
+  float tok_as[RT];
+  unsigned tok_flag[RT];
+  if constexpr (SWAP) {
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    if constexpr (FUSED) rc[rt] = row_const_from_lds(cst, hot.mode, R, hot.M, rt * 16 + 4 * g);  // (staged behind a barrier)
-    else rc[rt] = load_row_const(hot, rt * 16 + 4 * g);
-    any_flag |= rc[rt].flag;
+    for (int rt = 0; rt < RT; ++rt) {
+      const int m = rt * 16 + i;
+      tok_rs[rt] = m < R ? gload(hot.rowsum + m) : 0;
+      tok_as[rt] = m < R && hot.act_scale ? gload(hot.act_scale + m) : 1.0f;
+      tok_flag[rt] = m < R && hot.flags ? gload(hot.flags + m) : 0u;
+      any_flag |= tok_flag[rt];
+    }
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if constexpr (FUSED) rc[rt] = row_const_from_lds(cst, hot.mode, R, hot.M, rt * 16 + 4 * g);  // (staged behind a barrier)
+      else rc[rt] = load_row_const(hot, rt * 16 + 4 * g);
+      any_flag |= rc[rt].flag;
+    }
   }
   if constexpr (!FUSED) __syncthreads();
   const uint4 *lds4 = (const uint4 *)smem;
@@ -153,11 +175,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
   for (int s = 0; s < S; ++s) {
     // per-tile scales, issued now, consumed in the epilogue
     float sc[TW][P];
+    // SWAP: the scales of this lane's four channels (requested behind the K loop instead, they save the two-plane forms
+    // nine registers and cost every form 2-7%: the epilogue then waits for them)
+    float sc4[SWAP ? TW : 1][SWAP ? P : 1][4];
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
-      const int n = min((first + s * TW + tw) * 16 + i, hot.n - 1);
+      if constexpr (SWAP) {
+        const int n0 = (first + s * TW + tw) * 16 + 4 * g;
 #pragma unroll
-      for (int p = 0; p < P; ++p) sc[tw][p] = gload(scales[p] + n);
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sc4[tw][p][r] = gload(scales[p] + min(n0 + r, hot.n - 1));
+      } else {
+        const int n = min((first + s * TW + tw) * 16 + i, hot.n - 1);
+#pragma unroll
+        for (int p = 0; p < P; ++p) sc[tw][p] = gload(scales[p] + n);
+      }
     }
     v4i acc[TW][RT][P];
 #pragma unroll
@@ -197,7 +230,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
                 const v4i b = expand_codes(wj);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
-                  acc[tw][rt][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[tw][rt][p], 0, 0, 0);
+                  acc[tw][rt][p] = SWAP ? __builtin_amdgcn_mfma_i32_16x16x64_i8(b, a[rt], acc[tw][rt][p], 0, 0, 0)
+                                        : __builtin_amdgcn_mfma_i32_16x16x64_i8(a[rt], b, acc[tw][rt][p], 0, 0, 0);
               }
           }
         }
@@ -205,6 +239,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN
       kbg += DR;
     } while (kbg < nbpad);
 
+    if constexpr (SWAP) {
+#pragma unroll
+      for (int tw = 0; tw < TW; ++tw) {
+        const int t = first + s * TW + tw;
+        const int n0 = t * 16 + 4 * g;
+        if (t < n_tiles && n0 < hot.n) {
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            flow_epilogue_swapped<P>(hot, pr, rt * 16 + i, n0, acc[tw][rt], sc4[tw], tok_rs[rt], tok_as[rt], tok_flag[rt]);
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int tw = 0; tw < TW; ++tw) {
       const int t = first + s * TW + tw;

@@ -133,6 +133,7 @@ struct TkLaunchCfg {
   int base3;    // flow kernel: stream the planes' base-3 copies (tk_launch_flow3)
   int fused;    // flow kernel, one row tile, one problem: build the operand rows in the kernel (no prep launch)
   int zmap32;   // flow kernel, 32x32x32 form: the instantiations that consult the zero-chunk maps (tk_zskip.hip)
+  int swap;     // flow kernel, 16x16x64 form, int8 contract: the second operand order (tk_flow_a8.hip)
 };
 
 #ifdef __cplusplus
@@ -150,6 +151,10 @@ size_t tk_flow_zmap_words(size_t tiles_per_wg, size_t nb);
 // cfg.zmap32 is set): same arguments as tk_launch_flow
 hipError_t tk_launch_flow32_zmap(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
                                  const TkLaunchCfg &cfg);
+// the 16x16x64 flow kernel's forms with weights as the first operand (tk_flow_a8.hip; int8 contract only; tk_launch_flow
+// goes there when cfg.swap is set): same arguments as tk_launch_flow
+hipError_t tk_launch_flow_swapped(hipStream_t s, const TkProblem *single, const TkProblem *table, const int *wg_prob,
+                                  const TkLaunchCfg &cfg);
 hipError_t tk_launch_decode_trits(hipStream_t s, const uint8_t *codes, size_t n, size_t k, size_t nb,
                                   int8_t *trits);
 // uniform_m > 0 says that entry j of the table starts at token j * uniform_m (all tensors equally long).
