@@ -242,7 +242,8 @@ def test_grouped_prefill_kernel_every_plane_count(backend, oracle, planes, tiles
 def test_grouped_flow_kernel_wide_form_chosen_automatically(backend, oracle, mode, m, planes):
     """25..32 operand rows that take at most 64 KiB of LDS: the flow kernel picks the 32x32x32 matrix
     instruction by itself (tk_flow32_kernel<P,1,*,true> from a problem table: the headline's batch 8 is
-    8 tokens x 4 digit rows x 2 planes). The group is made wide enough for the flow kernel by lowering
+    8 tokens x 4 digit rows x 2 planes; under the int8 contract, where both forms put the weights first, only
+    with two planes). The group is made wide enough for the flow kernel by lowering
     the workgroup threshold, not by forcing a kernel. Forced onto the 16x16x64 form it gives the same
     bits."""
     print("case grouped-flow32", mode, m, planes, flush=True)
@@ -332,15 +333,17 @@ def test_two_row_tiles_in_eight_wave_workgroups(backend, oracle, mode, m, planes
 
 
 @pytest.mark.parametrize("m", [1, 3, 4, 9, 16, 20, 40, 64])
-@pytest.mark.parametrize("planes,n", [(1, 1029), (2, 520), (3, 134), (4, 48)])
-def test_both_operand_orders_of_the_decode_kernel(backend, oracle, m, planes, n):
+@pytest.mark.parametrize("planes,n,mfma", [(1, 1029, 0), (2, 520, 0), (3, 134, 0), (4, 48, 0), (1, 1029, 32), (2, 520, 32), (2, 56, 32)])
+def test_both_operand_orders_of_the_decode_kernel(backend, oracle, m, planes, n, mfma):
     """The decode kernel under the int8 contract with weights as the first operand of the matrix instruction (a lane
     finishes four channels of one token: one wide store) and with activations first: the same bits, and the CPU's --
     f32 and bf16 outputs, output rows whose stride does not allow the wide store, a residual, a token holding NaN
-    (recomputed in the reference's order), single launches and groups."""
-    print("case operand order", m, planes, n, flush=True)
+    (recomputed in the reference's order), single launches and groups; the 16x16x64 form where the library would pick
+    it and the 32x32x32 form forced (one and two planes; an odd tile count, so a pair whose second tile does not exist)."""
+    print("case operand order", m, planes, n, mfma, flush=True)
     backend.set_stream_min_groups(1)
     backend.set_decode_kernel(3)  # the flow kernel also for launches that would go elsewhere
+    backend.set_flow_mfma(mfma)
     rng = np.random.default_rng(m * 100 + planes * 7 + n)
     k = 1280 - 24
     act = rng.standard_normal((m, k)).astype(np.float32)
@@ -360,7 +363,7 @@ def test_both_operand_orders_of_the_decode_kernel(backend, oracle, m, planes, n)
             backend.set_flow_operand_order(order)
             o32, o16, ores = backend.empty(m * n, "f32"), backend.empty(m * n, "bf16"), backend.empty(m * n, "f32")
             backend.linear_a8(layer, dact, m, o32)
-            assert backend.last_kernel() == "flow", backend.last_kernel()
+            assert backend.last_kernel() == ("flow32" if mfma == 32 and m > 16 else "flow"), backend.last_kernel()
             backend.linear_a8(layer, dact, m, o16)
             backend.linear_a8_residual(layer, dact, m, dres, ores)
             g32 = backend.empty(m * n, "f32")
@@ -372,6 +375,7 @@ def test_both_operand_orders_of_the_decode_kernel(backend, oracle, m, planes, n)
                 x.free()
     finally:
         backend.set_flow_operand_order(1)
+        backend.set_flow_mfma(0)
     for a, b in zip(outs[0], outs[1]):
         assert same_bits(a, b)
     def like_cpu(got, ref):  # (NaN where the CPU has NaN -- the payload may differ -- and its bits everywhere else)

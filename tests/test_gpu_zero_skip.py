@@ -117,7 +117,8 @@ def test_bits_identical_with_and_without_the_map(backend, oracle, m, planes, run
 @pytest.mark.parametrize("planes", [1, 2])
 @pytest.mark.parametrize("mfma", [0, 32])
 def test_the_32x32x32_form_consults_the_maps_too(backend, oracle, m, planes, mfma):
-    """The 32x32x32 form of the flow kernel (automatic at 25..32 operand rows, forced here beyond) with mapped
+    """The 32x32x32 form of the flow kernel (automatic at 25..32 operand rows -- with weights as the first operand only
+    for two planes --, forced here beyond) with mapped
     planes, single launches and groups: the bits of the unmapped planes and of the CPU. A wave of that form walks a
     pair of tiles, so pairs with one marked chunk, with both and with none all occur."""
     print("case zero-skip 32x32x32", m, planes, mfma, flush=True)
@@ -141,12 +142,14 @@ def test_the_32x32x32_form_consults_the_maps_too(backend, oracle, m, planes, mfm
     want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, actb, m, n, k)
     backend.set_flow_mfma(mfma)
     try:
-        backend.linear_a8(with_map, dact, m, o[0])
-        took = backend.last_kernel()
-        backend.linear_a8(without, dact, m, o[1])
-        if mfma == 32 and m > 16 or 24 < m <= 32:
-            assert took == "flow32", (took, m, planes, mfma)
-        assert same_bits(o[0].to_host(), want) and same_bits(o[1].to_host(), want)
+        for weights_first in (0, 1):  # both operand orders of the matrix instruction
+            backend.set_flow_operand_order(weights_first)
+            backend.linear_a8(with_map, dact, m, o[0])
+            took = backend.last_kernel()
+            backend.linear_a8(without, dact, m, o[1])
+            if mfma == 32 and m > 16 or (24 < m <= 32 and (planes == 2 or not weights_first)):
+                assert took == "flow32", (took, m, planes, mfma, weights_first)
+            assert same_bits(o[0].to_host(), want) and same_bits(o[1].to_host(), want)
         if m <= 16:
             backend.linear_float(with_map, dact, m, o[0])
             tookf = backend.last_kernel()
@@ -163,6 +166,7 @@ def test_the_32x32x32_form_consults_the_maps_too(backend, oracle, m, planes, mfm
         grp.destroy()
     finally:
         backend.set_flow_mfma(0)
+        backend.set_flow_operand_order(1)
     for a in [dact] + o:
         a.free()
     with_map.free()

@@ -139,8 +139,9 @@ REGISTER_BUDGETS = (
     ("tk_flow_kernelILi2ELi1ELi1ELi2ELb1ELb0ELb0E", 96),    # ... on a ring of two (eight K blocks or fewer, 4 rows): five waves per SIMD
     ("tk_flow_kernelILi2ELi1ELi2ELi2ELb1ELb0ELb0E", 128),   # two planes, 9..16 rows on a ring of two: four waves per SIMD
     ("tk_flow_kernelILi2ELi1ELi2ELi4ELb1ELb0ELb0E", 168),   # two planes, 9..16 rows
-    ("tk_flow32_kernelILi2ELi1ELi4ELb1ELb0E", 168),     # two planes, 25..32 rows, four-wave workgroups
-    ("tk_flow32_kernelILi2ELi1ELi2ELb1ELb0E", 168),     # ... eight-wave workgroups (from 53 KiB of rows on) on a ring of two
+    ("tk_flow32_kernelILi2ELi1ELi4ELb1ELb0ELb0E", 168), # two planes, 25..32 rows, four-wave workgroups
+    ("tk_flow32_kernelILi2ELi1ELi2ELb1ELb0ELb0E", 168), # ... eight-wave workgroups (from 53 KiB of rows on) on a ring of two
+    ("tk_flow32_kernelILi2ELi1ELi2ELb1ELb0ELb1E", 168), # ... weights first (int8 contract; sixteen scales per plane held over a pair of tiles)
     ("tk_flow_kernelILi2ELi4ELi2ELi2ELb1ELb0ELb0E", 256),   # two planes, 33..64 rows
     ("tk_gemm32_kernelILi1ELi2ELb0ELb0E", 168),     # prefill, one plane (three waves per SIMD by design)
     ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
@@ -149,8 +150,9 @@ REGISTER_BUDGETS = (
     ("tk_gemm256_kernelILi0E", 512),                # prefill, 256 x 224 form, four waves (one per SIMD)
     ("tk_gemm256_kernelILi1E", 256),                # ... eight waves (two per SIMD)
     ("tk_gemm256_kernelILi2E", 256),                # ... four waves over 128 | 96 outputs, two workgroups per CU
-) + tuple(  # the 32x32x32 flow forms that consult the zero-chunk maps (last argument true): present, no spills
-    (f"tk_flow32_kernelILi{p}ELi{rt2}ELi{dr}ELb{t}ELb1E", 256) for p in (1, 2) for rt2 in (1, 2) for dr in (2, 3, 4) for t in (0, 1)
+) + tuple(  # the 32x32x32 flow forms that consult the zero-chunk maps, in both operand orders: present, no spills
+    (f"tk_flow32_kernelILi{p}ELi{rt2}ELi{dr}ELb{t}ELb1ELb{sw}E", 256)
+    for p in (1, 2) for rt2 in (1, 2) for dr in (2, 3, 4) for t in (0, 1) for sw in (0, 1)
 )
 
 

@@ -764,10 +764,15 @@ static size_t flow_wide_lds(int rt, size_t nb) { return nb * 256 * flow_wide_row
 // to 32), the 16x16x64 form is as fast or up to 4% faster. At 33..64 rows the picture is mixed (two
 // planes K=2048 int8: 9% faster; one plane: 4-18% slower), so those keep the 16x16x64 form unless
 // the wide one is asked for.
-static bool flow_wide(const tk_ctx *ctx, int planes, int rt, size_t nb, size_t rows) {
+// weights_first (int8 contract, both forms with weights as the first operand, 96 copies, bf16 out, 25..32 rows): with
+// one plane the 16x16x64 form is as fast or up to 19% faster (N=8192 K=2048 28 rows 94 vs 113 us; K=1024 32 rows 68 vs
+// 72); with two planes and K=1024 it is 14% faster (103..116 vs 119..122), with two planes and K=1536..2048 the wide form
+// wins by 0..8% at most sizes (N=8192 K=1536 28 rows 149 vs 139; K=2048 32 rows 178 vs 169; N=11008 K=2048 5% slower).
+static bool flow_wide(const tk_ctx *ctx, int planes, int rt, size_t nb, size_t rows, bool weights_first) {
   if (rt < 2 || planes > 2 || flow_wide_lds(rt, nb) + kFlowWideExtraLds > kLdsFlowMax) return false;
   if (ctx->flow_mfma == 16) return false;
   if (ctx->flow_mfma == 32) return true;
+  if (weights_first && (planes < 2 || flow_wide_lds(rt, nb) <= 32 * 1024)) return false;
   return rt == 2 && rows > 24 && flow_wide_lds(rt, nb) <= 64 * 1024;
 }
 static int flow_runs_per_wave(bool wide, bool b3, int planes, int rt, size_t rows) {
@@ -793,7 +798,7 @@ static size_t flow_zero_plan(bool wide, bool b3, bool fused, int planes, size_t 
 // zmap_tiles > 0: some plane of the launch carries a zero-chunk map (flow_zero_plan)
 // (b3: flow_lds includes the decode table; ring and runs per wave are the base-3 kernel's own)
 // swap: the launch runs under the int8 contract and the context asks for the second operand order where a form exists
-// (the 16x16x64 kernel from a prepared set of operand rows)
+// (both matrix-instruction forms of the kernel that reads a prepared set of operand rows)
 static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds, size_t rows, size_t zmap_tiles = 0,
                           size_t zmap_nb = 0, bool swap = false) {
   cfg->wide_mfma = wide ? 1 : 0;
@@ -804,7 +809,7 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
   if (zmap_tiles) cfg->lds_bytes += (size_t)cfg->planes * tk_flow_zmap_words(zmap_tiles, zmap_nb) * 4;
   if (wide && cfg->ring > 4) cfg->ring = 4;
   cfg->zmap32 = wide && zmap_tiles ? 1 : 0;
-  cfg->swap = swap && !wide && !b3 ? 1 : 0;
+  cfg->swap = swap && !b3 ? 1 : 0;
 }
 
 // Ring size of a flow launch: the kernels' own rule (tk_flow_ring), except that the 32x32x32 form in eight-wave
@@ -1129,7 +1134,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
   size_t flow_lds = pl.flow_lds;
   if (pl.skinny) {
     b3 = pl.flow_ok && flow_base3(pl.pr, pl.cfg.planes, pl.cfg.rt, flow_lds);
-    wide = !b3 && pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R);
+    wide = !b3 && pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R, mode == TK_MODE_INT8 && ctx->flow_swap);
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
     if (b3) flow_lds += TK_B3_TABLE_BYTES;
     const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt);
@@ -2181,7 +2186,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   }
   bool b3 = flow_ok;
   for (size_t i = 0; i < count && b3; ++i) b3 = flow_base3(plans[i].pr, planes, rt, flds);
-  const bool wide = !b3 && flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max);
+  const bool wide = !b3 && flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
   if (wide) flds = flow_wide_lds(rt, nb_max);
   if (b3) flds += TK_B3_TABLE_BYTES;
   const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds, rt);
@@ -2252,7 +2257,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       gemm_nt2 = ctx->gemm_tiles == 2 || (ctx->gemm_tiles == 0 && total < 4u * (unsigned)ctx->info.compute_units);
     }
     group_gemm_nt = gemm_nt2 ? 2 : 0;
-    const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max);
+    const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
     const int pfw = flow_waves(pflds, rt);
     int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max, tokens_max) : 1;

@@ -339,7 +339,10 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 // the plain forms keep their code and register budgets): as in tk_flow_kernel, a request for a marked chunk goes to
 // the plane's resident all-zero chunk -- the same bytes from the cache instead of from memory, same arithmetic, same
 // bits. The two halves of a wave walk different tiles, so the look-up is per lane; map words behind the row constants.
-template <int P, int RT2, int DR, bool TABLE, bool ZMAP = false>
+// SWAP (int8 contract only): weights as the first operand of the matrix instruction, as in tk_flow_kernel -- accumulator
+// register c of lane L is then channel 8*(c/4) + 4*kappa + c%4 of the pair's 32 for token 32*rt2 + (L & 31): four
+// consecutive registers are four consecutive output channels of one token, written with one store.
+template <int P, int RT2, int DR, bool TABLE, bool ZMAP = false, bool SWAP = false>
 __global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                         const int *__restrict__ wg_prob) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -461,7 +464,16 @@ __global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, 
   for (int s = 0; s < S; ++s) {
     const int t = first + 2 * s + h;  // this lane's tile of the pair
     float sc[P];
-    {
+    float sc4[SWAP ? P : 1][SWAP ? 4 : 1][4];  // SWAP: the scales of this lane's sixteen channels of the pair
+    if constexpr (SWAP) {
+      const int c0 = (first + 2 * s) * 16 + 4 * kappa;
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sc4[p][q][r] = gload(scales[p] + min(c0 + 8 * q + r, hot.n - 1));
+    } else {
       const int n = min(t * 16 + r16, hot.n - 1);
 #pragma unroll
       for (int p = 0; p < P; ++p) sc[p] = gload(scales[p] + n);
@@ -501,7 +513,8 @@ __global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, 
               const v4i b = expand_codes(wj);
 #pragma unroll
               for (int rt2 = 0; rt2 < RT2; ++rt2)
-                acc[rt2][p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_cur[rt2], b, acc[rt2][p], 0, 0, 0);
+                acc[rt2][p] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a_cur[rt2], acc[rt2][p], 0, 0, 0)
+                                   : __builtin_amdgcn_mfma_i32_32x32x32_i8(a_cur[rt2], b, acc[rt2][p], 0, 0, 0);
             }
 #pragma unroll
             for (int rt2 = 0; rt2 < RT2; ++rt2) a_cur[rt2] = a_nxt[rt2];
@@ -511,6 +524,35 @@ __global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, 
       kbg += DR;
     } while (kbg < nbpad);
 
+    if constexpr (SWAP) {
+      const int c0 = (first + 2 * s) * 16 + 4 * kappa;
+      const int *cst_rs = (const int *)cst;
+      const float *cst_as = (const float *)(cst + 256);
+      const uint32_t *cst_fl = (const uint32_t *)(cst + 512);
+#pragma unroll
+      for (int rt2 = 0; rt2 < RT2; ++rt2) {
+        const int m = rt2 * 32 + (lane & 31);
+        if (m >= R) continue;
+        const int rs = cst_rs[m];
+        const float as = cst_as[m];
+        const unsigned fl = cst_fl[m];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n0 = c0 + 8 * q;
+          if (n0 >= hot.n) continue;
+          v4i av[P];
+          float sq[P][4];
+#pragma unroll
+          for (int p = 0; p < P; ++p) {
+            av[p] = v4i{acc[rt2][p][4 * q], acc[rt2][p][4 * q + 1], acc[rt2][p][4 * q + 2], acc[rt2][p][4 * q + 3]};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sq[p][r] = sc4[p][q][r];
+          }
+          flow_epilogue_swapped<P>(hot, pr, m, n0, av, sq, rs, as, fl);
+        }
+      }
+      continue;
+    }
     const int n = t * 16 + r16;
     if (t < n_tiles && n < hot.n) {
 #pragma unroll

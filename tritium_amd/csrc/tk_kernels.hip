@@ -3063,7 +3063,7 @@ hipError_t tk_launch_flow(hipStream_t s, const TkProblem *single, const TkProble
                           const TkLaunchCfg &cfg) {
   if (!cfg.grid) return hipSuccess;
   if (cfg.wide_mfma && cfg.zmap32) return tk_launch_flow32_zmap(s, single, table, wg_prob, cfg);
-  if (cfg.swap && !cfg.wide_mfma && !cfg.fused) return tk_launch_flow_swapped(s, single, table, wg_prob, cfg);
+  if (cfg.swap && !cfg.fused) return tk_launch_flow_swapped(s, single, table, wg_prob, cfg);
   TkProblem dummy = {};
   const TkProblem &sg = single ? *single : dummy;
   switch (cfg.planes) {
