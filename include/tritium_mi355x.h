@@ -594,7 +594,10 @@ int tk_memcpy_h2d(tk_ctx *ctx, void *dst, const void *src, size_t bytes);
 int tk_memcpy_d2h(tk_ctx *ctx, void *dst, const void *src, size_t bytes);
 int tk_memset(tk_ctx *ctx, void *dst, int value, size_t bytes);
 int tk_sync(tk_ctx *ctx);
-void *tk_stream(tk_ctx *ctx); /* the hipStream_t the context launches on */
+/* The hipStream_t the context launches on. Once a call of the same shapes has run, a device-resident linear or
+ * group call enqueues kernels and event waits only (no allocation, no synchronisation, no memset), so a caller may
+ * capture this stream around such calls and replay the graph. */
+void *tk_stream(tk_ctx *ctx);
 typedef struct tk_event tk_event;
 int tk_event_create(tk_ctx *ctx, tk_event **out);
 int tk_event_record(tk_ctx *ctx, tk_event *ev);

@@ -464,6 +464,11 @@ class Mi355xBackend:
     def sync(self):
         _check(self._lib.tk_sync(self._ctx))
 
+    def stream_handle(self):
+        """The hipStream_t every call of this backend enqueues on, as an integer (for callers that record events on
+        it, wait for it from another stream, or capture it into a HIP graph)."""
+        return int(self._lib.tk_stream(self._ctx) or 0)
+
     def linear(self, packed_planes, scales_planes, n, k, format=TernaryFormat.Tq2_0):
         shape = GemmShape(0, n, k)  # upload is called with m = 0 (crates/tritium-nn/src/layers/linear.rs:97)
         planes = [self.upload_weights(p, shape, format) for p in packed_planes]
