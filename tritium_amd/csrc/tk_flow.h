@@ -342,6 +342,8 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 // SWAP (int8 contract only): weights as the first operand of the matrix instruction, as in tk_flow_kernel -- accumulator
 // register c of lane L is then channel 8*(c/4) + 4*kappa + c%4 of the pair's 32 for token 32*rt2 + (L & 31): four
 // consecutive registers are four consecutive output channels of one token, written with one store.
+// (Held to 128 registers -- four waves per SIMD, two eight-wave workgroups per CU at 64 KiB of rows -- the two-plane
+// form on a ring of two spills 10..16 registers and the headline's batch 8 falls from 5.63 to 5.10 TB/s.)
 template <int P, int RT2, int DR, bool TABLE, bool ZMAP = false, bool SWAP = false>
 __global__ __launch_bounds__(512) void tk_flow32_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                         const int *__restrict__ wg_prob) {
