@@ -206,12 +206,17 @@ int tk_weights_format(const tk_weights *w);
  * carry no map and take the plain path. tk_set_zero_skip acts on later uploads: 0 = by the threshold,
  * 1 = never keep a map, 2 = always. tk_weights_zero_chunks reports what an upload found. */
 int tk_set_zero_skip(tk_ctx *ctx, int mode);
-/* Operand order of the matrix instruction in the decode kernel (16x16x64 form) under the int8 contract: 1 (default) =
+/* Operand order of the matrix instruction in the decode kernel (both of its forms) under the int8 contract: 1 (default) =
  * weights first, so that a lane finishes four consecutive output channels of one token and writes them with one store;
  * 0 = activations first (four tokens of one channel per lane, four narrow stores), the order the float contract keeps.
  * Same integers, same epilogue arithmetic, identical bits; a tuning and test knob without a counterpart in the
  * reference. */
 int tk_set_flow_operand_order(tk_ctx *ctx, int weights_first);
+/* Waves per workgroup of the decode kernel where a CU has LDS room for the operand rows of one workgroup only (17..32
+ * rows that take more than 80 KiB): 0 = automatic, 8 = eight (two per SIMD), 16 = sixteen (four per SIMD) wherever a
+ * form of 1024 threads exists (int8 contract with weights first, one or two planes, 16x16x64 form). Same bits; a tuning
+ * and test knob without a counterpart in the reference. */
+int tk_set_flow_workgroup_waves(tk_ctx *ctx, int waves);
 int tk_weights_zero_chunks(const tk_weights *w, size_t *zero, size_t *total, int *map_kept);
 /* Base-3 weight stream: the decode GEMV of the reference that reads TQ1_0's five-trits-per-byte codes and
  * unpacks them in the kernel (crates/tritium-cuda/kernels/tq2_0_add.cu:744-774,796-913). Here: a second

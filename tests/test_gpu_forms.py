@@ -27,6 +27,7 @@ def automatic_dispatch(backend):
     backend.set_gemm_two_by_two(False)
     backend.set_gemm_rows(0)
     backend.set_gemm256_form(-1)
+    backend.set_flow_workgroup_waves(0)
     backend.set_stream_min_groups(backend.info.compute_units)
 
 
@@ -330,6 +331,72 @@ def test_two_row_tiles_in_eight_wave_workgroups(backend, oracle, mode, m, planes
     for x in (dact, out, out2):
         x.free()
     layer.free()
+
+
+@pytest.mark.parametrize("m,planes,k,n", [(24, 1, 4096, 1029), (32, 1, 4864, 520), (17, 2, 5120 - 40, 1029), (32, 2, 4096, 300), (32, 1, 2560, 1029),
+                                          (20, 3, 4096, 134)])
+def test_sixteen_wave_workgroups(backend, oracle, m, planes, k, n):
+    """17..32 int8 rows whose copy in LDS takes more than 80 KiB, so that a CU runs one workgroup: with sixteen waves
+    (tk_flow_kernel<P,2,*,2,*,false,true> at 1024 threads) the bits of eight waves and of the CPU, single launches,
+    groups of members of different widths, a member with a zero-chunk map, a residual. The last two cases have no
+    form of 1024 threads (rows within 80 KiB; three planes): the setting must leave them on eight waves."""
+    print("case sixteen waves", m, planes, k, n, flush=True)
+    backend.set_stream_min_groups(1)
+    backend.set_decode_kernel(3)
+    rng = np.random.default_rng(m * 1000 + planes * 100 + k + n)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    act[m // 2, 7] = np.inf  # a token that the kernel recomputes in the reference's order
+    dact = backend.to_device(act, "f32")
+    ws, scs, packed = _planes(rng, n, k, planes)
+    ws2 = [w.copy() for w in ws]
+    ws2[-1][16:64, :] = 0
+    ws2[-1][:, 256:1024] = 0
+    packed2 = [T.pack_rows(w, n, k) for w in ws2]
+    n3 = 136
+    ws3, scs3, packed3 = _planes(rng, n3, k, planes)
+    layer = backend.linear(packed, scs, n, k)
+    backend.set_zero_skip(2)
+    layer2 = backend.linear(packed2, scs, n, k)
+    backend.set_zero_skip(0)
+    layer3 = backend.linear(packed3, scs3, n3, k)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    dres = backend.to_device(res, "f32")
+    want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+    want2 = oracle.cpu_linear_a8_planes(packed2, FMT_TQ2_0, scs, act, m, n, k)
+    want3 = oracle.cpu_linear_a8_planes(packed3, FMT_TQ2_0, scs3, act, m, n3, k)
+    def like_cpu(got, ref):
+        got, ref = got.reshape(-1), np.asarray(ref, np.float32).reshape(-1)
+        fin = ~np.isnan(ref)
+        return bool((np.isnan(got) == np.isnan(ref)).all()) and same_bits(got[fin], ref[fin])
+    outs = {}
+    try:
+        for waves in (16, 8):
+            backend.set_flow_workgroup_waves(waves)
+            o1, o2, o3, ores, o16 = (backend.empty(m * n, "f32"), backend.empty(m * n, "f32"), backend.empty(m * n3, "f32"),
+                                     backend.empty(m * n, "f32"), backend.empty(m * n, "bf16"))
+            backend.linear_a8(layer, dact, m, o1)
+            assert backend.last_kernel() == "flow", backend.last_kernel()
+            backend.linear_a8(layer, dact, m, o16)
+            backend.linear_a8_residual(layer, dact, m, dres, ores)
+            single = o1.to_host().copy()
+            grp = backend.group([(layer, dact, m, o1), (layer2, dact, m, o2), (layer3, dact, m, o3)], 1, "f32", "f32")
+            grp.launch()
+            grp.launch()
+            outs[waves] = [single] + [x.to_host().copy() for x in (o1, o2, o3, ores, o16)]
+            grp.destroy()
+            for x in (o1, o2, o3, ores, o16):
+                x.free()
+    finally:
+        backend.set_flow_workgroup_waves(0)
+    for a, b in zip(outs[16], outs[8]):
+        assert same_bits(a, b)
+    assert like_cpu(outs[16][0], want) and like_cpu(outs[16][1], want)
+    assert like_cpu(outs[16][2], want2) and like_cpu(outs[16][3], want3)
+    assert like_cpu(outs[16][4], (res + want.reshape(m, n)).astype(np.float32))
+    for x in (dact, dres):
+        x.free()
+    for l in (layer, layer2, layer3):
+        l.free()
 
 
 @pytest.mark.parametrize("m", [1, 3, 4, 9, 16, 20, 40, 64])

@@ -65,6 +65,7 @@ SIGNATURES = {
     "tk_weights_format": (C.c_int, [vp]),
     "tk_set_zero_skip": (C.c_int, [vp, C.c_int]),
     "tk_set_flow_operand_order": (C.c_int, [vp, C.c_int]),
+    "tk_set_flow_workgroup_waves": (C.c_int, [vp, C.c_int]),
     "tk_set_prep_team_rows": (C.c_int, [vp, C.c_int]),
     "tk_set_gemm_two_by_two": (C.c_int, [vp, C.c_int]),
     "tk_set_base3_stream": (C.c_int, [vp, C.c_int]),

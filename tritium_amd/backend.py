@@ -633,6 +633,11 @@ class Mi355xBackend:
         store per lane), 0 activations first (same bits)."""
         _check(self._lib.tk_set_flow_operand_order(self._ctx, weights_first))
 
+    def set_flow_workgroup_waves(self, waves):
+        """Decode kernel, 17..32 operand rows beyond 80 KiB (one workgroup per CU): 0 automatic, 8 or 16 waves per
+        workgroup (same bits)."""
+        _check(self._lib.tk_set_flow_workgroup_waves(self._ctx, waves))
+
     def set_base3_stream(self, mode):
         """Later uploads: 0 no base-3 copy, 1 TQ1_0 uploads keep one beside the 2-bit codes, 2 every upload."""
         _check(self._lib.tk_set_base3_stream(self._ctx, mode))

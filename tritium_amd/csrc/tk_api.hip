@@ -97,6 +97,7 @@ struct tk_ctx {
   bool gemm256_form_forced = false;  // tk_set_gemm256_form was called: automatic launches keep that form
   int gemm256_form = 0;    // the 256-row kernel: 0 = 4 waves x 224 outputs, 1 = 8 waves x 224, 2 = 4 waves x (128 | 96), two workgroups per CU
   int zero_skip = 0;       // uploads: 0 = keep a zero-chunk map when at least 0.5% of the chunks are zero, 1 = never, 2 = always
+  int flow_wg16 = -1;      // flow kernel, sixteen-wave workgroups where a CU holds one workgroup's rows only: -1 = automatic, 0 = never, 1 = wherever a form exists
   int flow_swap = 1;       // flow kernel, int8 contract: 1 = weights as the first operand of the matrix instruction (one wide store per lane), 0 = activations first
   int base3 = 0;           // uploads: 0 = no base-3 stream, 1 = TQ1_0 uploads keep one beside the 2-bit codes, 2 = every upload
   unsigned *d_count = nullptr;  // a device counter for the uploads
@@ -444,6 +445,14 @@ extern "C" int tk_set_flow_operand_order(tk_ctx *ctx, int weights_first) {
   return TK_OK;
 }
 
+extern "C" int tk_set_flow_workgroup_waves(tk_ctx *ctx, int waves) {
+  if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_flow_workgroup_waves: null context");
+  if (waves != 0 && waves != 8 && waves != 16) return tk_fail(TK_ERR_INVALID_INPUT, "flow_workgroup_waves=%d - use 0 (automatic), 8 or 16", waves);
+  std::lock_guard<std::mutex> lk(ctx->mu);
+  ctx->flow_wg16 = waves == 16 ? 1 : (waves == 8 ? 0 : -1);
+  return TK_OK;
+}
+
 extern "C" int tk_set_base3_stream(tk_ctx *ctx, int mode) {
   if (!ctx) return tk_fail(TK_ERR_INVALID_INPUT, "tk_set_base3_stream: null context");
   if (mode < 0 || mode > 2) return tk_fail(TK_ERR_INVALID_INPUT, "base3_stream=%d - use 0 (off), 1 (TQ1_0 uploads) or 2 (every upload)", mode);
@@ -748,7 +757,26 @@ static const size_t kLdsFlowMax = 160 * 1024;
 // 22 / 24 int8 rows x 6912 outputs 3.35 -> 4.36 / 3.30 -> 4.32 TB/s, 2560 outputs 3.39 -> 4.20, six float tokens
 // 3.74 -> 4.83; the 32x32x32 form at 64 KiB (two planes K=2048, eight float tokens) 5.32 -> 5.70 with runs of four
 // pairs on a ring of two.
-static int flow_waves(size_t lds, int rt) { return lds > (rt >= 2 ? kLdsFlowMax / 3 : 64 * 1024) ? 8 : 4; }
+static int flow_waves(size_t lds, int rt, bool sixteen = false) {
+  if (sixteen && rt == 2 && lds > kLdsFlowMax / 2) return 16;
+  return lds > (rt >= 2 ? kLdsFlowMax / 3 : 64 * 1024) ? 8 : 4;
+}
+// Sixteen-wave workgroups for 17..32 operand rows that take more than half of the LDS, so that a CU runs one workgroup:
+// four waves per SIMD instead of two. The forms that exist with 1024 threads are those that stay within 128 registers by
+// themselves: int8 contract with weights first, one or two planes, two row tiles, ring of two. Measured, 64 layer copies
+// per launch, eight -> sixteen waves (the eight on the ring they would pick): one plane K=5120 N=5120 17 / 24 / 32 rows
+// 113 -> 102 / 118 -> 107 / 124 -> 112 us; K=4096 N=11008 24 / 32 rows 157 -> 149 / 167 -> 155; K=3584 N=8192 105 -> 102 /
+// 108 -> 107; K=3072 N=8192 32 rows 94 -> 92. Two planes are mixed -- K=4096 N=4096 24 / 32 rows 113 -> 108 / 116 -> 111,
+// K=3072 N=8192 32 rows 170 -> 173, K=5120 N=17408 17 / 24 / 32 rows 565 -> 602 / 585 -> 621 / 657 -> 636 (their eight-wave
+// launches sit on a ring of four, which the sixteen-wave form has no registers for) -- and keep eight waves unless
+// asked. A ring of three under sixteen waves is 2-6% slower than the ring of two. Launches too small to give every
+// CU a workgroup of sixteen waves with runs of two tiles keep eight.
+static bool flow_sixteen(const tk_ctx *ctx, bool int8_mode, bool wide, bool b3, int planes, size_t tiles, int tw) {
+  if (!ctx->flow_wg16 || !int8_mode || !ctx->flow_swap || wide || b3 || planes > 2) return false;
+  if (ctx->flow_ring != 0 && ctx->flow_ring != 2) return false;
+  if (ctx->flow_wg16 > 0) return true;
+  return planes == 1 && tiles >= (size_t)ctx->info.compute_units * 16u * (size_t)tw * 2u;
+}
 // widest row stride any kernel asks of the staged operand rows of an R-row problem
 static size_t kPrepRowsMax(size_t R) { return R + 16 > 64 ? R + 16 : 64; }
 
@@ -822,6 +850,7 @@ static void flow_cfg_form(TkLaunchCfg *cfg, bool wide, bool b3, size_t flow_lds,
 // no difference either way.
 static int pick_flow_ring(const tk_ctx *ctx, const int *nbs, const double *wts, int count, int rt, int rows, int tw,
                           bool wide, int waves, size_t lds, int planes) {
+  if (waves >= 16) return 2;  // (the only forms with 1024 threads)
   if (ctx->flow_ring) return ctx->flow_ring;
   if (wide && waves >= 8 && lds <= 64 * 1024) return 2;
   int nb_max = 0;
@@ -848,7 +877,8 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * (b3 ? TK_B3_CHUNK_BYTES : TK_CHUNK_BYTES);
-  size_t target = lds_bytes * (size_t)waves * (size_t)waves / (waves >= 8 && lds_bytes > 64 * 1024 ? 2 : 4);
+  const size_t w8 = waves > 8 ? 8 : (size_t)waves;  // (a sixteen-wave workgroup: twice the target of eight waves)
+  size_t target = lds_bytes * w8 * w8 / (waves >= 8 && lds_bytes > 64 * 1024 ? 2 : 4) * ((size_t)waves / w8);
   if (target < 64 * 1024) target = 64 * 1024;
   size_t s = 1;
   while (s < 16 && per_s * (2 * s) * tile_bytes <= target) s *= 2;
@@ -1137,7 +1167,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     wide = !b3 && pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R, mode == TK_MODE_INT8 && ctx->flow_swap);
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
     if (b3) flow_lds += TK_B3_TABLE_BYTES;
-    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt);
+    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt, flow_sixteen(ctx, mode == TK_MODE_INT8, wide, b3, pl.cfg.planes, (size_t)pl.pr.n_tiles, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R)));
     run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R, m);
     const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
@@ -1272,7 +1302,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
-    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt);
+    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt, flow_sixteen(ctx, mode == TK_MODE_INT8, wide, b3, pl.cfg.planes, (size_t)pl.pr.n_tiles, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R)));
     cfg.ring = pick_flow_ring(ctx, &pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R), wide, cfg.waves, flow_lds, pl.cfg.planes);
     const size_t ztiles = flow_zero_plan(wide, b3, fused, cfg.planes, flow_lds,
                                          pr.zskip ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0, nb);
@@ -2189,7 +2219,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   const bool wide = !b3 && flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
   if (wide) flds = flow_wide_lds(rt, nb_max);
   if (b3) flds += TK_B3_TABLE_BYTES;
-  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds, rt);
+  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds, rt, flow_sixteen(ctx, kmode == TK_MODE_INT8, wide, b3, planes, tiles, flow_runs_per_wave(wide, b3, planes, rt, rows_max)));
   int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, b3, rows_max, tokens_max);
   {
     std::vector<unsigned> member_tiles(count);
@@ -2259,7 +2289,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     group_gemm_nt = gemm_nt2 ? 2 : 0;
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
-    const int pfw = flow_waves(pflds, rt);
+    const int pfw = flow_waves(pflds, rt, flow_sixteen(ctx, kmode == TK_MODE_INT8, pwide, false, planes, ptiles, flow_runs_per_wave(pwide, false, planes, rt, prows_max)));
     int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max, tokens_max) : 1;
     {
       std::vector<unsigned> member_tiles;
