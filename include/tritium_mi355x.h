@@ -214,8 +214,9 @@ int tk_set_zero_skip(tk_ctx *ctx, int mode);
 int tk_set_flow_operand_order(tk_ctx *ctx, int weights_first);
 /* Waves per workgroup of the decode kernel where a CU has LDS room for the operand rows of one workgroup only (17..32
  * rows that take more than 80 KiB): 0 = automatic, 8 = eight (two per SIMD), 16 = sixteen (four per SIMD) wherever a
- * form of 1024 threads exists (int8 contract with weights first, one or two planes, 16x16x64 form). Same bits; a tuning
- * and test knob without a counterpart in the reference. */
+ * form of 1024 threads exists (16x16x64 form, one or two planes: every launch under the int8 contract with weights
+ * first, grouped launches otherwise). Automatic: sixteen for one plane when the launch has tiles for every CU. Same
+ * bits; a tuning and test knob without a counterpart in the reference. */
 int tk_set_flow_workgroup_waves(tk_ctx *ctx, int waves);
 int tk_weights_zero_chunks(const tk_weights *w, size_t *zero, size_t *total, int *map_kept);
 /* Base-3 weight stream: the decode GEMV of the reference that reads TQ1_0's five-trits-per-byte codes and

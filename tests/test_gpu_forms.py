@@ -337,7 +337,7 @@ def test_two_row_tiles_in_eight_wave_workgroups(backend, oracle, mode, m, planes
                                           (20, 3, 4096, 134)])
 def test_sixteen_wave_workgroups(backend, oracle, m, planes, k, n):
     """17..32 int8 rows whose copy in LDS takes more than 80 KiB, so that a CU runs one workgroup: with sixteen waves
-    (tk_flow_kernel<P,2,*,2,*,false,true> at 1024 threads) the bits of eight waves and of the CPU, single launches,
+    (tk_flow_kernel<P,2,*,2,*,false,*> at 1024 threads; both operand orders) the bits of eight waves and of the CPU, single launches,
     groups of members of different widths, a member with a zero-chunk map, a residual. The last two cases have no
     form of 1024 threads (rows within 80 KiB; three planes): the setting must leave them on eight waves."""
     print("case sixteen waves", m, planes, k, n, flush=True)
@@ -384,10 +384,18 @@ def test_sixteen_wave_workgroups(backend, oracle, m, planes, k, n):
             grp.launch()
             outs[waves] = [single] + [x.to_host().copy() for x in (o1, o2, o3, ores, o16)]
             grp.destroy()
+            backend.set_flow_operand_order(0)  # activations first: the table forms have 1024 threads too
+            grp = backend.group([(layer, dact, m, o1), (layer2, dact, m, o2), (layer3, dact, m, o3)], 1, "f32", "f32")
+            grp.launch()
+            backend.set_flow_operand_order(1)
+            for got, ref in zip((o1, o2, o3), outs[waves][1:4]):
+                assert same_bits(got.to_host(), ref)
+            grp.destroy()
             for x in (o1, o2, o3, ores, o16):
                 x.free()
     finally:
         backend.set_flow_workgroup_waves(0)
+        backend.set_flow_operand_order(1)
     for a, b in zip(outs[16], outs[8]):
         assert same_bits(a, b)
     assert like_cpu(outs[16][0], want) and like_cpu(outs[16][1], want)
@@ -397,6 +405,51 @@ def test_sixteen_wave_workgroups(backend, oracle, m, planes, k, n):
         x.free()
     for l in (layer, layer2, layer3):
         l.free()
+
+
+@pytest.mark.parametrize("m,planes,k", [(5, 1, 4096), (8, 1, 4864), (6, 2, 4096), (8, 1, 2048)])
+def test_sixteen_wave_workgroups_float_contract(backend, oracle, m, planes, k):
+    """5..8 float tokens (20..32 digit rows) beyond 80 KiB in grouped launches: the activations-first forms that read a
+    problem table also exist with 1024 threads. Bits of eight waves, bounds of the CPU; single launches (no such
+    form) and rows within 80 KiB (last case) stay on eight waves whatever is asked."""
+    print("case sixteen waves float", m, planes, k, flush=True)
+    backend.set_stream_min_groups(1)
+    backend.set_decode_kernel(3)
+    rng = np.random.default_rng(m * 1000 + planes * 100 + k)
+    act = rng.standard_normal((m, k)).astype(np.float32)
+    dact = backend.to_device(f32_to_bf16_bits(act), "bf16")
+    act = bf16_bits_to_f32(f32_to_bf16_bits(act)).reshape(m, k)
+    sets = []
+    for n in (1029, 136):
+        ws, scs, packed = _planes(rng, n, k, planes)
+        sets.append((n, scs, packed, backend.linear(packed, scs, n, k)))
+    outs = {}
+    try:
+        for waves in (16, 8):
+            backend.set_flow_workgroup_waves(waves)
+            o = [backend.empty(m * n, "f32") for n, *_ in sets]
+            single = backend.empty(m * sets[0][0], "f32")
+            grp = backend.group([(st[3], dact, m, oo) for st, oo in zip(sets, o)], 0, "bf16", "f32")
+            grp.launch()
+            grp.launch()
+            backend.linear_float(sets[0][3], dact, m, single)
+            assert backend.last_kernel() in ("flow", "flow32"), backend.last_kernel()
+            outs[waves] = [x.to_host().copy() for x in o + [single]]
+            grp.destroy()
+            for x in o + [single]:
+                x.free()
+    finally:
+        backend.set_flow_workgroup_waves(0)
+    for a, b in zip(outs[16], outs[8]):
+        assert same_bits(a, b)
+    assert same_bits(outs[16][0], outs[16][2])  # grouped and single launch
+    for (n, scs, packed, _), got in zip(sets, outs[16]):
+        want = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, act, m, n, k)
+        assert rel_err(got.reshape(m, n), want) <= 1e-3
+        assert accepts(got.reshape(m, n), want, rel=1e-4, floor=1.0).all()
+    dact.free()
+    for st in sets:
+        st[3].free()
 
 
 @pytest.mark.parametrize("m", [1, 3, 4, 9, 16, 20, 40, 64])

@@ -145,6 +145,8 @@ REGISTER_BUDGETS = (
     ("tk_flow_kernelILi2ELi4ELi2ELi2ELb1ELb0ELb0E", 256),   # two planes, 33..64 rows
     ("tk_flow_kernelILi1ELi2ELi2ELi2ELb1ELb0ELb1E", 128),   # weights first, two row tiles on a ring of two: the forms of 1024 threads
     ("tk_flow_kernelILi2ELi2ELi1ELi2ELb1ELb0ELb1E", 128),   # (sixteen waves per workgroup; no spills)
+    ("tk_flow_kernelILi1ELi2ELi2ELi2ELb1ELb0ELb0E", 128),   # ... activations first, from a problem table
+    ("tk_flow_kernelILi2ELi2ELi1ELi2ELb1ELb0ELb0E", 128),
     ("tk_gemm32_kernelILi1ELi2ELb0ELb0E", 168),     # prefill, one plane (three waves per SIMD by design)
     ("tk_gemm32_kernelILi1ELi4ELb0ELb0E", 168),
     ("tk_gemm32_kernelILi3ELi2ELb0ELb0E", 256),     # prefill, three planes (two waves per SIMD)

@@ -763,7 +763,9 @@ static int flow_waves(size_t lds, int rt, bool sixteen = false) {
 }
 // Sixteen-wave workgroups for 17..32 operand rows that take more than half of the LDS, so that a CU runs one workgroup:
 // four waves per SIMD instead of two. The forms that exist with 1024 threads are those that stay within 128 registers by
-// themselves: int8 contract with weights first, one or two planes, two row tiles, ring of two. Measured, 64 layer copies
+// themselves: two row tiles of one or two planes on a ring of two, with weights first (int8 contract) or, activations
+// first, from a problem table (float contract 5 / 6 / 8 tokens in groups: one plane K=5120 N=5120 102 -> 94.5 / 104 -> 96 /
+// 109 -> 100 us, K=4096 N=11008 129 -> 129 / 135 -> 129.5 / 138.5 -> 133.5). Measured under the int8 contract, 64 layer copies
 // per launch, eight -> sixteen waves (the eight on the ring they would pick): one plane K=5120 N=5120 17 / 24 / 32 rows
 // 113 -> 102 / 118 -> 107 / 124 -> 112 us; K=4096 N=11008 24 / 32 rows 157 -> 149 / 167 -> 155; K=3584 N=8192 105 -> 102 /
 // 108 -> 107; K=3072 N=8192 32 rows 94 -> 92. Two planes are mixed -- K=4096 N=4096 24 / 32 rows 113 -> 108 / 116 -> 111,
@@ -771,8 +773,9 @@ static int flow_waves(size_t lds, int rt, bool sixteen = false) {
 // launches sit on a ring of four, which the sixteen-wave form has no registers for) -- and keep eight waves unless
 // asked. A ring of three under sixteen waves is 2-6% slower than the ring of two. Launches too small to give every
 // CU a workgroup of sixteen waves with runs of two tiles keep eight.
-static bool flow_sixteen(const tk_ctx *ctx, bool int8_mode, bool wide, bool b3, int planes, size_t tiles, int tw) {
-  if (!ctx->flow_wg16 || !int8_mode || !ctx->flow_swap || wide || b3 || planes > 2) return false;
+static bool flow_sixteen(const tk_ctx *ctx, bool int8_mode, bool table, bool wide, bool b3, int planes, size_t tiles, int tw) {
+  if (!ctx->flow_wg16 || wide || b3 || planes > 2) return false;
+  if (!(int8_mode && ctx->flow_swap) && !table) return false;  // (activations first: only the forms that read a problem table)
   if (ctx->flow_ring != 0 && ctx->flow_ring != 2) return false;
   if (ctx->flow_wg16 > 0) return true;
   return planes == 1 && tiles >= (size_t)ctx->info.compute_units * 16u * (size_t)tw * 2u;
@@ -1167,7 +1170,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     wide = !b3 && pl.flow_ok && flow_wide(ctx, pl.cfg.planes, pl.cfg.rt, nb, R, mode == TK_MODE_INT8 && ctx->flow_swap);
     if (wide) flow_lds = flow_wide_lds(pl.cfg.rt, nb);
     if (b3) flow_lds += TK_B3_TABLE_BYTES;
-    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt, flow_sixteen(ctx, mode == TK_MODE_INT8, wide, b3, pl.cfg.planes, (size_t)pl.pr.n_tiles, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R)));
+    const int fw = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt, flow_sixteen(ctx, mode == TK_MODE_INT8, false, wide, b3, pl.cfg.planes, (size_t)pl.pr.n_tiles, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R)));
     run_tiles = flow_run_tiles(ctx, (unsigned)pl.pr.n_tiles, pl.cfg.planes, pl.cfg.rt, fw, flow_lds, nb, wide, b3, R, m);
     const unsigned per_wg = (unsigned)fw * (unsigned)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (unsigned)run_tiles;
     flow_groups = ((unsigned)pl.pr.n_tiles + per_wg - 1) / per_wg;
@@ -1302,7 +1305,7 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     TkLaunchCfg cfg = pl.cfg;
     cfg.grid = flow_groups;
     cfg.lds_bytes = flow_lds;
-    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt, flow_sixteen(ctx, mode == TK_MODE_INT8, wide, b3, pl.cfg.planes, (size_t)pl.pr.n_tiles, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R)));
+    cfg.waves = b3 ? tk_flow3_waves(pl.cfg.rt) : flow_waves(flow_lds, pl.cfg.rt, flow_sixteen(ctx, mode == TK_MODE_INT8, false, wide, b3, pl.cfg.planes, (size_t)pl.pr.n_tiles, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R)));
     cfg.ring = pick_flow_ring(ctx, &pr.nb, nullptr, 1, pl.cfg.rt, pr.R, flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R), wide, cfg.waves, flow_lds, pl.cfg.planes);
     const size_t ztiles = flow_zero_plan(wide, b3, fused, cfg.planes, flow_lds,
                                          pr.zskip ? (size_t)cfg.waves * (size_t)flow_runs_per_wave(wide, b3, pl.cfg.planes, pl.cfg.rt, R) * (size_t)run_tiles : 0, nb);
@@ -2219,7 +2222,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   const bool wide = !b3 && flow_ok && flow_wide(ctx, planes, rt, nb_max, rows_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
   if (wide) flds = flow_wide_lds(rt, nb_max);
   if (b3) flds += TK_B3_TABLE_BYTES;
-  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds, rt, flow_sixteen(ctx, kmode == TK_MODE_INT8, wide, b3, planes, tiles, flow_runs_per_wave(wide, b3, planes, rt, rows_max)));
+  const int fw = b3 ? tk_flow3_waves(rt) : flow_waves(flds, rt, flow_sixteen(ctx, kmode == TK_MODE_INT8, true, wide, b3, planes, tiles, flow_runs_per_wave(wide, b3, planes, rt, rows_max)));
   int run_tiles = flow_run_tiles(ctx, tiles, planes, rt, fw, flds, nb_max, wide, b3, rows_max, tokens_max);
   {
     std::vector<unsigned> member_tiles(count);
@@ -2289,7 +2292,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     group_gemm_nt = gemm_nt2 ? 2 : 0;
     const bool pwide = ptiles && flow_wide(ctx, planes, rt, pnb_max, prows_max, kmode == TK_MODE_INT8 && ctx->flow_swap);
     if (pwide) pflds = flow_wide_lds(rt, pnb_max);
-    const int pfw = flow_waves(pflds, rt, flow_sixteen(ctx, kmode == TK_MODE_INT8, pwide, false, planes, ptiles, flow_runs_per_wave(pwide, false, planes, rt, prows_max)));
+    const int pfw = flow_waves(pflds, rt, flow_sixteen(ctx, kmode == TK_MODE_INT8, true, pwide, false, planes, ptiles, flow_runs_per_wave(pwide, false, planes, rt, prows_max)));
     int prun = ptiles ? flow_run_tiles(ctx, ptiles, planes, rt, pfw, pflds, pnb_max, pwide, false, prows_max, tokens_max) : 1;
     {
       std::vector<unsigned> member_tiles;

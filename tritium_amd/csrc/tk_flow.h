@@ -26,9 +26,11 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
 // three (168 registers) -- left alone it takes 169, which costs a third of the waves in flight and 8% of
 // the rate at 9..16 operand rows.
 // Workgroups of sixteen waves (a CU whose LDS holds the rows of one workgroup only then still runs four waves per SIMD)
-// exist for the forms that stay within 128 registers by themselves: weights first, two row tiles of one or two planes
-// on a ring of two.
-#define TK_FLOW_MAX_THREADS(P, RT, DR, SWAP) (((SWAP) && (RT) == 2 && (P) <= 2 && (DR) == 2) ? 1024 : 512)
+// exist for the forms that stay within 128 registers by themselves: two row tiles of one or two planes on a ring of
+// two, with weights first (107 / 100 registers) or, activations first, from a problem table (126 / 124; the form for a
+// single problem takes 149).
+#define TK_FLOW_MAX_THREADS(P, RT, DR, TABLE, SWAP) \
+  (((RT) == 2 && (P) <= 2 && (DR) == 2 && ((SWAP) || (TABLE))) ? 1024 : 512)
 #define TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP) ((!(SWAP) && (P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
 // FUSED (one row tile, a single problem, 256 threads): the kernel builds the operand rows of its one to four
 // tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of two.
@@ -39,7 +41,7 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
 // four 2- or 4-byte stores to four output rows, and a decode launch of 8..64 tokens is held back by the number of
 // store instructions it issues, not by their bytes.
 template <int P, int RT, int TW, int DR, bool TABLE, bool FUSED = false, bool SWAP = false>
-__global__ __launch_bounds__(TK_FLOW_MAX_THREADS(P, RT, DR, SWAP)) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
+__global__ __launch_bounds__(TK_FLOW_MAX_THREADS(P, RT, DR, TABLE, SWAP)) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                       const int *__restrict__ wg_prob) {
   static_assert(!FUSED || (RT == 1 && !TABLE), "the fused form: one row tile, one problem");
   static_assert(!(FUSED && SWAP), "the fused form keeps the first operand order");
