@@ -768,17 +768,18 @@ static int flow_waves(size_t lds, int rt, bool sixteen = false) {
 // 109 -> 100 us, K=4096 N=11008 129 -> 129 / 135 -> 129.5 / 138.5 -> 133.5). Measured under the int8 contract, 64 layer copies
 // per launch, eight -> sixteen waves (the eight on the ring they would pick): one plane K=5120 N=5120 17 / 24 / 32 rows
 // 113 -> 102 / 118 -> 107 / 124 -> 112 us; K=4096 N=11008 24 / 32 rows 157 -> 149 / 167 -> 155; K=3584 N=8192 105 -> 102 /
-// 108 -> 107; K=3072 N=8192 32 rows 94 -> 92. Two planes are mixed -- K=4096 N=4096 24 / 32 rows 113 -> 108 / 116 -> 111,
-// K=3072 N=8192 32 rows 170 -> 173, K=5120 N=17408 17 / 24 / 32 rows 565 -> 602 / 585 -> 621 / 657 -> 636 (their eight-wave
-// launches sit on a ring of four, which the sixteen-wave form has no registers for) -- and keep eight waves unless
-// asked. A ring of three under sixteen waves is 2-6% slower than the ring of two. Launches too small to give every
-// CU a workgroup of sixteen waves with runs of two tiles keep eight.
+// 108 -> 107; K=3072 N=8192 32 rows 94 -> 92. With the run length of each chosen by flow_run_tiles' model of such launches
+// (32 layer copies, 24 / 32 rows, eight -> sixteen waves): three planes K=5120 N=17408 397 -> 387 / 407 -> 395, N=5120
+// 133 -> 123 / 138 -> 125; two planes K=5120 N=17408 286 -> 268 / 295 -> 278, K=4096 N=4096 61 -> 56 / 64 -> 57; one plane
+// K=5120 N=17408 164 -> 153 / 174 -> 156, K=4096 N=11008 88 -> 80 / 93 -> 84. A ring of three under sixteen waves is 2-6%
+// slower than the ring of two. Launches too small to give every CU a workgroup of sixteen waves with runs of two
+// tiles keep eight.
 static bool flow_sixteen(const tk_ctx *ctx, bool int8_mode, bool table, bool wide, bool b3, int planes, size_t tiles, int tw) {
-  if (!ctx->flow_wg16 || wide || b3 || planes > 2) return false;
+  if (!ctx->flow_wg16 || wide || b3 || planes > (int8_mode && ctx->flow_swap ? 3 : 2)) return false;
   if (!(int8_mode && ctx->flow_swap) && !table) return false;  // (activations first: only the forms that read a problem table)
   if (ctx->flow_ring != 0 && ctx->flow_ring != 2) return false;
   if (ctx->flow_wg16 > 0) return true;
-  return planes == 1 && tiles >= (size_t)ctx->info.compute_units * 16u * (size_t)tw * 2u;
+  return tiles >= (size_t)ctx->info.compute_units * 16u * (size_t)tw * 2u;
 }
 // widest row stride any kernel asks of the staged operand rows of an R-row problem
 static size_t kPrepRowsMax(size_t R) { return R + 16 > 64 ? R + 16 : 64; }
@@ -880,6 +881,32 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * (b3 ? TK_B3_CHUNK_BYTES : TK_CHUNK_BYTES);
+  // Two row tiles whose rows leave a CU room for ONE workgroup (more than 80 KiB; hidden sizes from 2816 on): the launch
+  // is a few rounds of one workgroup per CU, and what decides is how the workgroup count falls on the CUs. Cost of a
+  // run length = (rounds + 1/4) x (bytes a workgroup streams + bytes it stages), a last partial round counting for at
+  // least three quarters (its workgroups share the memory system among fewer: 160 of 256 CUs busy measured as fast as
+  // all) and the quarter standing for the start and the end of the launch, where every CU stages or drains at once
+  // (one round of exactly 256 workgroups measured 13% slower than two rounds of half their length).
+  // Measured against this model over N in {5120, 11008, 17408}, K in {4096, 5120}, one to three planes, 24 / 32 int8
+  // rows, 32 layer copies, runs of 1 / 2 / 4 / 8 tiles, eight- and sixteen-wave workgroups: the model's choice is the
+  // measured best or within 4% of it, where the rule below (fitted to K = 2048) was 15-29% behind (three planes N=17408
+  // K=5120 24 rows, eight waves: 423 / 400 / 420 / 472 us, rule: 8 tiles; one plane, sixteen waves: 153 / 165 / 196 / 177).
+  if (!b3 && rt == 2 && waves >= 8 && lds_bytes > kLdsFlowMax / 2) {
+    const double cus = (double)ctx->info.compute_units;
+    double best = 0.0;
+    int best_s = 1;
+    for (int c = 1; c <= 16; c *= 2) {
+      const double wgs = (double)((total_tiles + per_s * (size_t)c - 1) / (per_s * (size_t)c));
+      const double full = (double)(size_t)(wgs / cus), rem = wgs - full * cus;
+      const double rounds = 0.25 + full + (rem > 0.0 ? (rem > 0.75 * cus ? rem : 0.75 * cus) / cus : 0.0);
+      const double cost = rounds * ((double)c * (double)per_s * (double)tile_bytes + (double)lds_bytes);
+      if (c == 1 || cost < best) {
+        best = cost;
+        best_s = c;
+      }
+    }
+    return best_s;
+  }
   const size_t w8 = waves > 8 ? 8 : (size_t)waves;  // (a sixteen-wave workgroup: twice the target of eight waves)
   size_t target = lds_bytes * w8 * w8 / (waves >= 8 && lds_bytes > 64 * 1024 ? 2 : 4) * ((size_t)waves / w8);
   if (target < 64 * 1024) target = 64 * 1024;

@@ -30,7 +30,7 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
 // two, with weights first (107 / 100 registers) or, activations first, from a problem table (126 / 124; the form for a
 // single problem takes 149).
 #define TK_FLOW_MAX_THREADS(P, RT, DR, TABLE, SWAP) \
-  (((RT) == 2 && (P) <= 2 && (DR) == 2 && ((SWAP) || (TABLE))) ? 1024 : 512)
+  (((RT) == 2 && ((P) <= 2 || ((P) == 3 && (SWAP))) && (DR) == 2 && ((SWAP) || (TABLE))) ? 1024 : 512)
 #define TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP) ((!(SWAP) && (P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
 // FUSED (one row tile, a single problem, 256 threads): the kernel builds the operand rows of its one to four
 // tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of two.
