@@ -881,32 +881,6 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   if (ctx->flow_run_tiles > 0) return ctx->flow_run_tiles;
   const size_t per_s = (size_t)waves * (size_t)flow_runs_per_wave(wide, b3, planes, rt, rows);
   const size_t tile_bytes = (size_t)planes * (nb ? nb : 1) * (b3 ? TK_B3_CHUNK_BYTES : TK_CHUNK_BYTES);
-  // Two row tiles whose rows leave a CU room for ONE workgroup (more than 80 KiB; hidden sizes from 2816 on): the launch
-  // is a few rounds of one workgroup per CU, and what decides is how the workgroup count falls on the CUs. Cost of a
-  // run length = (rounds + 1/4) x (bytes a workgroup streams + bytes it stages), a last partial round counting for at
-  // least three quarters (its workgroups share the memory system among fewer: 160 of 256 CUs busy measured as fast as
-  // all) and the quarter standing for the start and the end of the launch, where every CU stages or drains at once
-  // (one round of exactly 256 workgroups measured 13% slower than two rounds of half their length).
-  // Measured against this model over N in {5120, 11008, 17408}, K in {4096, 5120}, one to three planes, 24 / 32 int8
-  // rows, 32 layer copies, runs of 1 / 2 / 4 / 8 tiles, eight- and sixteen-wave workgroups: the model's choice is the
-  // measured best or within 4% of it, where the rule below (fitted to K = 2048) was 15-29% behind (three planes N=17408
-  // K=5120 24 rows, eight waves: 423 / 400 / 420 / 472 us, rule: 8 tiles; one plane, sixteen waves: 153 / 165 / 196 / 177).
-  if (!b3 && rt == 2 && waves >= 8 && lds_bytes > kLdsFlowMax / 2) {
-    const double cus = (double)ctx->info.compute_units;
-    double best = 0.0;
-    int best_s = 1;
-    for (int c = 1; c <= 16; c *= 2) {
-      const double wgs = (double)((total_tiles + per_s * (size_t)c - 1) / (per_s * (size_t)c));
-      const double full = (double)(size_t)(wgs / cus), rem = wgs - full * cus;
-      const double rounds = 0.25 + full + (rem > 0.0 ? (rem > 0.75 * cus ? rem : 0.75 * cus) / cus : 0.0);
-      const double cost = rounds * ((double)c * (double)per_s * (double)tile_bytes + (double)lds_bytes);
-      if (c == 1 || cost < best) {
-        best = cost;
-        best_s = c;
-      }
-    }
-    return best_s;
-  }
   const size_t w8 = waves > 8 ? 8 : (size_t)waves;  // (a sixteen-wave workgroup: twice the target of eight waves)
   size_t target = lds_bytes * w8 * w8 / (waves >= 8 && lds_bytes > 64 * 1024 ? 2 : 4) * ((size_t)waves / w8);
   if (target < 64 * 1024) target = 64 * 1024;
@@ -918,6 +892,44 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   const unsigned per_cu = waves >= 8 ? 1u : 2u;
   while (s > 1 && total_tiles / (per_s * s) < per_cu * (unsigned)ctx->info.compute_units) --s;
   while (s & (s - 1)) s &= s - 1;  // a power of two: runs of 3 tiles measured 5% slower than runs of 2 or 4
+  // Two or four row tiles whose rows leave a CU room for ONE workgroup (more than 80 KiB): the launch
+  // is a few rounds of one workgroup per CU, and what decides is how the workgroup count falls on the CUs. Cost of a
+  // run length = (rounds + 1/4) x (bytes a workgroup streams + twice the bytes it stages), a last partial round counting for at
+  // least three quarters (its workgroups share the memory system among fewer: 160 of 256 CUs busy measured as fast as
+  // all) and the quarter standing for the start and the end of the launch, where every CU stages or drains at once
+  // (one round of exactly 256 workgroups measured 13% slower than two rounds of half their length).
+  // Measured against this model over N in {5120, 11008, 17408}, K in {4096, 5120}, one to three planes, 24 / 32 int8
+  // rows, 32 layer copies, runs of 1 / 2 / 4 / 8 tiles, eight- and sixteen-wave workgroups: the model's choice is the
+  // measured best or within 4% of it, where the rule above (fitted to K = 2048) was 15-29% behind (three planes N=17408
+  // K=5120 24 rows, eight waves: 423 / 400 / 420 / 472 us, rule: 8 tiles; one plane, sixteen waves: 153 / 165 / 196 / 177).
+  // Four row tiles likewise (40 / 64 int8 rows, 32 copies, runs of 1 / 2 / 4 / 8): one plane K=2560 N=6912 68 / 55 / 49 / 80
+  // and 79 / 67 / 54 / 89 us, N=2560 32 / 24 / 41 / 77; K=2048 N=11008 64 rows 102 / 84 / 88 / 81; three planes K=2048 N=5120
+  // 64 rows 95 / 90 / 102 / 86 -- the model picks the best of each. Four row tiles keep the rule's run length where it
+  // fills its rounds to nine tenths: 128 copies of two planes K=2048 N=8192 at 64 rows (the benchmark's launches of this
+  // kind) are ONE round of 256 workgroups with runs of 16, which measured 3% faster than the two rounds of 8 that the
+  // model would take.
+  bool use_model = !b3 && rt >= 2 && waves >= 8 && lds_bytes > kLdsFlowMax / 2;
+  if (use_model && rt > 2) {
+    const double wgs = (double)((total_tiles + per_s * s - 1) / (per_s * s)), cus = (double)ctx->info.compute_units;
+    const double rounds = (double)(size_t)((wgs + cus - 1.0) / cus);
+    use_model = wgs < 0.9 * rounds * cus;
+  }
+  if (use_model) {
+    const double cus = (double)ctx->info.compute_units;
+    double best = 0.0;
+    int best_s = 1;
+    for (int c = 1; c <= 16; c *= 2) {
+      const double wgs = (double)((total_tiles + per_s * (size_t)c - 1) / (per_s * (size_t)c));
+      const double full = (double)(size_t)(wgs / cus), rem = wgs - full * cus;
+      const double rounds = 0.25 + full + (rem > 0.0 ? (rem > 0.75 * cus ? rem : 0.75 * cus) / cus : 0.0);
+      const double cost = rounds * ((double)c * (double)per_s * (double)tile_bytes + 2.0 * (double)lds_bytes);
+      if (c == 1 || cost < best) {
+        best = cost;
+        best_s = c;
+      }
+    }
+    return best_s;
+  }
   return (int)s;
 }
 
