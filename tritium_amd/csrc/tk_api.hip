@@ -908,7 +908,11 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
   // fills its rounds to nine tenths: 128 copies of two planes K=2048 N=8192 at 64 rows (the benchmark's launches of this
   // kind) are ONE round of 256 workgroups with runs of 16, which measured 3% faster than the two rounds of 8 that the
   // model would take.
-  bool use_model = !b3 && rt >= 2 && waves >= 8 && lds_bytes > kLdsFlowMax / 2;
+  // One row tile in eight-wave workgroups (more than 64 KiB of rows: 13..16 rows of K > 4096) is priced the same way, also
+  // where two workgroups share a CU: a CU's time follows the number of workgroups it is handed (two planes K=5120 N=5120
+  // 16 rows, 32 copies, runs of 1 / 2 / 4 / 8: 86 / 94 / 77 / 123 us, rule: 2; three planes N=17408 370 / 364 / 387 / 425,
+  // rule: 4).
+  bool use_model = !b3 && waves >= 8 && (rt == 1 || (rt >= 2 && lds_bytes > kLdsFlowMax / 2));
   if (use_model && rt > 2) {
     const double wgs = (double)((total_tiles + per_s * s - 1) / (per_s * s)), cus = (double)ctx->info.compute_units;
     const double rounds = (double)(size_t)((wgs + cus - 1.0) / cus);
@@ -923,7 +927,9 @@ static int flow_run_tiles(const tk_ctx *ctx, unsigned total_tiles, int planes, i
       const double full = (double)(size_t)(wgs / cus), rem = wgs - full * cus;
       const double rounds = 0.25 + full + (rem > 0.0 ? (rem > 0.75 * cus ? rem : 0.75 * cus) / cus : 0.0);
       const double cost = rounds * ((double)c * (double)per_s * (double)tile_bytes + 2.0 * (double)lds_bytes);
-      if (c == 1 || cost < best) {
+      // (equal costs are common, the terms being powers of two: one row tile then measured better with the longer run
+      // -- K=5120 N=5120 16 rows 48 vs 42 us, K=8192 N=8192 105 vs 97 --, two row tiles with the shorter)
+      if (c == 1 || cost < best || (rt == 1 && cost <= best)) {
         best = cost;
         best_s = c;
       }
