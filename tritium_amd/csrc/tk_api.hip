@@ -1223,6 +1223,20 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     // 32 int8 rows, 136 such workgroups: 36.8 / 32.0 / 32.1 us through the K-split or prefill kernel, 21.2 / 26.3 / 27.5
     // through the flow kernel)
     variant = choose_decode(ctx, pl.flow_ok, flow_groups * (unsigned)(fw >= 8 ? 2 : 1), pl.stream_groups);
+    // One token of a layer of more than two tiles per CU: the K-split kernel's single-launch form has a workgroup per
+    // tile and, beyond two workgroups per CU, hands each several tiles one after the other; the flow kernel's
+    // single-launch form (below) walks them in waves side by side. bf16 token, int8 contract, rotating layer copies,
+    // K-split -> flow at 640 / 768 tiles (512 tiles are a tie; from 1024 on the flow kernel is chosen anyway): one plane
+    // K=2048 7.7 -> 5.9 / 8.8 -> 6.0 us, K=4096 10.3 -> 7.2 / 10.3 -> 7.3, K=8192 13.6 -> 10.1 / 13.9 -> 10.3; two planes
+    // K=4096 11.4 -> 8.6 / 11.6 -> 8.6; three planes K=4096 13.4 -> 10.2 / 15.1 -> 10.7. More tokens are mixed (4 tokens:
+    // two and three planes of K <= 4096 gain 10-20%, one plane of K=8192 loses 20%) and stay.
+    if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && pl.flow_ok && !wide && !b3 && m == 1 &&
+        ctx->fuse_tokens != 0 && (unsigned)pl.pr.n_tiles > 2u * (unsigned)ctx->info.compute_units && pl.cfg.rt == 1 &&
+        (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) && nb * 16 <= 512 && k % 256 == 0 &&
+        ((uintptr_t)act & 15) == 0 && (act_dtype == TK_F32 || act_dtype == TK_BF16) &&
+        (!norm || ((uintptr_t)norm->weight & 15) == 0) &&
+        flow_lds + 1024 + (norm ? k * 4 + 1024 : 0) + 1024 <= 64 * 1024)
+      variant = DECODE_FLOW;
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
     // Operand rows that do not fit in LDS: the prefill kernel (rows streamed from L2 block by block)
     // beats the decode kernels that re-stage slices of K behind barriers, beyond 32 rows always and
