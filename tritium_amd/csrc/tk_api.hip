@@ -2296,6 +2296,12 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     if (plans[i].stream_lds > slds) slds = plans[i].stream_lds;
   }
   int variant = choose_decode(ctx, flow_ok, fgroups, sgroups);
+  // One token for a group of more than two tiles per CU (gate,up): the flow kernel behind the prep launch, as for single
+  // calls (run_linear) -- the K-split kernel would hand its workgroups several tiles each. gate,up of hidden 2560 behind
+  // an RMSNorm, rotating over 30 layers: 13.4 -> 11.6 us (2 / 4 / 8 tokens 12.9 -> 12.9 / 13.9 -> 13.2 / 14.7 -> 13.8: left).
+  if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && flow_ok && !wide && !b3 && rt == 1 && tokens_max == 1 &&
+      tiles > 2u * (unsigned)ctx->info.compute_units)
+    variant = DECODE_FLOW;
   // Operand rows that do not fit in LDS, and more than one row tile of them: the prefill kernel
   // (operand rows streamed block by block, int8 MFMA over 64-row tiles) beats a decode kernel that
   // re-stages slices of K behind barriers.
