@@ -271,6 +271,67 @@ def test_group_of_single_tokens_is_one_launch(backend, oracle, kernel, m, normed
         a.free()
 
 
+@pytest.mark.parametrize("special", ["plain", "zero", "nan", "narrow"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("planes,normed", [(1, True), (1, False), (2, True), (3, False)])
+def test_wide_group_of_single_tokens_is_one_launch_of_the_flow_kernel(backend, oracle, kernel, planes, normed, dtype, special):
+    """gate,up of a wide FFN behind a norm, one token: more than two tiles per CU, so the automatic dispatch takes the
+    flow kernel, and with one or two planes that kernel builds every member's row (norm included) itself: one launch.
+    Same bits as the single two-launch calls, under both contracts; three planes keep the prep launch."""
+    if kernel != FLOW:
+        pytest.skip("the automatic dispatch is what is tested: once")
+    print("case fused-flow-group", planes, normed, dtype, special, flush=True)
+    backend.set_decode_kernel(0)
+    rng = np.random.default_rng(planes * 11 + normed + len(special))
+    h, f = 768, 16 * 257 + 5  # two members of 258 tiles
+    hid_h = _tokens(rng, 1, h, special)
+    conv = (lambda a: f32_to_bf16_bits(a)) if dtype == "bf16" else (lambda a: a)
+    hid = backend.to_device(conv(hid_h), dtype)
+    w2 = backend.to_device(rng.uniform(-0.5, 0.5, h).astype(np.float32), "f32")
+    nm = (w2, 1e-5, True) if normed else None
+    members, singles = [], []
+    for _ in range(2):
+        ws, scs, packed = _planes(rng, f, h, planes)
+        layer = backend.linear(packed, scs, f, h)
+        members.append((layer, hid, 1, backend.empty(f, "f32")))
+        singles.append(backend.empty(f, "f32"))
+    backend.set_fuse_tokens(-1)
+    grp = backend.group(members, 1, dtype, "f32", norms=[nm, nm] if normed else None)
+    before = backend.fused_calls()
+    grp.launch()
+    grp.launch()
+    # (three planes: the flow kernel has no such form from a table, the K-split kernel would have counted two)
+    assert backend.fused_calls() - before == (2 if planes <= 2 else 0)
+    backend.set_fuse_tokens(0)
+    for (layer, src, _, out_g), out_s in zip(members, singles):
+        if nm is None:
+            backend.linear_a8(layer, src, 1, out_s)
+        else:
+            backend.linear_rmsnorm_a8(layer, src, nm[0], nm[1], 1, out_s, zero_centered=nm[2])
+        assert _same(out_s.to_host(), out_g.to_host()), (planes, normed, dtype, special)
+    if not normed:
+        backend.set_fuse_tokens(-1)
+        fmembers = [(layer, src, 1, backend.empty(f, "f32")) for (layer, src, _, _) in members]
+        fgrp = backend.group(fmembers, 0, dtype, "f32")
+        before = backend.fused_calls()
+        fgrp.launch()
+        assert backend.fused_calls() - before == (1 if planes <= 2 else 0)
+        backend.set_fuse_tokens(0)
+        for (layer, src, _, out_g), out_s in zip(fmembers, singles):
+            backend.linear_float(layer, src, 1, out_s)
+            assert _same(out_s.to_host(), out_g.to_host())
+        fgrp.destroy()
+        for mem in fmembers:
+            mem[3].free()
+    grp.destroy()
+    for (layer, _, _, out_g), out_s in zip(members, singles):
+        out_g.free()
+        out_s.free()
+        layer.free()
+    for a in (hid, w2):
+        a.free()
+
+
 def test_group_with_members_of_different_k_and_token_counts(backend, oracle, kernel):
     """One launch for a group whose members differ in K, N, token count and norm: every workgroup sizes its rows, row
     constants and norm scratch from its own member."""

@@ -2460,10 +2460,31 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
       tiles = wgs;
     }
   }
+  // The flow kernel has the form too (one token per member, four-wave workgroups of the 16x16x64 kernel with
+  // activations first): every workgroup builds the row of the member it works for. gate,up of hidden 2560 behind an
+  // RMSNorm, one bf16 token: 11.6 us as prep + kernel.
+  // Every workgroup repeats its member's prep, so the form is for groups of a few workgroups per CU at most (as the K-split
+  // kernel's): the 210 projections of a 30-layer step as ONE group took 173 us this way against 91 us behind one prep launch.
+  bool gfused_flow = variant == DECODE_FLOW && !wide && !b3 && rt == 1 && planes <= 2 && fw == 4 && ctx->fuse_tokens != 0 &&
+                     tiles <= 8u * (unsigned)ctx->info.compute_units &&
+                     (prep_kind == TK_PREP_A8 || prep_kind == TK_PREP_DIGITS) && (act_dtype == TK_F32 || act_dtype == TK_BF16);
+  size_t fuse_flow_extra = 1024;  // row constants (+ the norm's scratch) behind the rows
+  for (size_t i = 0; i < count && gfused_flow; ++i) {
+    const TkPrep &pp = preps[prep_of[i]];
+    const size_t k = (size_t)plans[i].pr.k, nb = (size_t)plans[i].pr.nb;
+    gfused_flow = members[i].m == 1 && nb * 16 <= 512 && k % 256 == 0 && ((uintptr_t)members[i].act & 15) == 0 &&
+                  (!pp.norm_kind || ((uintptr_t)pp.norm_w & 15) == 0);
+    if (pp.norm_kind && 1024 + k * 4 + 1024 > fuse_flow_extra) fuse_flow_extra = 1024 + k * 4 + 1024;
+  }
+  gfused_flow = gfused_flow && flds + fuse_flow_extra + 1024 <= 64 * 1024;
+  if (gfused_flow) {  // (the form keeps its row constants where the zero-chunk maps would go)
+    group_ztiles = 0;
+    for (size_t i = 0; i < count; ++i) plans[i].pr.zskip = 0;
+  }
   tk_group *g = new (std::nothrow) tk_group();
   if (!g) return tk_fail(TK_ERR_BACKEND, "tk_group_create: host allocation failed");
   g->ctx = ctx;
-  g->fused = gfused;
+  g->fused = gfused || gfused_flow;
   int rc = dev_malloc(ws_bytes, &g->ws);
   const size_t wg_prob_off = count * sizeof(TkProblem) + preps.size() * sizeof(TkPrep);
   const size_t flow_wg_prob_off = wg_prob_off + wg_prob.size() * sizeof(int);
@@ -2502,7 +2523,7 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     } else {
       pr.exps = pp.exps;
     }
-    if (gfused) {  // the kernel reads (and normalizes) the raw rows itself
+    if (gfused || gfused_flow) {  // the kernel reads (and normalizes) the raw rows itself
       pr.raw_act = members[i].act;
       pr.raw_dtype = act_dtype;
       pr.norm_kind = pp.norm_kind;
@@ -2577,10 +2598,14 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
     }
     g->cfg.ring = pick_flow_ring(ctx, nbs.data(), wts.data(), (int)count, rt, (int)rows_max, flow_runs_per_wave(wide, b3, planes, rt, rows_max), wide, fw, flds, planes);
   }
-  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max, kmode == TK_MODE_INT8 && ctx->flow_swap && !gfused);
+  if (variant == DECODE_FLOW) flow_cfg_form(&g->cfg, wide, b3, flds, rows_max, group_ztiles, nb_max, kmode == TK_MODE_INT8 && ctx->flow_swap && !gfused && !gfused_flow);
   if (gfused) {
     g->cfg.fused = 1;
     g->cfg.lds_bytes = fuse_lds;
+  }
+  if (gfused_flow) {
+    g->cfg.fused = 1;
+    g->cfg.lds_bytes += fuse_flow_extra;
   }
   ctx->refs.fetch_add(1);
   *out = g;

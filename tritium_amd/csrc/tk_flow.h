@@ -32,7 +32,7 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
 #define TK_FLOW_MAX_THREADS(P, RT, DR, TABLE, SWAP) \
   (((RT) == 2 && ((P) <= 2 || ((P) == 3 && (SWAP))) && (DR) == 2 && ((SWAP) || (TABLE))) ? 1024 : 512)
 #define TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP) ((!(SWAP) && (P) == 2 && (RT) == 1 && (TW) == 2 && (DR) == 4) ? 3 : 2)
-// FUSED (one row tile, a single problem, 256 threads): the kernel builds the operand rows of its one to four
+// FUSED (one row tile, 256 threads; a single problem or, from a table, one token per member): the kernel builds the operand rows of its one to four
 // tokens itself from pr.raw_act -- see fused_stage_rows -- and the call is one launch instead of two.
 // SWAP (int8 contract only; instantiated in tk_flow_a8.hip): the two operands of the matrix instruction change places --
 // weights first, activations second -- so that an accumulator register holds four consecutive OUTPUT CHANNELS of one
@@ -43,7 +43,7 @@ __device__ __forceinline__ void exact_rows_fused(const TkProblem &pr, int n, int
 template <int P, int RT, int TW, int DR, bool TABLE, bool FUSED = false, bool SWAP = false>
 __global__ __launch_bounds__(TK_FLOW_MAX_THREADS(P, RT, DR, TABLE, SWAP)) __attribute__((amdgpu_waves_per_eu(TK_FLOW_MIN_WAVES(P, RT, TW, DR, SWAP)))) void tk_flow_kernel(const TkProblem single, const TkProblem *__restrict__ table,
                                                       const int *__restrict__ wg_prob) {
-  static_assert(!FUSED || (RT == 1 && !TABLE), "the fused form: one row tile, one problem");
+  static_assert(!FUSED || RT == 1, "the fused form: one row tile");
   static_assert(!(FUSED && SWAP), "the fused form keeps the first operand order");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const TkProblem &pr = TABLE ? table[wg_prob[blockIdx.x]] : *single_problem();

@@ -2914,19 +2914,27 @@ static hipError_t launch_flow_pr(hipStream_t s, const TkProblem &sg, const TkPro
   constexpr int TW = ((RT >= 4 && P <= 2) || (RT == 2 && P == 1)) ? 2 : 1;
   const int threads = cfg.waves * 64;
   if constexpr (RT == 1) {
-    if (cfg.fused) {  // the operand rows are built inside the kernel: one problem, 256 threads
-      if (table || threads != 256) return hipErrorInvalidValue;
+    if (cfg.fused) {  // the operand rows are built inside the kernel: 256 threads; from a table for one or two planes
+      if (threads != 256) return hipErrorInvalidValue;
       if constexpr (P <= 2) {
         if (cfg.tw == 2) {
           switch (cfg.ring) {
-            case 2: return flow_launch_one(tk_flow_kernel<P, 1, 2, 2, false, true>, s, sg, table, wg_prob, cfg, threads);
-            case 3: return flow_launch_one(tk_flow_kernel<P, 1, 2, 3, false, true>, s, sg, table, wg_prob, cfg, threads);
-            case 4: return flow_launch_one(tk_flow_kernel<P, 1, 2, 4, false, true>, s, sg, table, wg_prob, cfg, threads);
-            case 5: return flow_launch_one(tk_flow_kernel<P, 1, 2, 5, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 2: return table ? flow_launch_one(tk_flow_kernel<P, 1, 2, 2, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 2, 2, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 3: return table ? flow_launch_one(tk_flow_kernel<P, 1, 2, 3, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 2, 3, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 4: return table ? flow_launch_one(tk_flow_kernel<P, 1, 2, 4, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 2, 4, false, true>, s, sg, table, wg_prob, cfg, threads);
+            case 5: return table ? flow_launch_one(tk_flow_kernel<P, 1, 2, 5, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 2, 5, false, true>, s, sg, table, wg_prob, cfg, threads);
             default: return hipErrorInvalidValue;
           }
         }
+        switch (cfg.ring) {
+          case 2: return table ? flow_launch_one(tk_flow_kernel<P, 1, 1, 2, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 1, 2, false, true>, s, sg, table, wg_prob, cfg, threads);
+          case 3: return table ? flow_launch_one(tk_flow_kernel<P, 1, 1, 3, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 1, 3, false, true>, s, sg, table, wg_prob, cfg, threads);
+          case 4: return table ? flow_launch_one(tk_flow_kernel<P, 1, 1, 4, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 1, 4, false, true>, s, sg, table, wg_prob, cfg, threads);
+          case 5: return table ? flow_launch_one(tk_flow_kernel<P, 1, 1, 5, true, true>, s, sg, table, wg_prob, cfg, threads) : flow_launch_one(tk_flow_kernel<P, 1, 1, 5, false, true>, s, sg, table, wg_prob, cfg, threads);
+          default: return hipErrorInvalidValue;
+        }
       }
+      if (table) return hipErrorInvalidValue;
       switch (cfg.ring) {
         case 2: return flow_launch_one(tk_flow_kernel<P, 1, 1, 2, false, true>, s, sg, table, wg_prob, cfg, threads);
         case 3: return flow_launch_one(tk_flow_kernel<P, 1, 1, 3, false, true>, s, sg, table, wg_prob, cfg, threads);
