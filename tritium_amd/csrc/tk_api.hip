@@ -1237,6 +1237,14 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
         (!norm || ((uintptr_t)norm->weight & 15) == 0) &&
         flow_lds + 1024 + (norm ? k * 4 + 1024 : 0) + 1024 <= 64 * 1024)
       variant = DECODE_FLOW;
+    // Up to eight operand rows of two or more planes on such a layer likewise (both as prep + kernel, or against the
+    // K-split kernel's single launch of two tokens): 640 / 768 tiles, two planes, 2 / 4 / 8 int8 tokens, K=2048 11.4 -> 9.9 /
+    // 12.5 -> 10.4 / 13.0 -> 10.6 us, K=4096 13.6 -> 12.3 / 14.5 -> 12.7 / 15.6 -> 13.8, K=8192 21.2 -> 17.9 / 19.1 -> 18.6 /
+    // 21.9 -> 20.7; three planes K=4096 15.2 -> 14.2 / 16.9 -> 14.7 / 18.5 -> 15.7. One plane is within 5% either way for
+    // K <= 4096 and 15-24% slower through the flow kernel at K=8192: left.
+    if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && pl.flow_ok && !wide && !b3 && pl.cfg.rt == 1 &&
+        R >= 2 && R <= 8 && pl.cfg.planes >= 2 && (unsigned)pl.pr.n_tiles > 2u * (unsigned)ctx->info.compute_units)
+      variant = DECODE_FLOW;
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
     // Operand rows that do not fit in LDS: the prefill kernel (rows streamed from L2 block by block)
     // beats the decode kernels that re-stage slices of K behind barriers, beyond 32 rows always and
@@ -2298,9 +2306,10 @@ static int group_create(tk_ctx *ctx, const tk_group_member *members, const tk_rm
   int variant = choose_decode(ctx, flow_ok, fgroups, sgroups);
   // One token for a group of more than two tiles per CU (gate,up): the flow kernel behind the prep launch, as for single
   // calls (run_linear) -- the K-split kernel would hand its workgroups several tiles each. gate,up of hidden 2560 behind
-  // an RMSNorm, rotating over 30 layers: 13.4 -> 11.6 us (2 / 4 / 8 tokens 12.9 -> 12.9 / 13.9 -> 13.2 / 14.7 -> 13.8: left).
-  if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && flow_ok && !wide && !b3 && rt == 1 && tokens_max == 1 &&
-      tiles > 2u * (unsigned)ctx->info.compute_units)
+  // an RMSNorm, rotating over 30 layers: 13.4 -> 11.6 us (2 / 4 / 8 tokens 12.9 -> 12.9 / 13.9 -> 13.2 / 14.7 -> 13.8: left);
+  // up to eight rows of two or more planes as well, as single calls.
+  if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && flow_ok && !wide && !b3 && rt == 1 &&
+      (tokens_max == 1 || (rows_max <= 8 && planes >= 2)) && tiles > 2u * (unsigned)ctx->info.compute_units)
     variant = DECODE_FLOW;
   // Operand rows that do not fit in LDS, and more than one row tile of them: the prefill kernel
   // (operand rows streamed block by block, int8 MFMA over 64-row tiles) beats a decode kernel that
