@@ -1245,6 +1245,17 @@ static int run_linear(tk_ctx *ctx, const tk_linear_desc *layer, int mode, int pr
     if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && pl.flow_ok && !wide && !b3 && pl.cfg.rt == 1 &&
         R >= 2 && R <= 8 && pl.cfg.planes >= 2 && (unsigned)pl.pr.n_tiles > 2u * (unsigned)ctx->info.compute_units)
       variant = DECODE_FLOW;
+    // Narrower layers of two or more planes with short rows (K <= 2560), 3..8 operand rows that the K-split kernel would
+    // not build itself (three int8 tokens or more, two float tokens): the flow kernel again, both as prep + kernel.
+    // 3 / 4 / 8 int8 tokens, K-split -> flow: two planes K=2048 N=2560 10.0 -> 9.2 / 10.6 -> 9.9 / 11.3 -> 10.2 us, N=8192
+    // 4 / 8 tokens 11.8 -> 10.5 / 12.4 -> 10.5; three planes K=2048 N=6144 12.2 -> 10.3 / 12.7 -> 10.6 / 13.6 -> 11.3; K=2560
+    // from 256 tiles on: two planes N=5120 11.2 -> 10.9 / 11.9 -> 11.1 / 12.5 -> 11.9, three planes 12.5 -> 11.4 / 13.4 -> 11.6 /
+    // 14.0 -> 12.4 (160 tiles: two planes 10.4 -> 11.0: left). K=4096 is within 3-7% either way, K=5120 up to 14% slower
+    // through the flow kernel: left.
+    if (ctx->decode_force == DECODE_AUTO && variant == DECODE_KSPLIT && pl.flow_ok && !wide && !b3 && pl.cfg.rt == 1 &&
+        pl.cfg.planes >= 2 && R >= 3 && R <= 8 && m >= (prep_kind == TK_PREP_A8 ? 3u : 2u) &&
+        (nb <= 8 || (nb <= 10 && pl.pr.n_tiles >= 256)))
+      variant = DECODE_FLOW;
     if (variant == DECODE_FLOW && wide) pl.pr.rs = (int)flow_wide_rows(pl.cfg.rt);
     // Operand rows that do not fit in LDS: the prefill kernel (rows streamed from L2 block by block)
     // beats the decode kernels that re-stage slices of K behind barriers, beyond 32 rows always and
