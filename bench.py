@@ -608,6 +608,45 @@ def bench_salt_v2(T, be, rng, iters=10):
     return res
 
 
+def bench_other_widths(T, be, rng, iters=30):
+    """Decode launches at layer widths that none of the reference's configurations names (hidden 4096 / 5120, FFN
+    11008 / 17408): W1.58A8, bf16 in and out, 32 resident layer copies per grouped launch, decode kernel alone.
+    These are the launches whose run lengths, workgroup sizes and kernel choice come from the library's rules rather
+    than from a fit to the headline's shape."""
+    copies = 32
+    res = {"workload": f"{copies} layer copies per launch, W1.58A8, bf16 in/out, decode kernel alone (prep launch excluded)"}
+    for n, k, planes in ((11008, 4096, 1), (5120, 5120, 3), (17408, 5120, 3)):
+        hostw = []
+        for _ in range(2):
+            ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)[:planes]]
+            hostw.append((ws, [rng.uniform(0.01, 0.1, n).astype(np.float32) for _ in range(planes)]))
+        layers = [be.linear([T.pack_rows(w, n, k) for w in hostw[i % 2][0]], hostw[i % 2][1], n, k) for i in range(copies)]
+        leg = {}
+        for m in (1, 8, 24, 32):
+            abits = f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+            act = be.to_device(abits, "bf16")
+            outs = [be.empty(m * n, "bf16") for _ in range(copies)]
+            g = be.group([(layers[i], act, m, outs[i]) for i in range(copies)], 1, "bf16", "bf16")
+            g.launch()
+            be.sync()
+            tok = sorted({0, m // 2, m - 1})
+            c = copies - 1
+            ver = check_a8(f"other widths {n}x{k}x{planes} batch {m}", outs[c].to_host().reshape(m, n)[tok], hostw[c % 2][0],
+                           hostw[c % 2][1], bf16_to_f32(abits).reshape(m, k)[tok], "bf16")
+            g.launch_parts(True, False)
+            ms = time_calls(be, lambda i: g.launch_parts(False, True), iters)
+            nbytes = copies * algorithmic_bytes(m, n, k, planes, 1, 2, a8=True)
+            leg[f"batch{m}"] = {"kernel_us_per_launch": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
+                                "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "verified": ver}
+            g.destroy()
+            for x in outs + [act]:
+                x.free()
+        res[f"N{n}_K{k}_{planes}plane{'s' if planes > 1 else ''}"] = leg
+        for l in layers:
+            l.free()
+    return res
+
+
 def bench_vjp(T, be, rng, iters=5):
     """mpgemm_projected_vjp on the configs[2] projection (M=2048 tokens, K=2560, N=6912, one plane),
     device-resident f32 operands. Each gradient is timed on its own; flops = one multiply and one add
@@ -855,7 +894,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extra", action="store_true", help="skip the legs under `extra`")
-    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,base3,salt,salt_v2,vjp",
+    ap.add_argument("--extra-legs", default="sweep_a8,config1,prefill,stack,config5,zero_skip,base3,salt,salt_v2,vjp,other_widths",
                     help="comma-separated subset of the `extra` legs to run (profiling runs name one)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -915,7 +954,8 @@ def main():
                 "base3": ("base3_stream_vs_two_bit", lambda: bench_base3(T, be, rng)),
                 "salt": ("block_scale_planes", lambda: bench_salt(T, be, rng)),
                 "salt_v2": ("salt_v2_exact", lambda: bench_salt_v2(T, be, rng)),
-                "vjp": ("projected_vjp", lambda: bench_vjp(T, be, rng))}
+                "vjp": ("projected_vjp", lambda: bench_vjp(T, be, rng)),
+                "other_widths": ("decode_other_widths", lambda: bench_other_widths(T, be, rng))}
         out["extra"] = {}
         for leg in [x for x in args.extra_legs.split(",") if x]:
             if leg not in legs:
