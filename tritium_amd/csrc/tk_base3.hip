@@ -286,16 +286,9 @@ int tk_flow3_waves(int rt) { (void)rt; return TK_B3_WAVES; }
 template <typename K>
 static hipError_t flow3_launch_one(K kernel, hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                    const TkLaunchCfg &cfg) {
-  // the table alone is 64 KiB: the dynamic LDS limit has to be raised once per kernel
-  static thread_local const void *raised[16];
-  static thread_local int nraised = 0;
-  bool done = false;
-  for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
-  if (!done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return e;
-    if (nraised < 16) raised[nraised++] = (const void *)kernel;
-  }
+  // the table alone is 64 KiB: the dynamic LDS limit has to be raised
+  hipError_t e = tk_raise_lds_limit((const void *)kernel, 160 * 1024);
+  if (e != hipSuccess) return e;
   hipLaunchKernelGGL(kernel, dim3(cfg.grid), dim3(cfg.waves * 64), cfg.lds_bytes, s, sg, table, wg_prob);
   return hipGetLastError();
 }

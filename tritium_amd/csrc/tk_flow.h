@@ -590,16 +590,8 @@ template <typename K>
 static hipError_t flow_launch_one(K kernel, hipStream_t s, const TkProblem &sg, const TkProblem *table,
                                   const int *wg_prob, const TkLaunchCfg &cfg, int threads) {
   if (cfg.lds_bytes > 64 * 1024) {
-    // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    static thread_local const void *raised[512];
-    static thread_local int nraised = 0;
-    bool done = false;
-    for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
-    if (!done) {
-      hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-      if (e != hipSuccess) return e;
-      if (nraised < 512) raised[nraised++] = (const void *)kernel;
-    }
+    hipError_t e = tk_raise_lds_limit((const void *)kernel, 160 * 1024);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kernel, dim3(cfg.grid), dim3(threads), cfg.lds_bytes, s, sg, table, wg_prob);
   return hipGetLastError();

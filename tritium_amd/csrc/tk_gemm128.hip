@@ -242,12 +242,8 @@ int tk_gemm128_lds_bytes(void) { return TK_G128_CST + 1536; }
 hipError_t tk_launch_gemm128(hipStream_t s, const TkProblem *single) {
   const unsigned wgs = 8u * (unsigned)single->sub_m * (unsigned)single->sub_n;
   if (!wgs) return hipSuccess;
-  static thread_local bool raised = false;
-  if (!raised) {  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    hipError_t e = hipFuncSetAttribute((const void *)tk_gemm128_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-    if (e != hipSuccess) return e;
-    raised = true;
-  }
+  hipError_t e = tk_raise_lds_limit((const void *)tk_gemm128_kernel, 128 * 1024);
+  if (e != hipSuccess) return e;
   hipLaunchKernelGGL(tk_gemm128_kernel, dim3(wgs), dim3(TK_G128_THREADS), (size_t)tk_gemm128_lds_bytes(), s, *single);
   return hipGetLastError();
 }

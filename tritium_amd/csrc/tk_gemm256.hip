@@ -342,13 +342,8 @@ int tk_gemm256_lds_bytes(int form) {
 
 template <int FORM>
 static hipError_t launch_gemm256_form(hipStream_t s, const TkProblem *single, unsigned wgs) {
-  static thread_local bool raised = false;
-  if (!raised) {  // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    hipError_t e = hipFuncSetAttribute((const void *)tk_gemm256_kernel<FORM>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       tk_gemm256_lds_bytes(FORM));
-    if (e != hipSuccess) return e;
-    raised = true;
-  }
+  hipError_t e = tk_raise_lds_limit((const void *)tk_gemm256_kernel<FORM>, tk_gemm256_lds_bytes(FORM));
+  if (e != hipSuccess) return e;
   hipLaunchKernelGGL(tk_gemm256_kernel<FORM>, dim3(FORM == 2 ? 2 * wgs : wgs), dim3(FORM == 1 ? 512 : 256),
                      (size_t)tk_gemm256_lds_bytes(FORM), s, *single);
   return hipGetLastError();

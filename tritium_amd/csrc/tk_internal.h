@@ -24,6 +24,26 @@
 #define TK_ZERO_CHUNKS 1
 #endif
 
+// More than 64 KiB of dynamic LDS has to be asked for once per kernel AND device (a process may hold a context on
+// every GPU of a node): remembered per thread, keyed by both.
+static inline hipError_t tk_raise_lds_limit(const void *kernel, int bytes) {
+  static thread_local const void *done_kernel[1024];
+  static thread_local int done_dev[1024];
+  static thread_local int ndone = 0;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  for (int i = 0; i < ndone; ++i)
+    if (done_kernel[i] == kernel && done_dev[i] == dev) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return e;
+  if (ndone < 1024) {
+    done_kernel[ndone] = kernel;
+    done_dev[ndone++] = dev;
+  }
+  return hipSuccess;
+}
+
 // ---- base-3 weight stream ("T16B3"), an optional second copy of a plane ----------------------
 // The same tiles and K blocks, 832 bytes per chunk instead of 1024: lane l = g*16 + r keeps its 64
 // trits (the ones its 16 bytes of the T16 chunk hold) in 13 bytes of five base-3 digits each, encoded

@@ -3091,17 +3091,9 @@ template <typename K>
 static hipError_t gemm_launch_one(K kernel, hipStream_t s, const TkProblem &sg, const TkProblem *table, const int *wg_prob,
                                   const TkLaunchCfg &cfg, unsigned wgs) {
   if (cfg.lds_bytes > 64 * 1024) {
-    // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-    static thread_local const void *raised[16];
-    static thread_local int nraised = 0;
-    bool done = false;
-    for (int i = 0; i < nraised; ++i) done |= raised[i] == (const void *)kernel;
-    if (!done) {
-      // (not the full 160 KiB: the kernel also has a few static bytes)
-      hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-      if (e != hipSuccess) return e;
-      if (nraised < 16) raised[nraised++] = (const void *)kernel;
-    }
+    // (not the full 160 KiB: the kernel also has a few static bytes)
+    hipError_t e = tk_raise_lds_limit((const void *)kernel, 128 * 1024);
+    if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kernel, dim3(wgs), dim3(TK_GEMM_THREADS), cfg.lds_bytes, s, sg, table, wg_prob);
   return hipGetLastError();
@@ -3161,7 +3153,7 @@ static hipError_t launch_salt_p(hipStream_t s, const TkProblem &sg, const TkLaun
   TkLaunchCfg c = cfg;
   auto go = [&](auto kernel) {
     if (c.lds_bytes > 64 * 1024) {
-      hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      hipError_t e = tk_raise_lds_limit((const void *)kernel, 160 * 1024);
       if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kernel, dim3(c.grid), dim3(c.waves * 64), c.lds_bytes, s, sg);

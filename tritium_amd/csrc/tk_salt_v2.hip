@@ -356,7 +356,7 @@ hipError_t tk_launch_salt_v2_forward(hipStream_t s, const TkSaltV2 &t, const flo
   }
   const size_t lds = tk_salt_v2_lds_bytes(t.k, t.group);
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void *)tk_salt_v2_forward_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t e = tk_raise_lds_limit((const void *)tk_salt_v2_forward_kernel, 160 * 1024);
     if (e != hipSuccess) return e;
   }
   const dim3 grid(t.n, (unsigned)((m + TK_SALT_V2_TOKENS - 1) / TK_SALT_V2_TOKENS));
