@@ -14,7 +14,8 @@ launches included); `roofline` is the decode kernel alone, timed with events on 
 on; `cpu_baseline` is the CPU oracle's restatement of tritium-cpu timed on this host on one pass
 of the same sweep. `extra` carries the other configs measured in the same run: the batch-1 f32
 layer (configs[0]), the prefill GEMM (configs[2]), the projection-stack tokens/s (configs[3]) and
-the three-plane decode and prefill (configs[4]). Every timed region follows an untimed pre-warm of
+the three-plane decode and prefill (configs[4]), and decode launches at layer widths that none of the
+configurations names (`decode_other_widths`). Every timed region follows an untimed pre-warm of
 PREWARM_S seconds of the same work: from idle the clocks take tens of milliseconds to settle, and a
 cold first few milliseconds under-report a kernel by 10-25%.
 """
