@@ -60,3 +60,40 @@ def test_random_shape_a8_bits_and_float_tolerance(backend, oracle, seed):
     for a in (dact, dout, dob, dof):
         a.free()
     layer.free()
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_wide_layer_few_tokens(backend, oracle, seed):
+    """Layers of more than two tiles per CU (N > 8192) with 1..16 tokens: the shapes whose kernel the dispatch picks
+    by layer width -- the flow kernel's single-launch form for one token, the flow kernel behind a prep launch for few
+    rows of several planes, the K-split kernel otherwise. Bits of the CPU under the int8 contract, the reference's
+    tolerance under the float contract, ragged N and K."""
+    rng = np.random.default_rng(0xB1D00 + seed)
+    m = int(rng.choice([1, 1, 2, 3, 4, 8, 12, 16]))
+    n, k, planes = int(rng.integers(8200, 13000)), int(rng.integers(200, 800)), int(rng.integers(1, 4))
+    if seed % 4 == 0:
+        k = int(rng.integers(1, 4)) * 256  # whole K blocks: the single-launch forms apply
+    print("case random-wide", seed, m, n, k, planes, flush=True)
+    ws = [ternary(rng, n, k, p0) for p0 in (0.4, 0.7, 0.85)[:planes]]
+    scs = [scales(rng, n) for _ in range(planes)]
+    packed = [T.pack_rows(w, n, k) for w in ws]
+    layer = backend.linear(packed, scs, n, k)
+    act = (rng.standard_normal((m, k)) * 10.0 ** rng.integers(-2, 3)).astype(np.float32)
+    if m > 2:
+        act[m // 2] = 0.0
+    for dt in ("f32", "bf16"):
+        a = act if dt == "f32" else (f32_to_bf16_bits(act).astype(np.uint32) << 16).view(np.float32).reshape(m, k)
+        dact = backend.to_device(a if dt == "f32" else f32_to_bf16_bits(act), dt)
+        want = oracle.cpu_linear_a8_planes(packed, FMT_TQ2_0, scs, a, m, n, k)
+        dout = backend.empty(m * n, "f32")
+        backend.linear_a8(layer, dact, m, dout)
+        assert same_bits(dout.to_host(), want), (dt, backend.last_kernel())
+        mf = min(m, 3)
+        dof = backend.empty(mf * n, "f32")
+        backend.linear_float(layer, dact, mf, dof)
+        wantf = oracle.cpu_mpgemm_planes(packed, FMT_TQ2_0, scs, a[:mf], mf, n, k)
+        top = max(float(np.abs(wantf).max()), 1e-30)
+        assert accepts(dof.to_host().reshape(mf, n), wantf, rel=1e-4, floor=top).all(), (dt, backend.last_kernel())
+        for x in (dact, dout, dof):
+            x.free()
+    layer.free()
