@@ -22,7 +22,8 @@ def test_noalloc_equals_linear_a8_on_consecutive_calls(backend, oracle):
     """A big call (prefill kernel, two planes), then smaller ones on the same scratch (decode kernels,
     other K, other plane count): what the earlier call left in the scratch must not leak into the later."""
     rng = np.random.default_rng(77)
-    cases = [(200, 136, 2560, 2, "f32"), (40, 136, 2560, 2, "f32"), (3, 129, 700, 1, "bf16"), (1, 48, 300, 3, "f32")]
+    cases = [(200, 136, 2560, 2, "f32"), (40, 136, 2560, 2, "f32"), (3, 129, 700, 1, "bf16"), (1, 48, 300, 3, "f32"),
+             (1, 8300, 512, 1, "bf16"), (4, 8300, 512, 2, "f32")]  # (wide layers: the flow kernel, in one launch for one token)
     for m, n, k, planes, dt in cases:
         print("case noalloc", m, n, k, planes, dt, flush=True)
         packed, scs, layer = _layer(backend, rng, n, k, planes)
